@@ -1,0 +1,40 @@
+"""MI355X-native RG-LRU scan, temporal conv1d and decode kernels for Hawk, with the
+operator / module surface of fattorib/hawk-pytorch (``from hawk import HawkModel, HawkConfig``
+becomes ``from hawk_pytorch_amd import HawkModel, HawkConfig``)."""
+
+from .cache import RNNCache
+from .external import (
+    BlockDiagonalLinear,
+    Conv1D,
+    rglru_step,
+    rnn_param_init,
+    temporal_conv1d,
+    temporal_conv1d_step,
+)
+from .hawk import Hawk, HawkConfig, HawkModel, MLP, RMSNorm, RNNLayer
+from .scan_fused import (
+    DiagonalRecurrence,
+    fused_linear_scan,
+    sequential_scan_backward,
+    sequential_scan_forward,
+)
+
+__all__ = [
+    "BlockDiagonalLinear",
+    "Conv1D",
+    "DiagonalRecurrence",
+    "Hawk",
+    "HawkConfig",
+    "HawkModel",
+    "MLP",
+    "RMSNorm",
+    "RNNCache",
+    "RNNLayer",
+    "fused_linear_scan",
+    "rglru_step",
+    "rnn_param_init",
+    "sequential_scan_backward",
+    "sequential_scan_forward",
+    "temporal_conv1d",
+    "temporal_conv1d_step",
+]

@@ -1,0 +1,154 @@
+"""ctypes binding of libhawk_hip.so (declared in include/hawk_hip.h).
+
+The library is the product: there is no CPU or eager fallback.  If the shared object
+cannot be found or built, or a call reports a non-zero status, an exception is raised.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import os
+import threading
+
+import torch
+
+_CSRC = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc")
+LIB_PATH = os.path.join(_CSRC, "libhawk_hip.so")
+
+HAWK_OK = 0
+HAWK_ERR_NULL_POINTER = 1
+HAWK_ERR_BAD_SHAPE = 2
+HAWK_ERR_BAD_DTYPE = 3
+HAWK_ERR_WORKSPACE = 4
+HAWK_ERR_LAUNCH = 5
+HAWK_ERR_ALIGNMENT = 6
+
+HAWK_DTYPE_BF16 = 0
+HAWK_DTYPE_F32 = 1
+
+_c_void_p = ctypes.c_void_p
+_c_int = ctypes.c_int
+_c_size_t = ctypes.c_size_t
+
+# name -> (restype, argtypes); mirrors include/hawk_hip.h one to one
+SIGNATURES = {
+    "hawk_version": (_c_int, []),
+    "hawk_status_string": (ctypes.c_char_p, [_c_int]),
+    "hawk_scan_workspace_bytes": (_c_size_t, [_c_int] * 4),
+    "hawk_scan_workspace_init": (_c_int, [_c_void_p, _c_size_t, _c_void_p]),
+    "hawk_scan_workspace_status": (_c_int, [_c_void_p, _c_void_p, ctypes.POINTER(_c_int)]),
+    "hawk_rglru_scan_fwd": (_c_int, [_c_void_p] * 5 + [_c_int] * 4 + [_c_void_p, _c_size_t, _c_void_p]),
+    "hawk_rglru_scan_bwd": (_c_int, [_c_void_p] * 10 + [_c_int] * 4 + [_c_void_p, _c_size_t, _c_void_p]),
+    "hawk_conv1d_fwd": (_c_int, [_c_void_p] * 5 + [_c_int] * 6 + [_c_void_p]),
+    "hawk_conv1d_bwd_workspace_bytes": (_c_size_t, [_c_int] * 4),
+    "hawk_conv1d_bwd": (_c_int, [_c_void_p] * 6 + [_c_int] * 6 + [_c_void_p, _c_size_t, _c_void_p]),
+    "hawk_conv1d_step": (_c_int, [_c_void_p] * 5 + [_c_int] * 5 + [_c_void_p]),
+    "hawk_rglru_step": (_c_int, [_c_void_p] * 6 + [_c_int] * 4 + [_c_void_p]),
+}
+
+
+class HawkHipError(RuntimeError):
+    """A libhawk_hip entry point returned a non-zero hawk_status."""
+
+    def __init__(self, fn: str, status: int, message: str):
+        super().__init__(f"{fn} failed with status {status}: {message}")
+        self.status = status
+
+
+_lib = None
+_lock = threading.Lock()
+
+
+def load() -> ctypes.CDLL:
+    """Load libhawk_hip.so, building it first only if no built library is present."""
+    global _lib
+    with _lock:
+        if _lib is not None:
+            return _lib
+        if not os.path.exists(LIB_PATH):
+            from .csrc.build import build
+
+            build(force=False)
+        lib = ctypes.CDLL(LIB_PATH)
+        for name, (restype, argtypes) in SIGNATURES.items():
+            fn = getattr(lib, name)  # AttributeError here means header and library disagree
+            fn.restype = restype
+            fn.argtypes = argtypes
+        _lib = lib
+        return lib
+
+
+def status_string(status: int) -> str:
+    return load().hawk_status_string(status).decode()
+
+
+def check(fn: str, status: int) -> None:
+    if status != HAWK_OK:
+        raise HawkHipError(fn, status, status_string(status))
+
+
+def dtype_code(dt: torch.dtype) -> int:
+    if dt == torch.bfloat16:
+        return HAWK_DTYPE_BF16
+    if dt == torch.float32:
+        return HAWK_DTYPE_F32
+    raise TypeError(f"libhawk_hip supports bfloat16 and float32 activations, got {dt}")
+
+
+def require_cuda(*tensors: torch.Tensor) -> torch.device:
+    """All tensors must live on one GPU; returns that device.  There is no CPU path."""
+    dev = tensors[0].device
+    for t in tensors:
+        if t.device.type != "cuda":
+            raise RuntimeError(
+                "hawk_pytorch_amd kernels run on an AMD GPU only; got a tensor on "
+                f"{t.device} (there is no CPU fallback)"
+            )
+        if t.device != dev:
+            raise RuntimeError(f"tensors on different devices: {dev} and {t.device}")
+    return dev
+
+
+def stream_ptr(dev: torch.device) -> int:
+    return torch.cuda.current_stream(dev).cuda_stream
+
+
+def ptr(t):
+    return None if t is None else t.data_ptr()
+
+
+def dense16(t: torch.Tensor) -> torch.Tensor:
+    """Contiguous and 16-byte aligned view or copy of t (the kernels use vector loads)."""
+    if not t.is_contiguous():
+        t = t.contiguous()
+    if t.data_ptr() % 16 != 0:
+        t = t.clone(memory_format=torch.contiguous_format)
+    return t
+
+
+# ---------------------------------------------------------------------------------------
+# Scan workspace: one zero-initialised buffer per (device, stream), grown on demand.
+# Scans that share a workspace must be ordered on one stream, hence the key.
+# ---------------------------------------------------------------------------------------
+_workspaces: dict = {}
+
+
+def scan_workspace(dev: torch.device, nbytes: int) -> torch.Tensor:
+    key = (dev.index if dev.index is not None else torch.cuda.current_device(), stream_ptr(dev))
+    ws = _workspaces.get(key)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.zeros(max(nbytes, 1 << 20), dtype=torch.uint8, device=dev)
+        _workspaces[key] = ws
+    return ws
+
+
+def scan_workspace_status(dev: torch.device) -> int:
+    """Synchronising check of the carry-timeout flag of the current stream's workspace."""
+    key = (dev.index if dev.index is not None else torch.cuda.current_device(), stream_ptr(dev))
+    ws = _workspaces.get(key)
+    if ws is None:
+        return 0
+    flag = ctypes.c_int(0)
+    check("hawk_scan_workspace_status",
+          load().hawk_scan_workspace_status(ws.data_ptr(), stream_ptr(dev), ctypes.byref(flag)))
+    return flag.value

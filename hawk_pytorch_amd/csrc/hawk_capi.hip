@@ -1,0 +1,138 @@
+// extern "C" surface of libhawk_hip.so: argument validation, then dispatch to the kernel
+// translation units.  Validation happens before any HIP call, so bad arguments are
+// reported without touching a GPU.
+#include "hawk_scan.h"
+
+#include <stdint.h>
+
+namespace {
+
+inline bool dtype_ok(int d) { return d == HAWK_DTYPE_BF16 || d == HAWK_DTYPE_F32; }
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+inline hipStream_t as_stream(void* s) { return static_cast<hipStream_t>(s); }
+
+constexpr int kMaxGridY = 65535;
+constexpr long long kMaxTiles = 0x7fffffffLL;
+
+int check_scan_shape(int B, int T, int D) {
+    if (B < 1 || T < 1 || D < 1) return HAWK_ERR_BAD_SHAPE;
+    // tiles are at least 64 rows x 64 channels; the flattened grid must fit 31 bits
+    const long long tiles = (long long)B * ((T + 63) / 64) * ((D + 63) / 64);
+    if (tiles > kMaxTiles) return HAWK_ERR_BAD_SHAPE;
+    return HAWK_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int hawk_version(void) { return 100; }
+
+const char* hawk_status_string(int status) {
+    switch (status) {
+        case HAWK_OK: return "ok";
+        case HAWK_ERR_NULL_POINTER: return "a required pointer is NULL";
+        case HAWK_ERR_BAD_SHAPE: return "bad shape: sizes must be >= 1 and within the documented limits";
+        case HAWK_ERR_BAD_DTYPE: return "unsupported dtype (expected HAWK_DTYPE_BF16 or HAWK_DTYPE_F32)";
+        case HAWK_ERR_WORKSPACE: return "workspace is NULL or smaller than the size query reports";
+        case HAWK_ERR_LAUNCH: return "the HIP runtime refused a kernel launch or copy";
+        case HAWK_ERR_ALIGNMENT: return "tensor pointers must be 16-byte aligned";
+        default: return "unknown status";
+    }
+}
+
+size_t hawk_scan_workspace_bytes(int B, int T, int D, int dtype) {
+    if (check_scan_shape(B, T, D) != HAWK_OK || !dtype_ok(dtype)) return 0;
+    return hawk::scan_workspace_bytes(B, T, D, dtype);
+}
+
+int hawk_scan_workspace_init(void* workspace_device, size_t workspace_bytes, void* stream) {
+    if (workspace_device == nullptr) return HAWK_ERR_NULL_POINTER;
+    if (!aligned16(workspace_device)) return HAWK_ERR_ALIGNMENT;
+    if (workspace_bytes < 256) return HAWK_ERR_WORKSPACE;
+    return hawk::workspace_init(workspace_device, workspace_bytes, as_stream(stream));
+}
+
+int hawk_scan_workspace_status(const void* workspace_device, void* stream, int* flag) {
+    if (workspace_device == nullptr || flag == nullptr) return HAWK_ERR_NULL_POINTER;
+    return hawk::workspace_status(workspace_device, as_stream(stream), flag);
+}
+
+int hawk_rglru_scan_fwd(const void* x, const void* x_rg_lru, const void* a_rg_lru, const float* a_param, void* h,
+                        int B, int T, int D, int dtype, void* workspace_device, size_t workspace_bytes,
+                        void* stream) {
+    if (!x || !x_rg_lru || !a_rg_lru || !a_param || !h) return HAWK_ERR_NULL_POINTER;
+    if (!dtype_ok(dtype)) return HAWK_ERR_BAD_DTYPE;
+    if (int rc = check_scan_shape(B, T, D)) return rc;
+    if (!aligned16(x) || !aligned16(x_rg_lru) || !aligned16(a_rg_lru) || !aligned16(h)) return HAWK_ERR_ALIGNMENT;
+    if (workspace_device && !aligned16(workspace_device)) return HAWK_ERR_ALIGNMENT;
+    return hawk::scan_fwd(x, x_rg_lru, a_rg_lru, a_param, h, B, T, D, dtype, workspace_device, workspace_bytes,
+                          as_stream(stream));
+}
+
+int hawk_rglru_scan_bwd(const void* x, const void* x_rg_lru, const void* a_rg_lru, const float* a_param,
+                        const void* h_saved, const void* grad_out, void* dx, void* dx_rg_lru, void* da_rg_lru,
+                        float* da_param, int B, int T, int D, int dtype, void* workspace_device,
+                        size_t workspace_bytes, void* stream) {
+    if (!x || !x_rg_lru || !a_rg_lru || !a_param || !h_saved || !grad_out || !dx || !dx_rg_lru || !da_rg_lru ||
+        !da_param)
+        return HAWK_ERR_NULL_POINTER;
+    if (!dtype_ok(dtype)) return HAWK_ERR_BAD_DTYPE;
+    if (int rc = check_scan_shape(B, T, D)) return rc;
+    if (!aligned16(x) || !aligned16(x_rg_lru) || !aligned16(a_rg_lru) || !aligned16(h_saved) ||
+        !aligned16(grad_out) || !aligned16(dx) || !aligned16(dx_rg_lru) || !aligned16(da_rg_lru))
+        return HAWK_ERR_ALIGNMENT;
+    if (workspace_device == nullptr) return HAWK_ERR_WORKSPACE;
+    if (!aligned16(workspace_device)) return HAWK_ERR_ALIGNMENT;
+    return hawk::scan_bwd(x, x_rg_lru, a_rg_lru, a_param, h_saved, grad_out, dx, dx_rg_lru, da_rg_lru, da_param, B,
+                          T, D, dtype, workspace_device, workspace_bytes, as_stream(stream));
+}
+
+int hawk_conv1d_fwd(const void* x, const float* w, const float* bias, const void* state, void* y, int B, int T,
+                    int D, int W, int x_dtype, int y_dtype, void* stream) {
+    if (!x || !w || !bias || !y) return HAWK_ERR_NULL_POINTER;
+    if (!dtype_ok(x_dtype) || !dtype_ok(y_dtype)) return HAWK_ERR_BAD_DTYPE;
+    if (B < 1 || T < 1 || D < 1 || W < 1 || W > 8 || B > kMaxGridY) return HAWK_ERR_BAD_SHAPE;
+    if (W != 4 && T > kMaxGridY) return HAWK_ERR_BAD_SHAPE;
+    if (!aligned16(x) || !aligned16(y) || (state && !aligned16(state))) return HAWK_ERR_ALIGNMENT;
+    return hawk::conv1d_fwd(x, w, bias, state, y, B, T, D, W, x_dtype, y_dtype, as_stream(stream));
+}
+
+size_t hawk_conv1d_bwd_workspace_bytes(int B, int T, int D, int W) {
+    if (B < 1 || T < 1 || D < 1 || W < 1 || W > 8) return 0;
+    return hawk::conv1d_bwd_workspace_bytes(B, T, D, W);
+}
+
+int hawk_conv1d_bwd(const void* grad_y, const void* x, const float* w, void* dx, float* dw, float* db, int B, int T,
+                    int D, int W, int x_dtype, int gy_dtype, void* workspace_device, size_t workspace_bytes,
+                    void* stream) {
+    if (!grad_y || !x || !w || !dx || !dw || !db) return HAWK_ERR_NULL_POINTER;
+    if (!dtype_ok(x_dtype) || !dtype_ok(gy_dtype)) return HAWK_ERR_BAD_DTYPE;
+    if (B < 1 || T < 1 || D < 1 || W < 1 || W > 8 || B > kMaxGridY) return HAWK_ERR_BAD_SHAPE;
+    if (!aligned16(grad_y) || !aligned16(x) || !aligned16(dx)) return HAWK_ERR_ALIGNMENT;
+    if (workspace_device == nullptr) return HAWK_ERR_WORKSPACE;
+    return hawk::conv1d_bwd(grad_y, x, w, dx, dw, db, B, T, D, W, x_dtype, gy_dtype, workspace_device,
+                            workspace_bytes, as_stream(stream));
+}
+
+int hawk_conv1d_step(void* conv_state, const void* x_new, const float* w, const float* bias, void* y, int B, int D,
+                     int W, int dtype, int y_dtype, void* stream) {
+    if (!x_new || !w || !bias || !y || (W > 1 && !conv_state)) return HAWK_ERR_NULL_POINTER;
+    if (!dtype_ok(dtype) || !dtype_ok(y_dtype)) return HAWK_ERR_BAD_DTYPE;
+    if (B < 1 || D < 1 || W < 1 || W > 8 || B > kMaxGridY) return HAWK_ERR_BAD_SHAPE;
+    if (!aligned16(x_new) || !aligned16(y) || (conv_state && !aligned16(conv_state))) return HAWK_ERR_ALIGNMENT;
+    return hawk::conv1d_step(conv_state, x_new, w, bias, y, B, D, W, dtype, y_dtype, as_stream(stream));
+}
+
+int hawk_rglru_step(const void* x, const void* x_rg_lru, const void* a_rg_lru, const float* a_param,
+                    void* recc_state, void* h_out, int B, int D, int dtype, int state_dtype, void* stream) {
+    if (!x || !x_rg_lru || !a_rg_lru || !a_param || !recc_state || !h_out) return HAWK_ERR_NULL_POINTER;
+    if (!dtype_ok(dtype) || !dtype_ok(state_dtype)) return HAWK_ERR_BAD_DTYPE;
+    if (B < 1 || D < 1 || B > kMaxGridY) return HAWK_ERR_BAD_SHAPE;
+    if (!aligned16(x) || !aligned16(x_rg_lru) || !aligned16(a_rg_lru) || !aligned16(recc_state) || !aligned16(h_out))
+        return HAWK_ERR_ALIGNMENT;
+    return hawk::rglru_step(x, x_rg_lru, a_rg_lru, a_param, recc_state, h_out, B, D, dtype, state_dtype,
+                            as_stream(stream));
+}
+
+}  // extern "C"

@@ -1,0 +1,143 @@
+// Device-side helpers shared by the RG-LRU scan, conv1d and decode-step kernels (gfx950).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace hawk {
+
+constexpr int kWave = 64;
+constexpr float kLog2e = 1.4426950408889634f;
+
+// ---------------------------------------------------------------------------------------
+// Element types.  Activations are either bf16 (stored as raw uint16_t) or fp32.
+// ---------------------------------------------------------------------------------------
+struct bf16_t {
+    uint16_t bits;
+};
+
+typedef __bf16 bf16x2_native __attribute__((ext_vector_type(2)));
+typedef float float2_native __attribute__((ext_vector_type(2)));
+// Native vector types for raw register images (accepted by the nontemporal builtins).
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+// Two fp32 -> packed bf16 pair, round-to-nearest-even (one v_cvt_pk_bf16_f32 on gfx950).
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+    float2_native v = {lo, hi};
+    bf16x2_native r = __builtin_convertvector(v, bf16x2_native);
+    return __builtin_bit_cast(uint32_t, r);
+}
+__device__ __forceinline__ uint16_t to_bf16_bits(float f) {
+    return __builtin_bit_cast(uint16_t, (__bf16)f);
+}
+__device__ __forceinline__ float bf16_lo(uint32_t w) { return __uint_as_float(w << 16); }
+__device__ __forceinline__ float bf16_hi(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
+
+// Raw register image of V consecutive elements of type ET.
+template <typename ET, int V>
+struct Raw;
+template <>
+struct Raw<bf16_t, 1> { typedef uint16_t type; };
+template <>
+struct Raw<bf16_t, 2> { typedef uint32_t type; };
+template <>
+struct Raw<bf16_t, 4> { typedef u32x2 type; };
+template <>
+struct Raw<bf16_t, 8> { typedef u32x4 type; };
+template <>
+struct Raw<float, 1> { typedef float type; };
+template <>
+struct Raw<float, 2> { typedef f32x2 type; };
+template <>
+struct Raw<float, 4> { typedef f32x4 type; };
+
+__device__ __forceinline__ void unpack(uint16_t r, float (&o)[1]) { o[0] = __uint_as_float((uint32_t)r << 16); }
+__device__ __forceinline__ void unpack(uint32_t r, float (&o)[2]) { o[0] = bf16_lo(r); o[1] = bf16_hi(r); }
+__device__ __forceinline__ void unpack(u32x2 r, float (&o)[4]) {
+    o[0] = bf16_lo(r.x); o[1] = bf16_hi(r.x); o[2] = bf16_lo(r.y); o[3] = bf16_hi(r.y);
+}
+__device__ __forceinline__ void unpack(u32x4 r, float (&o)[8]) {
+    o[0] = bf16_lo(r.x); o[1] = bf16_hi(r.x); o[2] = bf16_lo(r.y); o[3] = bf16_hi(r.y);
+    o[4] = bf16_lo(r.z); o[5] = bf16_hi(r.z); o[6] = bf16_lo(r.w); o[7] = bf16_hi(r.w);
+}
+__device__ __forceinline__ void unpack(float r, float (&o)[1]) { o[0] = r; }
+__device__ __forceinline__ void unpack(f32x2 r, float (&o)[2]) { o[0] = r.x; o[1] = r.y; }
+__device__ __forceinline__ void unpack(f32x4 r, float (&o)[4]) { o[0] = r.x; o[1] = r.y; o[2] = r.z; o[3] = r.w; }
+
+__device__ __forceinline__ void pack(const float (&v)[1], uint16_t& r) { r = to_bf16_bits(v[0]); }
+__device__ __forceinline__ void pack(const float (&v)[2], uint32_t& r) { r = pack_bf16x2(v[0], v[1]); }
+__device__ __forceinline__ void pack(const float (&v)[4], u32x2& r) {
+    r.x = pack_bf16x2(v[0], v[1]); r.y = pack_bf16x2(v[2], v[3]);
+}
+__device__ __forceinline__ void pack(const float (&v)[8], u32x4& r) {
+    r.x = pack_bf16x2(v[0], v[1]); r.y = pack_bf16x2(v[2], v[3]);
+    r.z = pack_bf16x2(v[4], v[5]); r.w = pack_bf16x2(v[6], v[7]);
+}
+__device__ __forceinline__ void pack(const float (&v)[1], float& r) { r = v[0]; }
+__device__ __forceinline__ void pack(const float (&v)[2], f32x2& r) { r.x = v[0]; r.y = v[1]; }
+__device__ __forceinline__ void pack(const float (&v)[4], f32x4& r) { r.x = v[0]; r.y = v[1]; r.z = v[2]; r.w = v[3]; }
+
+template <typename R>
+__device__ __forceinline__ R raw_zero() {
+    R r;
+    __builtin_memset(&r, 0, sizeof(R));
+    return r;
+}
+
+template <typename ET, int V>
+__device__ __forceinline__ typename Raw<ET, V>::type load_raw(const ET* p) {
+    return *reinterpret_cast<const typename Raw<ET, V>::type*>(p);
+}
+// Streaming store: the outputs are written once and not read again by this kernel.
+template <typename ET, int V>
+__device__ __forceinline__ void store_raw(ET* p, typename Raw<ET, V>::type r) {
+    __builtin_nontemporal_store(r, reinterpret_cast<typename Raw<ET, V>::type*>(p));
+}
+
+// ---------------------------------------------------------------------------------------
+// Transcendentals: one hardware instruction each (v_exp_f32, v_rcp_f32, v_sqrt_f32,
+// v_rsq_f32; about 1 ulp), which is what keeps the scan bandwidth-bound.
+// ---------------------------------------------------------------------------------------
+__device__ __forceinline__ float hw_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+__device__ __forceinline__ float hw_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
+__device__ __forceinline__ float hw_sqrt(float x) { return __builtin_amdgcn_sqrtf(x); }
+__device__ __forceinline__ float hw_rsq(float x) { return __builtin_amdgcn_rsqf(x); }
+
+// logistic(x) = 1 / (1 + 2^(-x log2 e)); saturates cleanly to 0 and 1 at +-inf.
+__device__ __forceinline__ float sigmoid_fast(float x) {
+    return hw_rcp(1.0f + hw_exp2(-kLog2e * x));
+}
+
+// 1 - exp(y) for y <= 0 without cancellation: a degree-8 series for |y| < 1/4
+// (truncation below 3e-9 relative), the direct form elsewhere (result >= 0.22).
+__device__ __forceinline__ float one_minus_exp(float y) {
+    float direct = 1.0f - hw_exp2(kLog2e * y);
+    float p = 1.0f / 40320.0f;
+    p = fmaf(p, y, 1.0f / 5040.0f);
+    p = fmaf(p, y, 1.0f / 720.0f);
+    p = fmaf(p, y, 1.0f / 120.0f);
+    p = fmaf(p, y, 1.0f / 24.0f);
+    p = fmaf(p, y, 1.0f / 6.0f);
+    p = fmaf(p, y, 0.5f);
+    p = fmaf(p, y, 1.0f);
+    float series = -y * p;
+    return (y > -0.25f) ? series : direct;
+}
+
+// Numerically safe softplus / logistic for the per-channel Lambda (evaluated once per
+// lane, not per element, so the precise library routines are affordable here).
+__device__ __forceinline__ float softplus_precise(float x) {
+    return x > 20.0f ? x : log1pf(expf(x));
+}
+__device__ __forceinline__ float sigmoid_precise(float x) {
+    if (x >= 0.0f) return 1.0f / (1.0f + expf(-x));
+    float e = expf(x);
+    return e / (1.0f + e);
+}
+
+__device__ __forceinline__ float clamp01(float z) { return fminf(fmaxf(z, 0.0f), 1.0f); }
+
+}  // namespace hawk

@@ -1,0 +1,34 @@
+// Internal C++ interface between the C ABI (hawk_capi.hip) and the kernel translation units.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+
+#include "../../include/hawk_hip.h"
+
+namespace hawk {
+
+// hawk_scan.hip
+size_t scan_workspace_bytes(int B, int T, int D, int dtype);
+int workspace_init(void* ws, size_t bytes, hipStream_t st);
+int workspace_status(const void* ws, hipStream_t st, int* flag);
+int scan_fwd(const void* x, const void* xg, const void* ag, const float* lam, void* h, int B, int T, int D,
+             int dtype, void* ws, size_t ws_bytes, hipStream_t st);
+int scan_bwd(const void* x, const void* xg, const void* ag, const float* lam, const void* hs, const void* gout,
+             void* dx, void* dxg, void* dag, float* dlam, int B, int T, int D, int dtype, void* ws,
+             size_t ws_bytes, hipStream_t st);
+
+// hawk_conv.hip
+int conv1d_fwd(const void* x, const float* w, const float* bias, const void* state, void* y, int B, int T, int D,
+               int W, int x_dtype, int y_dtype, hipStream_t st);
+size_t conv1d_bwd_workspace_bytes(int B, int T, int D, int W);
+int conv1d_bwd(const void* gy, const void* x, const float* w, void* dx, float* dw, float* db, int B, int T, int D,
+               int W, int x_dtype, int gy_dtype, void* ws, size_t ws_bytes, hipStream_t st);
+
+// hawk_step.hip
+int conv1d_step(void* conv_state, const void* x_new, const float* w, const float* bias, void* y, int B, int D,
+                int W, int dtype, int y_dtype, hipStream_t st);
+int rglru_step(const void* x, const void* xg, const void* ag, const float* lam, void* state, void* h_out, int B,
+               int D, int dtype, int state_dtype, hipStream_t st);
+
+}  // namespace hawk

@@ -1,0 +1,273 @@
+"""Building blocks around the scan: the temporal Conv1D (HIP kernels), the block-diagonal
+gate projection and the Lambda initialiser.
+
+``Conv1D`` keeps the module surface of upstream's hawk/external.py:12-98 (constructor
+arguments, parameter names ``w`` [temporal_width, width] and ``b`` [width], fp32) but its
+forward and backward are single streaming HIP kernels instead of a Python loop of
+slice / pad / concat / multiply passes differentiated by autograd.
+"""
+
+from __future__ import annotations
+
+import math
+from typing import Optional, Tuple
+
+import torch
+import torch.nn as nn
+from torch.autograd import Function
+
+from . import _lib
+
+MAX_TEMPORAL_WIDTH = 8
+
+
+# ---------------------------------------------------------------------------------------
+# conv1d custom ops
+# ---------------------------------------------------------------------------------------
+def _launch_conv_fwd(x, w, b, state, out_dtype) -> torch.Tensor:
+    tensors = [x, w, b] + ([state] if state is not None else [])
+    dev = _lib.require_cuda(*tensors)
+    x, w, b = _lib.dense16(x), _lib.dense16(w), _lib.dense16(b)
+    if state is not None:
+        state = _lib.dense16(state)
+    B, T, D = x.shape
+    W = w.shape[0]
+    y = torch.empty((B, T, D), dtype=out_dtype, device=dev)
+    lib = _lib.load()
+    with torch.cuda.device(dev):
+        status = lib.hawk_conv1d_fwd(
+            x.data_ptr(), w.data_ptr(), b.data_ptr(), _lib.ptr(state), y.data_ptr(),
+            B, T, D, W, _lib.dtype_code(x.dtype), _lib.dtype_code(out_dtype), _lib.stream_ptr(dev),
+        )
+    _lib.check("hawk_conv1d_fwd", status)
+    return y
+
+
+def _launch_conv_bwd(grad_y, x, w):
+    dev = _lib.require_cuda(grad_y, x, w)
+    grad_y, x, w = _lib.dense16(grad_y), _lib.dense16(x), _lib.dense16(w)
+    B, T, D = x.shape
+    W = w.shape[0]
+    dx = torch.empty_like(x)
+    dw = torch.empty((W, D), dtype=torch.float32, device=dev)
+    db = torch.empty((D,), dtype=torch.float32, device=dev)
+    lib = _lib.load()
+    nbytes = lib.hawk_conv1d_bwd_workspace_bytes(B, T, D, W)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    with torch.cuda.device(dev):
+        status = lib.hawk_conv1d_bwd(
+            grad_y.data_ptr(), x.data_ptr(), w.data_ptr(), dx.data_ptr(), dw.data_ptr(), db.data_ptr(),
+            B, T, D, W, _lib.dtype_code(x.dtype), _lib.dtype_code(grad_y.dtype),
+            ws.data_ptr(), ws.numel(), _lib.stream_ptr(dev),
+        )
+    _lib.check("hawk_conv1d_bwd", status)
+    return dx, dw, db
+
+
+@torch.library.custom_op("hawk_amd::conv1d_fwd", mutates_args=(), device_types="cuda")
+def _conv1d_fwd_op(
+    x: torch.Tensor, w: torch.Tensor, b: torch.Tensor, state: Optional[torch.Tensor], out_fp32: bool
+) -> torch.Tensor:
+    return _launch_conv_fwd(x, w, b, state, torch.float32 if out_fp32 else torch.bfloat16)
+
+
+@_conv1d_fwd_op.register_fake
+def _(x, w, b, state, out_fp32):
+    return torch.empty(x.shape, dtype=torch.float32 if out_fp32 else torch.bfloat16, device=x.device)
+
+
+@torch.library.custom_op("hawk_amd::conv1d_bwd", mutates_args=(), device_types="cuda")
+def _conv1d_bwd_op(
+    grad_y: torch.Tensor, x: torch.Tensor, w: torch.Tensor
+) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    return _launch_conv_bwd(grad_y, x, w)
+
+
+@_conv1d_bwd_op.register_fake
+def _(grad_y, x, w):
+    return (
+        torch.empty_like(x, memory_format=torch.contiguous_format),
+        torch.empty(w.shape, dtype=torch.float32, device=x.device),
+        torch.empty((x.shape[-1],), dtype=torch.float32, device=x.device),
+    )
+
+
+class _TemporalConv(Function):
+    """y = causal depthwise conv(x; w, b) with zero history; hand-written backward."""
+
+    @staticmethod
+    def forward(ctx, x, w, b, out_fp32: bool):
+        xc = x if x.is_contiguous() else x.contiguous()
+        ctx.save_for_backward(xc, w)
+        ctx.in_dtype = x.dtype
+        return _conv1d_fwd_op(xc, w, b, None, out_fp32)
+
+    @staticmethod
+    def backward(ctx, grad_y):  # type: ignore[override]
+        xc, w = ctx.saved_tensors
+        if grad_y.dtype not in (torch.bfloat16, torch.float32):
+            grad_y = grad_y.float()
+        gy = grad_y if grad_y.is_contiguous() else grad_y.contiguous()
+        dx, dw, db = _conv1d_bwd_op(gy, xc, w)
+        return dx, dw, db, None
+
+
+def temporal_conv1d(x, w, b, out_dtype: Optional[torch.dtype] = None, state=None):
+    """Functional form: x [B,T,D] (bf16 or fp32), w [W,D] fp32, b [D] fp32.
+
+    ``out_dtype`` defaults to the promotion of x and w dtypes (fp32), which is what
+    upstream's ``x_window * w`` produces (hawk/external.py:90).  With ``state``
+    ([B,W-1,D], the rows preceding x) no gradient is defined.
+    """
+    assert x.dim() == 3, f"expected x of shape [B,T,D], got {tuple(x.shape)}"
+    W, D = w.shape
+    assert x.shape[-1] == D and b.shape == (D,), "conv weight / bias do not match the channel count"
+    assert 1 <= W <= MAX_TEMPORAL_WIDTH, f"temporal width must be in [1, {MAX_TEMPORAL_WIDTH}]"
+    if x.dtype not in (torch.bfloat16, torch.float32):
+        x = x.float()
+    if out_dtype is None:
+        out_dtype = torch.promote_types(x.dtype, w.dtype)
+    assert out_dtype in (torch.bfloat16, torch.float32)
+    w32, b32 = w.float(), b.float()
+    if state is not None:
+        assert state.shape == (x.shape[0], W - 1, D)
+        xc = x if x.is_contiguous() else x.contiguous()
+        return _conv1d_fwd_op(xc, w32, b32, state.to(x.dtype), out_dtype == torch.float32)
+    return _TemporalConv.apply(x, w32, b32, out_dtype == torch.float32)
+
+
+class Conv1D(nn.Module):
+    """Causal depthwise temporal convolution, y_t = b + sum_s w[W-1-s] * x_{t-s}.
+
+    Drop-in for upstream's ``Conv1D(width, temporal_width)`` (hawk/external.py:12-47):
+    same parameters (``w`` drawn from N(0, w_init_variance_scale / temporal_width), ``b``
+    zero) and ``forward(x) -> y``.  ``out_dtype=None`` reproduces upstream's type
+    promotion (fp32 output for bf16 input); pass ``torch.bfloat16`` to keep activations
+    in bf16 and halve the write traffic.
+    """
+
+    def __init__(
+        self,
+        width: int,
+        temporal_width: int,
+        w_init_variance_scale: float = 0.01,
+        out_dtype: Optional[torch.dtype] = None,
+    ):
+        super().__init__()
+        self.width = width
+        self.temporal_width = temporal_width
+        self.w_init_variance_scale = w_init_variance_scale
+        self.out_dtype = out_dtype
+        self.w = nn.Parameter(torch.empty([temporal_width, width], dtype=torch.float32))
+        self.b = nn.Parameter(torch.empty([width], dtype=torch.float32))
+        self.reset_parameters()
+
+    def reset_parameters(self) -> None:
+        nn.init.normal_(self.w, mean=0.0, std=math.sqrt(self.w_init_variance_scale / self.temporal_width))
+        nn.init.zeros_(self.b)
+
+    def forward(self, x: torch.Tensor, state: Optional[torch.Tensor] = None) -> torch.Tensor:
+        return temporal_conv1d(x, self.w, self.b, self.out_dtype, state)
+
+    def step(self, conv_state: torch.Tensor, x_new: torch.Tensor) -> torch.Tensor:
+        """Decode step: rolls ``conv_state`` [B,W-1,D] in place and returns y [B,1,D]."""
+        return temporal_conv1d_step(conv_state, x_new, self.w, self.b, self.out_dtype)
+
+
+def temporal_conv1d_step(conv_state, x_new, w, b, out_dtype: Optional[torch.dtype] = None):
+    """One-token conv: window = concat(conv_state, x_new); conv_state is updated in place
+    (rolled up one row, x_new written last).  Replaces hawk/hawk.py:169-179 +
+    hawk/cache.py:37-43 upstream.  x_new is [B,1,D] or [B,D]; returns the same rank."""
+    W, D = w.shape
+    squeeze = x_new.dim() == 2
+    xn = x_new.reshape(x_new.shape[0], D)
+    B = xn.shape[0]
+    assert conv_state.shape == (B, W - 1, D), (
+        f"conv_state must be [B, W-1, D] = {(B, W - 1, D)}, got {tuple(conv_state.shape)}"
+    )
+    assert conv_state.is_contiguous(), "conv_state is updated in place and must be contiguous"
+    dev = _lib.require_cuda(conv_state, xn, w, b)
+    xn = _lib.dense16(xn.to(conv_state.dtype))
+    if out_dtype is None:
+        out_dtype = torch.promote_types(conv_state.dtype, w.dtype)
+    y = torch.empty((B, D), dtype=out_dtype, device=dev)
+    w32, b32 = _lib.dense16(w.detach().float()), _lib.dense16(b.detach().float())
+    with torch.cuda.device(dev):
+        status = _lib.load().hawk_conv1d_step(
+            conv_state.data_ptr(), xn.data_ptr(), w32.data_ptr(), b32.data_ptr(), y.data_ptr(),
+            B, D, W, _lib.dtype_code(conv_state.dtype), _lib.dtype_code(out_dtype), _lib.stream_ptr(dev),
+        )
+    _lib.check("hawk_conv1d_step", status)
+    return y if squeeze else y.unsqueeze(1)
+
+
+def rglru_step(x, x_rg_lru, a_rg_lru, a_param, recc_state):
+    """One-token RG-LRU update.  ``recc_state`` [B,1,D] or [B,D] is read and overwritten
+    with the new state; the new state is also returned in x's dtype and shape.
+    Replaces Hawk.inference_prologue + step + cache write (hawk/hawk.py:137-151, :196-198)."""
+    D = x.shape[-1]
+    shape = x.shape
+    B = x.numel() // D
+    assert recc_state.numel() == B * D and recc_state.is_contiguous()
+    dev = _lib.require_cuda(x, x_rg_lru, a_rg_lru, a_param, recc_state)
+    run_dtype = x.dtype if x.dtype in (torch.bfloat16, torch.float32) else torch.float32
+    xs = [_lib.dense16(t.reshape(B, D).to(run_dtype)) for t in (x, x_rg_lru, a_rg_lru)]
+    lam = _lib.dense16(a_param.detach().float())
+    h = torch.empty((B, D), dtype=run_dtype, device=dev)
+    with torch.cuda.device(dev):
+        status = _lib.load().hawk_rglru_step(
+            xs[0].data_ptr(), xs[1].data_ptr(), xs[2].data_ptr(), lam.data_ptr(),
+            recc_state.data_ptr(), h.data_ptr(), B, D,
+            _lib.dtype_code(run_dtype), _lib.dtype_code(recc_state.dtype), _lib.stream_ptr(dev),
+        )
+    _lib.check("hawk_rglru_step", status)
+    return h.reshape(shape)
+
+
+# ---------------------------------------------------------------------------------------
+# Pieces of the harness model that are not on the hot path (library GEMMs, initialisers).
+# ---------------------------------------------------------------------------------------
+def rnn_param_init(
+    tensor: torch.Tensor, min_rad: float, max_rad: float, transform: str = "softplus", eps: float = 1e-8
+) -> torch.Tensor:
+    """Draws Lambda so that exp(-softplus(Lambda))^2 is uniform in [min_rad^2, max_rad^2]
+    (same distribution as hawk/external.py:153-168 upstream)."""
+    if transform != "softplus":
+        raise NotImplementedError(f"transform {transform!r}")
+    with torch.no_grad():
+        u = torch.empty_like(tensor).uniform_(min_rad**2 + eps, max_rad**2 + eps)
+        # softplus(L) = -0.5 ln(u)  <=>  L = ln(u^(-1/2) - 1)
+        tensor.copy_(torch.log(torch.expm1(-0.5 * torch.log(u))))
+    return tensor
+
+
+class BlockDiagonalLinear(nn.Module):
+    """y = blockdiag(w_0..w_{n-1}) x + b: the gate projections of the RG-LRU.
+
+    Parameter names and shapes follow hawk/external.py:200-209 upstream (``w``
+    [num_blocks, block_width, block_width], ``b`` [num_blocks, block_width]).  The
+    contraction is a batched library GEMM (rocBLAS through torch.bmm-style einsum); it is
+    dense MFMA work and not part of the memory-bound scan path.
+    """
+
+    def __init__(self, width: int, num_blocks: int, w_init_variance_scale: float = 1.0, device=None, dtype=None):
+        super().__init__()
+        assert width % num_blocks == 0, "width must be divisible by num_blocks"
+        self.width = width
+        self.num_blocks = num_blocks
+        self.w_init_variance_scale = w_init_variance_scale
+        self.block_width = width // num_blocks
+        shape = (num_blocks, self.block_width, self.block_width)
+        self.w = nn.Parameter(torch.empty(shape, device=device, dtype=dtype))
+        self.b = nn.Parameter(torch.empty(shape[:2], device=device, dtype=dtype))
+        self.reset_parameters()
+
+    def reset_parameters(self) -> None:
+        nn.init.normal_(self.w, mean=0.0, std=math.sqrt(self.w_init_variance_scale / self.block_width))
+        nn.init.zeros_(self.b)
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        lead = x.shape[:-1]
+        xb = x.reshape(*lead, self.num_blocks, self.block_width)
+        yb = torch.einsum("...hi,hij->...hj", xb, self.w) + self.b
+        return yb.reshape(*lead, self.width)

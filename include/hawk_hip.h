@@ -1,0 +1,132 @@
+/*
+ * libhawk_hip: C ABI of the MI355X (gfx950) kernels for Hawk's RG-LRU hot path.
+ *
+ * Plain pointers and sizes only.  Every pointer named "device" must be device memory of
+ * the GPU that is current when the call is made.  All calls are asynchronous on `stream`
+ * (a hipStream_t passed as void*; NULL is the default stream) unless stated otherwise,
+ * never synchronise the device, never allocate or free memory, keep no host-side state,
+ * and may be called from any host thread.  Every function returns a hawk_status; nothing
+ * throws or aborts.
+ *
+ * Tensors are dense row-major: activations [B,T,D] (strides T*D, D, 1), Lambda [D] fp32,
+ * conv weight [W,D] fp32, conv bias [D] fp32, conv state [B,W-1,D], recurrent state [B,D].
+ * `dtype` is the element type of the activation tensors of that call.
+ *
+ * Citations name the interface of the upstream tree (fattorib/hawk-pytorch, paths under
+ * hawk/) that each entry point replaces.
+ */
+#ifndef HAWK_HIP_H_
+#define HAWK_HIP_H_
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum hawk_status {
+    HAWK_OK = 0,
+    HAWK_ERR_NULL_POINTER = 1,  /* a required pointer is NULL */
+    HAWK_ERR_BAD_SHAPE = 2,     /* a size is < 1, too large, or breaks a stated divisibility rule */
+    HAWK_ERR_BAD_DTYPE = 3,     /* dtype is not a hawk_dtype this entry point supports */
+    HAWK_ERR_WORKSPACE = 4,     /* workspace missing or smaller than the size query says */
+    HAWK_ERR_LAUNCH = 5,        /* the HIP runtime refused a launch or copy */
+    HAWK_ERR_ALIGNMENT = 6      /* a tensor pointer is not aligned to its element size */
+} hawk_status;
+
+typedef enum hawk_dtype {
+    HAWK_DTYPE_BF16 = 0, /* bf16 storage, fp32 arithmetic and state */
+    HAWK_DTYPE_F32 = 1
+} hawk_dtype;
+
+/* Library version (major*10000 + minor*100 + patch) and a static message per status. */
+int hawk_version(void);
+const char* hawk_status_string(int status);
+
+/* ---------------------------------------------------------------------------------------
+ * Scan workspace.  The scan passes carries between tiles through a caller-owned device
+ * buffer.  Query its size for a problem shape, allocate it, zero it ONCE with
+ * hawk_scan_workspace_init (stream-ordered), then pass it to any number of later scan
+ * calls of that or any smaller shape.  Calls that share a workspace must be ordered on
+ * one stream; concurrent streams need a workspace each.
+ * Upstream allocates nothing comparable: its kernels walk T serially
+ * (hawk/scan_fused.py:83, :199).
+ * ------------------------------------------------------------------------------------- */
+size_t hawk_scan_workspace_bytes(int B, int T, int D, int dtype);
+int hawk_scan_workspace_init(void* workspace_device, size_t workspace_bytes, void* stream);
+/* Synchronises `stream` and reports in *flag whether any scan on this workspace gave up
+ * waiting for a carry (0 = all carries arrived).  A non-zero flag means results of that
+ * launch are invalid and the workspace must be re-initialised. */
+int hawk_scan_workspace_status(const void* workspace_device, void* stream, int* flag);
+
+/* ---------------------------------------------------------------------------------------
+ * RG-LRU scan forward.
+ *   r = sigmoid(a_rg_lru), i = sigmoid(x_rg_lru), alpha = exp(-8 r softplus(Lambda)),
+ *   h_t = alpha_t h_{t-1} + sqrt(1 - alpha_t^2) (i_t x_t),  h_{-1} = 0.
+ * Replaces sequential_scan_forward / sequential_scan_fwd_kernel
+ * (hawk/scan_fused.py:319-360, :34-109).  Lambda stays fp32 for both dtypes.  Any D >= 1
+ * is accepted (upstream requires D % 64 == 0); even D takes the two-channels-per-lane
+ * path.  The workspace may be NULL when T fits one tile.
+ * ------------------------------------------------------------------------------------- */
+int hawk_rglru_scan_fwd(const void* x, const void* x_rg_lru, const void* a_rg_lru,
+                        const float* a_param, void* h, int B, int T, int D, int dtype,
+                        void* workspace_device, size_t workspace_bytes, void* stream);
+
+/* RG-LRU scan backward (reverse time).  Inputs are the forward's inputs, the saved h and
+ * the upstream gradient; outputs are dx, dx_rg_lru, da_rg_lru in `dtype` and
+ * da_param [D] fp32, already reduced over batch and time.
+ * Replaces sequential_scan_backward / sequential_scan_bwd_kernel and the trailing
+ * .sum(dim=0) (hawk/scan_fused.py:363-424, :112-317).  T = 1 is handled (the upstream
+ * kernel needs T >= 2).  The workspace is always required. */
+int hawk_rglru_scan_bwd(const void* x, const void* x_rg_lru, const void* a_rg_lru,
+                        const float* a_param, const void* h_saved, const void* grad_out,
+                        void* dx, void* dx_rg_lru, void* da_rg_lru, float* da_param, int B,
+                        int T, int D, int dtype, void* workspace_device,
+                        size_t workspace_bytes, void* stream);
+
+/* ---------------------------------------------------------------------------------------
+ * Temporal causal depthwise conv1d.
+ *   y[b,t,c] = bias[c] + sum_{s<W} w[W-1-s,c] x[b,t-s,c]
+ * Rows before t = 0 are zero, or are taken from `state` [B,W-1,D] (oldest row first,
+ * dtype of x) when it is not NULL.  Replaces Conv1D.forward (hawk/external.py:49-98).
+ * x and y may have different dtypes (upstream returns fp32 for bf16 x by promotion).
+ * 1 <= W <= 8.
+ * ------------------------------------------------------------------------------------- */
+int hawk_conv1d_fwd(const void* x, const float* w, const float* bias, const void* state,
+                    void* y, int B, int T, int D, int W, int x_dtype, int y_dtype,
+                    void* stream);
+
+/* Size of the scratch buffer hawk_conv1d_bwd needs for its dw/db partial sums. */
+size_t hawk_conv1d_bwd_workspace_bytes(int B, int T, int D, int W);
+
+/* Conv1d backward with zero history: dx (x_dtype), dw [W,D] fp32, db [D] fp32.
+ * Upstream has no hand-written backward; this is the adjoint autograd builds from
+ * hawk/external.py:78-93.  grad_y has dtype gy_dtype. */
+int hawk_conv1d_bwd(const void* grad_y, const void* x, const float* w, void* dx, float* dw,
+                    float* db, int B, int T, int D, int W, int x_dtype, int gy_dtype,
+                    void* workspace_device, size_t workspace_bytes, void* stream);
+
+/* ---------------------------------------------------------------------------------------
+ * Decode steps (one new token per batch row).
+ * ------------------------------------------------------------------------------------- */
+
+/* conv_state [B,W-1,D] is consumed and updated in place (rolled up one row, x_new written
+ * last); y [B,D] is the conv output for the new token.  Replaces the
+ * concat / RNNCache.update_conv_cache / Conv1D / last-row slice sequence
+ * (hawk/hawk.py:169-179, hawk/cache.py:37-43).  state, x_new share `dtype`; y has y_dtype. */
+int hawk_conv1d_step(void* conv_state, const void* x_new, const float* w, const float* bias,
+                     void* y, int B, int D, int W, int dtype, int y_dtype, void* stream);
+
+/* h = alpha * recc_state + sqrt(1-alpha^2) (i x); recc_state [B,D] (state_dtype) is read,
+ * then overwritten with h; h_out [B,D] (`dtype`) also receives h.  Replaces
+ * Hawk.inference_prologue + step + RNNCache.update_cache (hawk/hawk.py:137-151, :196-198,
+ * hawk/cache.py:29-35).  x, x_rg_lru, a_rg_lru are [B,D] of `dtype`. */
+int hawk_rglru_step(const void* x, const void* x_rg_lru, const void* a_rg_lru,
+                    const float* a_param, void* recc_state, void* h_out, int B, int D,
+                    int dtype, int state_dtype, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* HAWK_HIP_H_ */

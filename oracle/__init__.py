@@ -1,0 +1,139 @@
+"""TEST INFRASTRUCTURE, NOT PRODUCT CODE.
+
+numpy front end of the C oracle in ``rglru_oracle.c`` (fp64 ground truth and a scalar fp32
+port of the same loops).  Only ``tests/``, ``__graft_entry__.smoke()`` and the
+``cpu_baseline`` leg of ``bench.py`` may import this package.
+
+Every function here takes and returns numpy arrays; nothing touches a GPU.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "_build", "librglru_oracle.so")
+_lib = None
+
+
+def build(force: bool = False) -> str:
+    """Compile the C oracle with gcc (``make`` in this directory)."""
+    if force:
+        subprocess.run(["make", "-C", _HERE, "clean"], check=True, capture_output=True)
+    subprocess.run(["make", "-C", _HERE], check=True, capture_output=True)
+    return _LIB_PATH
+
+
+def _load():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB_PATH):
+            build()
+        _lib = ctypes.CDLL(_LIB_PATH)
+    return _lib
+
+
+def _np_dtype(precision: str):
+    if precision == "f64":
+        return np.float64
+    if precision == "f32":
+        return np.float32
+    raise ValueError(f"precision must be 'f64' or 'f32', got {precision!r}")
+
+
+def _prep(a, dt):
+    return np.ascontiguousarray(np.asarray(a), dtype=dt)
+
+
+def _ptr(a):
+    return a.ctypes.data_as(ctypes.c_void_p) if a is not None else None
+
+
+def rglru_scan_fwd(x, x_rg_lru, a_rg_lru, a_param, precision: str = "f64"):
+    """h[B,T,D] of the RG-LRU scan (restates hawk/scan_fused.py:44-109)."""
+    dt = _np_dtype(precision)
+    x, xg, ag, lam = (_prep(v, dt) for v in (x, x_rg_lru, a_rg_lru, a_param))
+    B, T, D = x.shape
+    assert xg.shape == x.shape and ag.shape == x.shape and lam.shape == (D,)
+    h = np.empty_like(x)
+    fn = getattr(_load(), f"oracle_rglru_scan_fwd_{precision}")
+    fn(_ptr(x), _ptr(xg), _ptr(ag), _ptr(lam), _ptr(h), B, T, D)
+    return h
+
+
+def rglru_scan_bwd(x, x_rg_lru, a_rg_lru, a_param, h_saved, grad_out, precision: str = "f64"):
+    """(dx, dx_rg_lru, da_rg_lru, dLambda[D]) (restates hawk/scan_fused.py:123-317, :424)."""
+    dt = _np_dtype(precision)
+    x, xg, ag, lam, hs, go = (
+        _prep(v, dt) for v in (x, x_rg_lru, a_rg_lru, a_param, h_saved, grad_out)
+    )
+    B, T, D = x.shape
+    assert hs.shape == x.shape and go.shape == x.shape
+    dx, dxg, dag = np.empty_like(x), np.empty_like(x), np.empty_like(x)
+    dlam = np.empty(D, dtype=dt)
+    fn = getattr(_load(), f"oracle_rglru_scan_bwd_{precision}")
+    fn(_ptr(x), _ptr(xg), _ptr(ag), _ptr(lam), _ptr(hs), _ptr(go),
+       _ptr(dx), _ptr(dxg), _ptr(dag), _ptr(dlam), B, T, D)
+    return dx, dxg, dag, dlam
+
+
+def conv1d_fwd(x, w, b, state=None, precision: str = "f64"):
+    """y[B,T,D] of the causal depthwise temporal conv (restates hawk/external.py:49-95)."""
+    dt = _np_dtype(precision)
+    x, w, b = _prep(x, dt), _prep(w, dt), _prep(b, dt)
+    B, T, D = x.shape
+    W = w.shape[0]
+    assert w.shape == (W, D) and b.shape == (D,)
+    if state is not None:
+        state = _prep(state, dt)
+        assert state.shape == (B, W - 1, D)
+    y = np.empty_like(x)
+    fn = getattr(_load(), f"oracle_conv1d_fwd_{precision}")
+    fn(_ptr(x), _ptr(w), _ptr(b), _ptr(state), _ptr(y), B, T, D, W)
+    return y
+
+
+def conv1d_bwd(grad_y, x, w, precision: str = "f64"):
+    """(dx, dw, db): adjoint of conv1d_fwd with zero history."""
+    dt = _np_dtype(precision)
+    gy, x, w = _prep(grad_y, dt), _prep(x, dt), _prep(w, dt)
+    B, T, D = x.shape
+    W = w.shape[0]
+    dx = np.empty_like(x)
+    dw = np.empty((W, D), dtype=dt)
+    db = np.empty(D, dtype=dt)
+    fn = getattr(_load(), f"oracle_conv1d_bwd_{precision}")
+    fn(_ptr(gy), _ptr(x), _ptr(w), _ptr(dx), _ptr(dw), _ptr(db), B, T, D, W)
+    return dx, dw, db
+
+
+def rglru_step(x, x_rg_lru, a_rg_lru, a_param, state, precision: str = "f64"):
+    """One decode step h[B,D] (restates hawk/hawk.py:137-151, :196)."""
+    dt = _np_dtype(precision)
+    x, xg, ag, lam, st = (_prep(v, dt) for v in (x, x_rg_lru, a_rg_lru, a_param, state))
+    B, D = x.shape
+    h = np.empty_like(x)
+    fn = getattr(_load(), f"oracle_rglru_step_{precision}")
+    fn(_ptr(x), _ptr(xg), _ptr(ag), _ptr(lam), _ptr(st), _ptr(h), B, D)
+    return h
+
+
+def conv1d_step(conv_state, x_new, w, b, precision: str = "f64"):
+    """One decode step of the conv: returns (y[B,D], new_state[B,W-1,D]).
+
+    Restates hawk/hawk.py:169-179 with hawk/cache.py:37-43.
+    """
+    dt = _np_dtype(precision)
+    st = np.array(conv_state, dtype=dt, order="C", copy=True)
+    xn, w, b = _prep(x_new, dt), _prep(w, dt), _prep(b, dt)
+    B, D = xn.shape
+    W = w.shape[0]
+    assert st.shape == (B, W - 1, D)
+    y = np.empty_like(xn)
+    fn = getattr(_load(), f"oracle_conv1d_step_{precision}")
+    fn(_ptr(st), _ptr(xn), _ptr(w), _ptr(b), _ptr(y), B, D, W)
+    return y, st
