@@ -1,0 +1,221 @@
+#!/usr/bin/env python3
+"""Benchmark of the RG-LRU scan hot path on one MI355X.
+
+A step is one forward scan plus one backward scan over one synthetic batch, called
+through the C ABI of libhawk_hip.so with every buffer already resident in HBM and
+pre-allocated (nothing is allocated inside the timed region).
+
+Default workload: B=8, T=4096, D=2560, bf16 activations, fp32 state (the configuration
+the 70 %-of-HBM-peak target is quoted on).  ``--workload long`` runs B=2, T=32768,
+D=4096; ``--workload scan_conv`` adds the temporal conv1d forward and backward.
+
+Prints one JSON line:
+  value        tokens/s = B*T / (wall time per step), whole job on one GPU
+  roofline     for the dominant kernel (the backward scan): algorithmic bytes per launch
+               (16 B/element in bf16: five tensors read, three written) over the mean
+               duration of the backward launch measured with HIP events on the launch
+               stream, against the 8 TB/s HBM peak
+  cpu_baseline the PyTorch CPU loop over time of the same recurrence (forward + autograd
+               backward, fp32) on this host's cores, on a bounded sample of the workload
+"""
+
+from __future__ import annotations
+
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+import numpy as np
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+
+WORKLOADS = {
+    # name: (B, T, D, a^8 range, includes conv)
+    "scan": (8, 4096, 2560, (0.9, 0.999), False),
+    "long": (2, 32768, 4096, (0.99, 0.9999), False),
+    "scan_conv": (8, 4096, 2560, (0.9, 0.999), True),
+}
+
+
+def lambda_for_a8_range(gen, D, lo, hi):
+    u = torch.empty(D, dtype=torch.float64).uniform_(lo, hi, generator=gen)
+    return torch.log(u.pow(-1.0 / 8.0) - 1.0).float()
+
+
+def cpu_baseline(B, D, lo, hi, seed, budget_rows=512):
+    """PyTorch CPU loop (oracle/rglru_torch.py) on the first `budget_rows` time rows of the
+    workload's shape: forward plus autograd backward in fp32."""
+    from oracle import rglru_torch
+
+    gen = torch.Generator().manual_seed(seed)
+    T = budget_rows
+    x, xg, ag, go = (torch.randn(B, T, D, generator=gen) for _ in range(4))
+    lam = lambda_for_a8_range(gen, D, lo, hi)
+    rglru_torch.rglru_scan_fwd_bwd(x[:, :8], xg[:, :8], ag[:, :8], lam, go[:, :8])  # warm-up
+    t0 = time.perf_counter()
+    rglru_torch.rglru_scan_fwd_bwd(x, xg, ag, lam, go)
+    dt = time.perf_counter() - t0
+    return {
+        "value": B * T / dt,
+        "unit": "tokens/s",
+        "cores": torch.get_num_threads(),
+        "kind": "port",
+        "sample": f"first {T} of the time rows at B={B}, D={D}, fp32, forward + autograd backward, "
+                  f"{dt:.2f} s, host has {os.cpu_count()} logical cpus",
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", choices=sorted(WORKLOADS), default="scan")
+    ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+
+    if args.gpus != 1:
+        print("bench.py: this build runs on exactly one GPU (the path needs no collective); "
+              "--gpus must be 1", file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the HIP kernels have no CPU fallback", file=sys.stderr)
+        sys.exit(1)
+
+    from hawk_pytorch_amd import _lib
+
+    lib = _lib.load()
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    B, T, D, (lo, hi), with_conv = WORKLOADS[args.workload]
+    N = B * T * D
+    code = _lib.HAWK_DTYPE_BF16
+    bf = torch.bfloat16
+
+    gen = torch.Generator(device=dev).manual_seed(args.seed)
+    x, xg, ag, gout = (torch.randn(B, T, D, device=dev, generator=gen).to(bf) for _ in range(4))
+    lam = lambda_for_a8_range(torch.Generator().manual_seed(args.seed), D, lo, hi).to(dev)
+    h = torch.empty_like(x)
+    dx, dxg, dag = torch.empty_like(x), torch.empty_like(x), torch.empty_like(x)
+    dlam = torch.empty(D, dtype=torch.float32, device=dev)
+    ws = torch.zeros(lib.hawk_scan_workspace_bytes(B, T, D, code), dtype=torch.uint8, device=dev)
+    if with_conv:
+        W = 4
+        cw = (torch.randn(W, D, device=dev, generator=gen) * 0.5).float()
+        cb = torch.zeros(D, device=dev)
+        u = torch.empty_like(x)       # conv output, the scan's x
+        du = torch.empty_like(x)      # conv input gradient
+        dw = torch.empty(W, D, device=dev)
+        db = torch.empty(D, device=dev)
+        cws = torch.empty(lib.hawk_conv1d_bwd_workspace_bytes(B, T, D, W), dtype=torch.uint8, device=dev)
+    stream = torch.cuda.current_stream(dev).cuda_stream
+
+    def fwd():
+        src = x
+        if with_conv:
+            _lib.check("conv_fwd", lib.hawk_conv1d_fwd(x.data_ptr(), cw.data_ptr(), cb.data_ptr(), None,
+                                                       u.data_ptr(), B, T, D, W, code, code, stream))
+            src = u
+        _lib.check("scan_fwd", lib.hawk_rglru_scan_fwd(src.data_ptr(), xg.data_ptr(), ag.data_ptr(),
+                                                       lam.data_ptr(), h.data_ptr(), B, T, D, code,
+                                                       ws.data_ptr(), ws.numel(), stream))
+
+    def bwd():
+        src = u if with_conv else x
+        _lib.check("scan_bwd", lib.hawk_rglru_scan_bwd(src.data_ptr(), xg.data_ptr(), ag.data_ptr(),
+                                                       lam.data_ptr(), h.data_ptr(), gout.data_ptr(),
+                                                       dx.data_ptr(), dxg.data_ptr(), dag.data_ptr(),
+                                                       dlam.data_ptr(), B, T, D, code, ws.data_ptr(),
+                                                       ws.numel(), stream))
+
+    def conv_bwd():
+        _lib.check("conv_bwd", lib.hawk_conv1d_bwd(dx.data_ptr(), x.data_ptr(), cw.data_ptr(), du.data_ptr(),
+                                                   dw.data_ptr(), db.data_ptr(), B, T, D, W, code, code,
+                                                   cws.data_ptr(), cws.numel(), stream))
+
+    for _ in range(args.warmup):
+        fwd()
+        bwd()
+        if with_conv:
+            conv_bwd()
+    torch.cuda.synchronize()
+
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
+    t0 = time.perf_counter()
+    for k in range(args.steps):
+        ev[k][0].record()
+        fwd()
+        ev[k][1].record()
+        bwd()
+        ev[k][2].record()
+        if with_conv:
+            conv_bwd()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+
+    flag = ctypes.c_int(0)
+    _lib.check("status", lib.hawk_scan_workspace_status(ws.data_ptr(), stream, ctypes.byref(flag)))
+    if flag.value != 0:
+        print("bench.py: a scan tile gave up waiting for its carry; results are invalid", file=sys.stderr)
+        sys.exit(1)
+
+    fwd_ms = float(np.mean([e[0].elapsed_time(e[1]) for e in ev]))
+    bwd_ms = float(np.mean([e[1].elapsed_time(e[2]) for e in ev]))
+    ms_per_step = wall * 1e3 / args.steps
+    elem = 2  # bytes per bf16 activation element
+    fwd_bytes = 4 * elem * N + (2 * elem * N if with_conv else 0)
+    bwd_bytes = 8 * elem * N
+    step_bytes = 12 * elem * N + (5 * elem * N if with_conv else 0)
+    bwd_gbs = bwd_bytes / (bwd_ms * 1e-3) / 1e9
+
+    out = {
+        "metric": "RG-LRU scan fwd+bwd tokens/s and achieved HBM GB/s (% of peak), 1 GPU",
+        "value": B * T / (ms_per_step * 1e-3),
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16 in/out, f32 state and accumulation",
+        "data": f"synthetic, seed {args.seed}: x, gate logits, grad ~ N(0,1); a^8 ~ U({lo},{hi})",
+        "config": {
+            "workload": f"{args.workload}: RG-LRU scan"
+                        + (" + temporal conv1d (W=4)" if with_conv else "")
+                        + f" fwd+bwd, B={B}, T={T}, D={D}, bf16",
+            "B": B, "T": T, "D": D,
+        },
+        "roofline": {
+            "bound": "hbm",
+            "kernel": "rglru_scan_bwd_kernel (+ dlam_reduce_kernel, same launch call)",
+            "achieved": bwd_gbs,
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": bwd_gbs / HBM_PEAK_GBS,
+            "traffic": None,
+            "algorithmic_bytes_per_launch": bwd_bytes,
+            "launch_ms": bwd_ms,
+        },
+        "fwd": {"ms": fwd_ms, "GBs": fwd_bytes / (fwd_ms * 1e-3) / 1e9,
+                "frac": fwd_bytes / (fwd_ms * 1e-3) / 1e9 / HBM_PEAK_GBS},
+        "step_hbm": {"GBs": step_bytes / (ms_per_step * 1e-3) / 1e9,
+                     "frac": step_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS},
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(B, D, lo, hi, args.seed)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -16,10 +16,10 @@
 //   1. each lane scans its TC rows from a zero state, keeping per row the running product
 //      P_j and the local state H_j, and ends with the slice aggregate (P, H);
 //   2. slice aggregates are combined across the NW waves through LDS;
-//   3. tile aggregates are combined across workgroups with a decoupled look-back over
-//      per-channel words in a caller-provided workspace: a tile first publishes its
-//      aggregate, then walks back over its predecessors (taking an inclusive state where
-//      one is already there, an aggregate otherwise), then publishes its inclusive state;
+//   3. tile aggregates are combined across workgroups with a look-back over per-channel
+//      words in a caller-provided workspace: a tile publishes its aggregate, folds the
+//      aggregates of its predecessors back to the nearest checkpoint tile, and adds that
+//      checkpoint's inclusive state (checkpoint tiles publish theirs once they have it);
 //   4. the carry is applied: h_j = H_j + P_j * carry, rounded once and stored.
 // The backward runs the same machinery in reverse time on c_t = alpha_t (gout_t + c_{t+1}).
 //
@@ -59,9 +59,18 @@ __device__ __forceinline__ bool try_read(const unsigned long long* p, uint32_t t
     return (uint32_t)(w >> 32) == tag;
 }
 
-// Walk back over the predecessors of chain position `pos` (pos >= 1) for one channel and
-// return the state carried into this tile.  `stride` is the distance in words between
-// consecutive chain positions of the same channel.
+// Every kCheckpointEvery-th chain position is a checkpoint: it publishes the inclusive
+// state at its end; every other position publishes only its own aggregate.  A tile folds
+// the aggregates of its predecessors back to the nearest checkpoint and finishes with that
+// checkpoint's inclusive state.  The order of the floating-point operations is therefore
+// fixed by the position alone, never by timing, so results are bitwise reproducible, and
+// the serial dependency runs over checkpoints only (nseg / kCheckpointEvery hops).
+constexpr int kCheckpointEvery = 8;
+
+__device__ __forceinline__ bool is_checkpoint(int pos) { return (pos % kCheckpointEvery) == 0; }
+
+// Return the state carried into chain position `pos` (pos >= 1) for one channel.  `stride`
+// is the distance in words between consecutive chain positions of the same channel.
 __device__ __forceinline__ float look_back(const ScanWsPtrs& ws, size_t idx_pos0, size_t stride,
                                            int pos, uint32_t tag) {
     float acc_p = 1.0f, acc_h = 0.0f;
@@ -69,16 +78,19 @@ __device__ __forceinline__ float look_back(const ScanWsPtrs& ws, size_t idx_pos0
     uint32_t spins = 0;
     while (true) {
         const size_t idx = idx_pos0 + (size_t)j * stride;
-        float vi;
-        if (try_read(ws.incl + idx, tag, vi)) return fmaf(acc_p, vi, acc_h);
-        float vp, vh;
-        const bool okp = try_read(ws.agg_p + idx, tag, vp);
-        const bool okh = try_read(ws.agg_h + idx, tag, vh);
-        if (okp && okh && j > 0) {
-            acc_h = fmaf(acc_p, vh, acc_h);
-            acc_p *= vp;
-            --j;
-            continue;
+        if (is_checkpoint(j)) {
+            float vi;
+            if (try_read(ws.incl + idx, tag, vi)) return fmaf(acc_p, vi, acc_h);
+        } else {
+            float vp, vh;
+            const bool okp = try_read(ws.agg_p + idx, tag, vp);
+            const bool okh = try_read(ws.agg_h + idx, tag, vh);
+            if (okp && okh) {
+                acc_h = fmaf(acc_p, vh, acc_h);
+                acc_p *= vp;
+                --j;
+                continue;
+            }
         }
         if (++spins > kSpinLimit) {
             __hip_atomic_store(ws.ctrl + kError, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -231,17 +243,20 @@ __global__ __launch_bounds__(NW * kWave) void rglru_scan_fwd_kernel(
             const size_t stride = (size_t)B * D;
             const size_t idx0 = (size_t)b * D + c0;  // chain position 0 of this channel
             const size_t idx = idx0 + (size_t)seg * stride;
-            if (seg > 0) {
+            const bool publishes = seg + 1 < nseg;
+            if (publishes && !is_checkpoint(seg)) {
 #pragma unroll
                 for (int v = 0; v < V; ++v) {
                     publish(ws.agg_p + idx + v, tag, p_tot[v]);
                     publish(ws.agg_h + idx + v, tag, h_tot[v]);
                 }
                 asm volatile("" ::: "memory");
+            }
+            if (seg > 0) {
 #pragma unroll
                 for (int v = 0; v < V; ++v) cin[v] = look_back(ws, idx0 + v, stride, seg, tag);
             }
-            if (seg + 1 < nseg) {
+            if (publishes && is_checkpoint(seg)) {
 #pragma unroll
                 for (int v = 0; v < V; ++v) publish(ws.incl + idx + v, tag, fmaf(p_tot[v], cin[v], h_tot[v]));
             }
@@ -417,17 +432,20 @@ __global__ __launch_bounds__(NW * kWave) void rglru_scan_bwd_kernel(
             const size_t stride = (size_t)B * D;
             const size_t idx0 = (size_t)b * D + c0;
             const size_t idx = idx0 + (size_t)pos * stride;
-            if (pos > 0) {
+            const bool publishes = pos + 1 < nseg;
+            if (publishes && !is_checkpoint(pos)) {
 #pragma unroll
                 for (int v = 0; v < V; ++v) {
                     publish(ws.agg_p + idx + v, tag, p_tot[v]);
                     publish(ws.agg_h + idx + v, tag, h_tot[v]);
                 }
                 asm volatile("" ::: "memory");
+            }
+            if (pos > 0) {
 #pragma unroll
                 for (int v = 0; v < V; ++v) cin[v] = look_back(ws, idx0 + v, stride, pos, tag);
             }
-            if (pos + 1 < nseg) {
+            if (publishes && is_checkpoint(pos)) {
 #pragma unroll
                 for (int v = 0; v < V; ++v) publish(ws.incl + idx + v, tag, fmaf(p_tot[v], cin[v], h_tot[v]));
             }

@@ -1,0 +1,120 @@
+"""Direct ctypes calls into libhawk_hip.so for the GPU tests: raw device pointers, sizes
+and a stream, exactly what a non-Python host would pass.  No torch op wrappers involved."""
+
+import ctypes
+
+import numpy as np
+import torch
+
+from hawk_pytorch_amd import _lib
+
+TORCH_DTYPE = {"f32": torch.float32, "bf16": torch.bfloat16}
+
+
+def to_dev(a, dtype):
+    return torch.from_numpy(np.ascontiguousarray(a)).to(device="cuda", dtype=TORCH_DTYPE[dtype]).contiguous()
+
+
+def to_np(t):
+    return t.detach().float().cpu().numpy().astype(np.float64)
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def new_workspace(B, T, D, dtype, through_init=True):
+    lib = _lib.load()
+    n = lib.hawk_scan_workspace_bytes(B, T, D, _lib.dtype_code(TORCH_DTYPE[dtype]))
+    assert n > 0
+    if through_init:
+        ws = torch.empty(n, dtype=torch.uint8, device="cuda")
+        ws.fill_(0xAB)  # garbage, so that the init call is what zeroes it
+        _lib.check("hawk_scan_workspace_init", lib.hawk_scan_workspace_init(ws.data_ptr(), n, _stream()))
+    else:
+        ws = torch.zeros(n, dtype=torch.uint8, device="cuda")
+    return ws
+
+
+def workspace_flag(ws):
+    flag = ctypes.c_int(-1)
+    _lib.check("hawk_scan_workspace_status",
+               _lib.load().hawk_scan_workspace_status(ws.data_ptr(), _stream(), ctypes.byref(flag)))
+    return flag.value
+
+
+def scan_fwd(x, xg, ag, lam, ws=None):
+    """x, xg, ag: device tensors [B,T,D] (bf16 or fp32); lam: device fp32 [D]."""
+    B, T, D = x.shape
+    h = torch.empty_like(x)
+    if ws is None:
+        ws = new_workspace(B, T, D, "bf16" if x.dtype == torch.bfloat16 else "f32")
+    rc = _lib.load().hawk_rglru_scan_fwd(
+        x.data_ptr(), xg.data_ptr(), ag.data_ptr(), lam.data_ptr(), h.data_ptr(), B, T, D,
+        _lib.dtype_code(x.dtype), ws.data_ptr(), ws.numel(), _stream())
+    _lib.check("hawk_rglru_scan_fwd", rc)
+    return h
+
+
+def scan_bwd(x, xg, ag, lam, h, gout, ws=None):
+    B, T, D = x.shape
+    dx, dxg, dag = torch.empty_like(x), torch.empty_like(x), torch.empty_like(x)
+    dlam = torch.empty(D, dtype=torch.float32, device="cuda")
+    if ws is None:
+        ws = new_workspace(B, T, D, "bf16" if x.dtype == torch.bfloat16 else "f32")
+    rc = _lib.load().hawk_rglru_scan_bwd(
+        x.data_ptr(), xg.data_ptr(), ag.data_ptr(), lam.data_ptr(), h.data_ptr(), gout.data_ptr(),
+        dx.data_ptr(), dxg.data_ptr(), dag.data_ptr(), dlam.data_ptr(), B, T, D,
+        _lib.dtype_code(x.dtype), ws.data_ptr(), ws.numel(), _stream())
+    _lib.check("hawk_rglru_scan_bwd", rc)
+    return dx, dxg, dag, dlam
+
+
+def conv_fwd(x, w, b, state=None, y_dtype=None):
+    B, T, D = x.shape
+    W = w.shape[0]
+    y_dtype = y_dtype or x.dtype
+    y = torch.empty((B, T, D), dtype=y_dtype, device="cuda")
+    rc = _lib.load().hawk_conv1d_fwd(
+        x.data_ptr(), w.data_ptr(), b.data_ptr(), None if state is None else state.data_ptr(), y.data_ptr(),
+        B, T, D, W, _lib.dtype_code(x.dtype), _lib.dtype_code(y_dtype), _stream())
+    _lib.check("hawk_conv1d_fwd", rc)
+    return y
+
+
+def conv_bwd(gy, x, w):
+    B, T, D = x.shape
+    W = w.shape[0]
+    lib = _lib.load()
+    dx = torch.empty_like(x)
+    dw = torch.empty((W, D), dtype=torch.float32, device="cuda")
+    db = torch.empty((D,), dtype=torch.float32, device="cuda")
+    n = lib.hawk_conv1d_bwd_workspace_bytes(B, T, D, W)
+    ws = torch.empty(n, dtype=torch.uint8, device="cuda")
+    rc = lib.hawk_conv1d_bwd(
+        gy.data_ptr(), x.data_ptr(), w.data_ptr(), dx.data_ptr(), dw.data_ptr(), db.data_ptr(), B, T, D, W,
+        _lib.dtype_code(x.dtype), _lib.dtype_code(gy.dtype), ws.data_ptr(), n, _stream())
+    _lib.check("hawk_conv1d_bwd", rc)
+    return dx, dw, db
+
+
+def conv_step(state, x_new, w, b, y_dtype=None):
+    B, D = x_new.shape
+    W = w.shape[0]
+    y_dtype = y_dtype or x_new.dtype
+    y = torch.empty((B, D), dtype=y_dtype, device="cuda")
+    rc = _lib.load().hawk_conv1d_step(
+        state.data_ptr(), x_new.data_ptr(), w.data_ptr(), b.data_ptr(), y.data_ptr(), B, D, W,
+        _lib.dtype_code(x_new.dtype), _lib.dtype_code(y_dtype), _stream())
+    _lib.check("hawk_conv1d_step", rc)
+    return y
+
+
+def rglru_step(x, xg, ag, lam, state):
+    B, D = x.shape
+    h = torch.empty_like(x)
+    rc = _lib.load().hawk_rglru_step(
+        x.data_ptr(), xg.data_ptr(), ag.data_ptr(), lam.data_ptr(), state.data_ptr(), h.data_ptr(), B, D,
+        _lib.dtype_code(x.dtype), _lib.dtype_code(state.dtype), _stream())
+    _lib.check("hawk_rglru_step", rc)
+    return h

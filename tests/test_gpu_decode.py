@@ -1,0 +1,90 @@
+"""GPU parity of the decode-step kernels and of the prefill -> decode hand-off."""
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+import capi
+from conftest import TOL, make_scan_inputs, max_rel
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+@pytest.mark.parametrize("B,D", [(1, 64), (1, 2560), (3, 130), (256, 2560), (5, 7)])
+def test_rglru_step(B, D, dtype):
+    x, xg, ag, lam, st = make_scan_inputs(B, 1, D, seed=B + D)
+    d = [capi.to_dev(a[:, 0], dtype) for a in (x, xg, ag, st)]
+    xr, xgr, agr, sr = (capi.to_np(t) for t in d)
+    lam_d = capi.to_dev(lam, "f32")
+    state = d[3].clone()
+    h = capi.rglru_step(d[0], d[1], d[2], lam_d, state)
+    ref = oracle.rglru_step(xr, xgr, agr, capi.to_np(lam_d), sr)
+    assert max_rel(capi.to_np(h), ref) < TOL[dtype]
+    assert torch.equal(state, h)  # the cache buffer now holds the new state
+
+
+def test_rglru_step_bf16_cache_fp32_activations():
+    """Upstream keeps the cache in bf16 while the step runs in fp32 (hawk/cache.py:12-17)."""
+    B, D = 4, 256
+    x, xg, ag, lam, st = make_scan_inputs(B, 1, D, seed=3)
+    d = [capi.to_dev(a[:, 0], "f32") for a in (x, xg, ag)]
+    state = capi.to_dev(st[:, 0], "bf16")
+    sr = capi.to_np(state)
+    lam_d = capi.to_dev(lam, "f32")
+    h = capi.rglru_step(d[0], d[1], d[2], lam_d, state)
+    ref = oracle.rglru_step(*(capi.to_np(t) for t in d), capi.to_np(lam_d), sr)
+    assert max_rel(capi.to_np(h), ref) < TOL["f32"]
+    assert torch.equal(state, h.to(torch.bfloat16))
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+@pytest.mark.parametrize("W", [1, 2, 4, 8])
+@pytest.mark.parametrize("B,D", [(1, 64), (256, 2560), (3, 30)])
+def test_conv_step(B, D, W, dtype):
+    rng = np.random.default_rng(B + D + W)
+    st = capi.to_dev(rng.standard_normal((B, max(W - 1, 1), D))[:, : W - 1], dtype) if W > 1 else None
+    xn = capi.to_dev(rng.standard_normal((B, D)), dtype)
+    w = capi.to_dev(rng.standard_normal((W, D)) * 0.5, "f32")
+    b = capi.to_dev(rng.standard_normal(D), "f32")
+    if W == 1:
+        st = torch.empty((B, 0, D), dtype=xn.dtype, device="cuda")
+        st_np = np.zeros((B, 0, D))
+        dummy = torch.zeros(16, device="cuda")  # a valid pointer for the unused state argument
+        y = capi.conv_step(dummy, xn, w, b)
+        ref_y, _ = oracle.conv1d_step(st_np, capi.to_np(xn), capi.to_np(w), capi.to_np(b))
+        assert max_rel(capi.to_np(y), ref_y) < TOL[dtype]
+        return
+    st = st.contiguous()
+    before = capi.to_np(st)
+    y = capi.conv_step(st, xn, w, b)
+    ref_y, ref_state = oracle.conv1d_step(before, capi.to_np(xn), capi.to_np(w), capi.to_np(b))
+    assert max_rel(capi.to_np(y), ref_y) < TOL[dtype]
+    assert np.array_equal(capi.to_np(st), ref_state)  # pure data movement: bit exact
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_prefill_then_steps_track_the_full_scan(dtype):
+    """scan over T rows, then K single-token steps from its last state, against the scan
+    over T+K rows; same for the conv with its rolling window."""
+    B, T, K, D, W = 2, 200, 5, 128, 4
+    x, xg, ag, lam, _ = make_scan_inputs(B, T + K, D, seed=17)
+    d = [capi.to_dev(a, dtype) for a in (x, xg, ag)]
+    lam_d = capi.to_dev(lam, "f32")
+    h_full = capi.scan_fwd(*d, lam_d)
+    h_pre = capi.scan_fwd(*(t[:, :T].contiguous() for t in d), lam_d)
+    state = h_pre[:, -1].contiguous().float()  # fp32 cache: no extra rounding between steps
+    for k in range(K):
+        row = [t[:, T + k].contiguous() for t in d]
+        h = capi.rglru_step(*row, lam_d, state)
+        assert max_rel(capi.to_np(h), capi.to_np(h_full[:, T + k])) < TOL[dtype]
+
+    rng = np.random.default_rng(4)
+    w = capi.to_dev(rng.standard_normal((W, D)) * 0.5, "f32")
+    b = capi.to_dev(rng.standard_normal(D), "f32")
+    y_full = capi.conv_fwd(d[0], w, b)
+    conv_state = d[0][:, T - (W - 1): T].contiguous()
+    for k in range(K):
+        y = capi.conv_step(conv_state, d[0][:, T + k].contiguous(), w, b)
+        assert max_rel(capi.to_np(y), capi.to_np(y_full[:, T + k])) < TOL[dtype]

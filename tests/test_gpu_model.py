@@ -1,0 +1,216 @@
+"""The operator boundary as the model uses it: autograd Function, autocast, Conv1D module,
+RNNCache, prefill -> decode, and torch.compile traceability.  All on the GPU."""
+
+import math
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+import oracle
+from oracle import rglru_torch
+import capi
+from conftest import TOL, make_scan_inputs, max_rel
+
+import hawk_pytorch_amd as hk
+
+pytestmark = pytest.mark.gpu
+
+
+def _leaves(B, T, D, dtype, seed=0):
+    x, xg, ag, lam, gout = make_scan_inputs(B, T, D, seed=seed)
+    td = capi.TORCH_DTYPE[dtype]
+    ts = [torch.tensor(a, device="cuda", dtype=td, requires_grad=True) for a in (x, xg, ag)]
+    lam_t = torch.tensor(lam, device="cuda", dtype=torch.float32, requires_grad=True)
+    return ts, lam_t, torch.tensor(gout, device="cuda", dtype=td)
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_fused_linear_scan_autograd(dtype):
+    (x, xg, ag), lam, gout = _leaves(2, 300, 128, dtype, seed=1)
+    h = hk.fused_linear_scan(x, xg, ag, lam)
+    assert h.dtype == x.dtype and h.shape == x.shape
+    h.backward(gout)
+    xr, xgr, agr = (capi.to_np(t) for t in (x, xg, ag))
+    h_ref = oracle.rglru_scan_fwd(xr, xgr, agr, capi.to_np(lam))
+    ref = oracle.rglru_scan_bwd(xr, xgr, agr, capi.to_np(lam), capi.to_np(h), capi.to_np(gout))
+    assert max_rel(capi.to_np(h), h_ref) < TOL[dtype]
+    for t, want in zip((x, xg, ag, lam), ref):
+        assert t.grad is not None and t.grad.dtype == t.dtype
+        assert max_rel(capi.to_np(t.grad), want) < TOL[dtype]
+
+
+def test_fused_linear_scan_under_autocast_casts_activations_not_lambda():
+    (x, xg, ag), lam, gout = _leaves(1, 130, 64, "f32", seed=2)
+    with torch.autocast(device_type="cuda", dtype=torch.bfloat16):
+        h = hk.fused_linear_scan(x, xg, ag, lam)
+    assert h.dtype == torch.bfloat16  # as upstream's custom_fwd(cast_inputs=bfloat16)
+    h.backward(gout.to(torch.bfloat16))
+    assert x.grad.dtype == torch.float32 and lam.grad.dtype == torch.float32
+    xr, xgr, agr = (capi.to_np(t.detach().to(torch.bfloat16)) for t in (x, xg, ag))
+    h_ref = oracle.rglru_scan_fwd(xr, xgr, agr, capi.to_np(lam))  # Lambda NOT rounded to bf16
+    assert max_rel(capi.to_np(h), h_ref) < TOL["bf16"]
+
+
+def test_scan_wrapper_contract_errors_and_copies():
+    (x, xg, ag), lam, gout = _leaves(1, 20, 64, "f32", seed=3)
+    with pytest.raises(AssertionError, match="multiple of 64"):
+        hk.sequential_scan_forward(x[..., :60], xg[..., :60], ag[..., :60], lam[:60])
+    # non-contiguous inputs are copied silently
+    xt = x.detach().transpose(0, 1).contiguous().transpose(0, 1)
+    assert not xt.is_contiguous() or xt.shape[0] == 1
+    h1 = hk.sequential_scan_forward(x.detach(), xg.detach(), ag.detach(), lam.detach())
+    big = torch.randn(1, 20, 128, device="cuda")
+    big[..., :64] = x.detach()
+    h2 = hk.sequential_scan_forward(big[..., :64], xg.detach(), ag.detach(), lam.detach())
+    assert torch.equal(h1, h2)
+    # non-contiguous grad_out: copied, with upstream's warning
+    go = torch.randn(1, 20, 128, device="cuda")[..., :64]
+    with pytest.warns(UserWarning, match="not contiguous"):
+        hk.sequential_scan_backward(x.detach(), xg.detach(), ag.detach(), lam.detach(), h1, go)
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_conv1d_module_forward_backward(dtype):
+    torch.manual_seed(0)
+    conv = hk.Conv1D(width=128, temporal_width=4).cuda()
+    with torch.no_grad():
+        conv.w.normal_(0, 0.5)
+        conv.b.normal_(0, 0.1)
+    td = capi.TORCH_DTYPE[dtype]
+    x = torch.randn(2, 90, 128, device="cuda").to(td).requires_grad_(True)
+    y = conv(x)
+    assert y.dtype == torch.float32  # promotion of x with the fp32 weight, as upstream
+    gy = torch.randn_like(y)
+    y.backward(gy)
+    xr = x.detach().float().clone().requires_grad_(True)
+    wr = conv.w.detach().clone().requires_grad_(True)
+    br = conv.b.detach().clone().requires_grad_(True)
+    y_ref = rglru_torch.conv1d_library(xr, wr, br)
+    y_ref.backward(gy)
+    assert max_rel(capi.to_np(y), capi.to_np(y_ref)) < 1e-4
+    assert max_rel(capi.to_np(x.grad), capi.to_np(xr.grad)) < TOL[dtype]
+    assert max_rel(capi.to_np(conv.w.grad), capi.to_np(wr.grad)) < 1e-4
+    assert max_rel(capi.to_np(conv.b.grad), capi.to_np(br.grad)) < 1e-4
+
+
+def test_rnn_cache_semantics_on_gpu():
+    c = hk.RNNCache(64, torch.device("cuda"), 4, batch_size=3)
+    assert c.recc_state.shape == (3, 1, 64) and c.conv_state.shape == (3, 3, 64)
+    assert c.recc_state.dtype == torch.bfloat16 and torch.isnan(c.conv_state.float()).all()
+    assert c.current_cache_size == 0
+    rows = [torch.randn(3, 1, 64, device="cuda").bfloat16() for _ in range(5)]
+    c.conv_state.zero_()
+    for r in rows:
+        before = c.conv_state.clone()
+        c.update_conv_cache(r)
+        assert torch.equal(c.conv_state, torch.cat([before[:, 1:], r], dim=1))  # roll(-1) + write last
+    c.update_cache(rows[0])
+    assert c.current_cache_size == 1 and torch.equal(c.recc_state, rows[0])
+    with pytest.raises(AssertionError):
+        c.update_cache(torch.zeros(2, 1, 64, device="cuda"))
+
+
+def _small_config():
+    return hk.HawkConfig(vocab_size=512, hidden_size=128, intermediate_size=256, num_hidden_layers=2,
+                         recurrent_size=128, num_blocks=4, conv_width=4)
+
+
+def _randomise_zero_inits(model):
+    """resid_proj and lm_head are zero at init, which silences the scan; redraw them."""
+    g = torch.Generator(device="cpu").manual_seed(5)
+    with torch.no_grad():
+        for name, p in model.named_parameters():
+            if name.endswith("resid_proj.weight") or name == "lm_head.weight":
+                p.copy_(torch.randn(p.shape, generator=g) / math.sqrt(p.shape[1]))
+
+
+def test_model_loss_at_init_is_log_vocab_and_only_lm_head_gets_gradient():
+    torch.manual_seed(0)
+    cfg = _small_config()
+    model = hk.HawkModel(cfg).cuda()
+    ids = torch.randint(1, cfg.vocab_size, (2, 96), device="cuda")
+    with torch.autocast(device_type="cuda", dtype=torch.bfloat16):
+        loss = model(ids, ids)
+    assert abs(float(loss) - math.log(cfg.vocab_size)) < 1e-4
+    loss.backward()
+    for name, p in model.named_parameters():
+        if name == "lm_head.weight":
+            assert p.grad.abs().max() > 0
+        elif p.grad is not None:
+            assert p.grad.abs().max() == 0, name
+
+
+def test_model_prefill_then_decode_matches_full_forward():
+    torch.manual_seed(1)
+    cfg = _small_config()
+    model = hk.HawkModel(cfg, use_cache=True).cuda().eval()
+    _randomise_zero_inits(model)
+    B, T, K = 3, 40, 4
+    ids = torch.randint(1, cfg.vocab_size, (B, T + K), device="cuda")
+    with torch.no_grad():
+        full_logits, _ = model(ids, layer_past=model.new_cache(B))
+        caches = model.new_cache(B)
+        for c in caches:  # fp32 caches so the comparison is not limited by cache rounding
+            c.recc_state = c.recc_state.float()
+            c.conv_state = c.conv_state.float()
+        logits, caches = model(ids[:, :T], layer_past=caches)
+        assert torch.allclose(logits, full_logits[:, :T], atol=1e-4, rtol=1e-4)
+        for k in range(K):
+            step_logits, caches = model(ids[:, T + k: T + k + 1], layer_past=caches)
+            assert step_logits.shape == (B, 1, cfg.vocab_size)
+            assert max_rel(capi.to_np(step_logits[:, 0]), capi.to_np(full_logits[:, T + k])) < 1e-3
+
+
+def test_model_gradients_match_a_pure_torch_model_of_the_same_weights():
+    """End-to-end fwd+bwd of the small model in fp32 against the same model with the scan
+    and conv swapped for the torch-loop oracle pieces."""
+    torch.manual_seed(2)
+    cfg = _small_config()
+    model = hk.HawkModel(cfg).cuda()
+    _randomise_zero_inits(model)
+    ids = torch.randint(1, cfg.vocab_size, (2, 48), device="cuda")
+    loss = model(ids, ids)
+    loss.backward()
+    got = {n: p.grad.detach().clone() for n, p in model.named_parameters()}
+
+    import hawk_pytorch_amd.hawk as hm
+    import hawk_pytorch_amd.external as he
+
+    def ref_scan(x, xg, ag, lam):
+        return rglru_torch.rglru_scan_loop(x, xg, ag, lam)
+
+    def ref_conv(self, x, state=None):
+        return rglru_torch.conv1d_library(x, self.w, self.b)
+
+    model.zero_grad()
+    old_scan, old_conv = hm.fused_linear_scan, he.Conv1D.forward
+    try:
+        hm.fused_linear_scan = ref_scan
+        he.Conv1D.forward = ref_conv
+        ref_loss = model(ids, ids)
+        ref_loss.backward()
+    finally:
+        hm.fused_linear_scan, he.Conv1D.forward = old_scan, old_conv
+    assert abs(float(loss) - float(ref_loss)) < 1e-4
+    for n, p in model.named_parameters():
+        assert max_rel(capi.to_np(got[n]), capi.to_np(p.grad)) < 1e-3, n
+
+
+def test_torch_compile_traces_the_ops_without_graph_breaks():
+    (x, xg, ag), lam, gout = _leaves(1, 70, 64, "f32", seed=4)
+    conv = hk.Conv1D(64, 4).cuda()
+
+    def fn(x, xg, ag, lam):
+        return hk.fused_linear_scan(conv(x), xg, ag, lam)
+
+    eager = fn(x, xg, ag, lam)
+    compiled = torch.compile(fn, backend="aot_eager", fullgraph=True)
+    out = compiled(x, xg, ag, lam)
+    assert torch.allclose(out, eager, atol=1e-6)
+    out.backward(gout)
+    g_compiled = x.grad.clone()
+    x.grad = None
+    fn(x, xg, ag, lam).backward(gout)
+    assert torch.allclose(g_compiled, x.grad, atol=1e-6)

@@ -1,0 +1,207 @@
+"""GPU parity of the RG-LRU scan kernels against the fp64 oracle, through the C ABI.
+
+Tolerances are the benchmark's: max-rel (max |err| / max |ref| per tensor) 1e-4 for fp32
+activations, 2e-2 for bf16 activations with fp32 state.  Inputs are rounded to the
+activation dtype first and the oracle sees exactly the rounded values.
+"""
+
+import numpy as np
+import pytest
+import scipy.signal
+import torch
+
+import oracle
+import capi
+from conftest import TOL, make_scan_inputs, max_rel
+
+pytestmark = pytest.mark.gpu
+
+
+def _round_inputs(arrs, dtype):
+    """Device tensors in `dtype` plus the fp64 numpy image of what the device holds."""
+    dev = [capi.to_dev(a, dtype) for a in arrs]
+    return dev, [capi.to_np(t) for t in dev]
+
+
+def _run_case(B, T, D, dtype, seed=0, lo=0.9, hi=0.999, ws=None, channels=None):
+    x, xg, ag, lam, gout = make_scan_inputs(B, T, D, seed=seed, lo=lo, hi=hi)
+    (dx_, dxg_, dag_, dgo_), (x, xg, ag, gout) = _round_inputs((x, xg, ag, gout), dtype)
+    lam_d = capi.to_dev(lam, "f32")
+    lam = capi.to_np(lam_d)
+    h_d = capi.scan_fwd(dx_, dxg_, dag_, lam_d, ws)
+    g_d = capi.scan_bwd(dx_, dxg_, dag_, lam_d, h_d, dgo_, ws)
+    torch.cuda.synchronize()
+    sl = slice(None) if channels is None else channels
+    h_ref = oracle.rglru_scan_fwd(x[..., sl], xg[..., sl], ag[..., sl], lam[sl])
+    tol = TOL[dtype]
+    h_gpu = capi.to_np(h_d)[..., sl]
+    assert max_rel(h_gpu, h_ref) < tol, ("h", B, T, D, dtype, max_rel(h_gpu, h_ref))
+    # the backward consumes the h the forward stored (rounded to dtype), as upstream does
+    ref = oracle.rglru_scan_bwd(x[..., sl], xg[..., sl], ag[..., sl], lam[sl], h_gpu, gout[..., sl])
+    names = ("dx", "dx_rg_lru", "da_rg_lru", "da_param")
+    for name, got, want in zip(names, g_d, ref):
+        got = capi.to_np(got)[..., sl]
+        assert np.all(np.isfinite(got)), name
+        assert max_rel(got, want) < tol, (name, B, T, D, dtype, max_rel(got, want))
+    # and the whole fwd+bwd chain against the all-fp64 chain
+    ref64 = oracle.rglru_scan_bwd(x[..., sl], xg[..., sl], ag[..., sl], lam[sl], h_ref, gout[..., sl])
+    for name, got, want in zip(names, g_d, ref64):
+        assert max_rel(capi.to_np(got)[..., sl], want) < tol, (name + " (fp64 chain)", B, T, D, dtype)
+    return h_d, g_d
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_config0_shape(dtype):
+    """B=1, T=256, D=512: the CPU-reference configuration of the benchmark definition."""
+    _run_case(1, 256, 512, dtype, seed=0)
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+@pytest.mark.parametrize("T", [1, 2, 3, 7, 8, 9, 63, 64, 65, 127, 128, 129, 200, 257, 1000])
+def test_time_lengths_around_tile_edges(T, dtype):
+    _run_case(2, T, 128, dtype, seed=T)
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+@pytest.mark.parametrize("D", [1, 2, 3, 64, 66, 128, 130, 192, 320, 1000])
+def test_channel_counts_including_ragged_tiles(D, dtype):
+    """The C ABI takes any D; odd D runs one channel per lane, and D that does not fill the
+    last channel tile leaves lanes idle."""
+    _run_case(2, 150, D, dtype, seed=100 + D)
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_many_tiles_long_memory(dtype):
+    """Long-memory regime of the long-context configuration (alpha^8 in [0.99, 0.9999]) over
+    many time tiles: the carry chain is what is exercised."""
+    _run_case(1, 8192, 128, dtype, seed=5, lo=0.99, hi=0.9999)
+
+
+def test_workspace_reuse_across_shapes_and_launches():
+    """One workspace serves repeated launches and smaller shapes; tags of earlier launches
+    must never be taken for fresh ones."""
+    ws = capi.new_workspace(2, 2048, 256, "bf16")
+    first = _run_case(2, 2048, 256, "bf16", seed=1, ws=ws)
+    for seed, (B, T, D) in enumerate([(2, 2048, 256), (1, 700, 128), (2, 2048, 256), (2, 65, 64)]):
+        _run_case(B, T, D, "bf16", seed=seed + 1, ws=ws)
+    again = _run_case(2, 2048, 256, "bf16", seed=1, ws=ws)
+    assert torch.equal(first[0], again[0])
+    for a, b in zip(first[1][:3], again[1][:3]):
+        assert torch.equal(a, b)
+    assert capi.workspace_flag(ws) == 0
+
+
+def test_result_does_not_depend_on_how_time_is_tiled():
+    """Chunk invariance: the first T1 rows of a long scan equal a scan of only those rows
+    (a different number of tiles and a different position of every row inside its tile)."""
+    x, xg, ag, lam, _ = make_scan_inputs(1, 1024, 128, seed=11, lo=0.99, hi=0.9999)
+    d = [capi.to_dev(a, "f32") for a in (x, xg, ag)]
+    lam_d = capi.to_dev(lam, "f32")
+    h_long = capi.to_np(capi.scan_fwd(*d, lam_d))
+    for T1 in (1, 50, 64, 100, 513):
+        part = [t[:, :T1].contiguous() for t in d]
+        h_short = capi.to_np(capi.scan_fwd(*part, lam_d))
+        assert max_rel(h_short, h_long[:, :T1]) < 2e-6, T1
+
+
+def test_constant_gates_equal_lfilter_on_gpu():
+    rng = np.random.default_rng(3)
+    B, T, D = 2, 700, 64
+    x = rng.standard_normal((B, T, D))
+    xg = np.broadcast_to(rng.standard_normal((1, 1, D)), (B, T, D)).copy()
+    ag = np.broadcast_to(rng.standard_normal((1, 1, D)), (B, T, D)).copy()
+    lam = rng.uniform(-6.0, 1.0, size=D)
+    d = [capi.to_dev(a, "f32") for a in (x, xg, ag)]
+    xr, xgr, agr = (capi.to_np(t) for t in d)
+    lam_d = capi.to_dev(lam, "f32")
+    lam_r = capi.to_np(lam_d)
+    h = capi.to_np(capi.scan_fwd(*d, lam_d))
+    alpha = np.exp(-8.0 / (1.0 + np.exp(-agr[0, 0])) * np.log1p(np.exp(lam_r)))
+    beta = np.sqrt(1 - alpha**2) / (1.0 + np.exp(-xgr[0, 0])) * xr
+    for c in range(D):
+        ref = scipy.signal.lfilter([1.0], [1.0, -alpha[c]], beta[:, :, c], axis=1)
+        assert max_rel(h[:, :, c], ref) < 1e-4, c
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_gate_extremes(dtype):
+    x, xg, ag, lam, gout = make_scan_inputs(1, 200, 64, seed=21)
+    lam_d = capi.to_dev(lam, "f32")
+    # r -> 0: alpha = 1, beta = 0, h == 0 exactly; gradients stay finite
+    d = [capi.to_dev(a, dtype) for a in (x, xg, np.full_like(ag, -300.0), gout)]
+    h = capi.scan_fwd(d[0], d[1], d[2], lam_d)
+    assert torch.all(h == 0)
+    grads = capi.scan_bwd(d[0], d[1], d[2], lam_d, h, d[3])
+    for g in grads:
+        assert torch.all(torch.isfinite(g.float()))
+    # alpha -> 0: h_t = i_t x_t
+    d2 = [capi.to_dev(a, dtype) for a in (x, xg, np.full_like(ag, 60.0))]
+    big = capi.to_dev(np.full_like(lam, 30.0), "f32")
+    h2 = capi.to_np(capi.scan_fwd(*d2, big))
+    ref = capi.to_np(d2[0]) / (1.0 + np.exp(-capi.to_np(d2[1])))
+    assert max_rel(h2, ref) < TOL[dtype]
+    # huge logits of both signs do not produce NaN
+    wild = np.where(np.random.default_rng(2).random(ag.shape) < 0.5, -1e4, 1e4)
+    d3 = [capi.to_dev(a, dtype) for a in (x, wild, -wild, gout)]
+    h3 = capi.scan_fwd(d3[0], d3[1], d3[2], lam_d)
+    assert torch.all(torch.isfinite(h3.float()))
+    for g in capi.scan_bwd(d3[0], d3[1], d3[2], lam_d, h3, d3[3]):
+        assert torch.all(torch.isfinite(g.float()))
+
+
+def test_clip_branch_of_the_sqrt_derivative():
+    """Lambda = -20 puts every element inside the clip (1 - alpha^2 < 2.5e-7), where the
+    oracle's closed form (derivative = 1000) was pinned on the CPU."""
+    x, xg, ag, _, gout = make_scan_inputs(2, 70, 64, seed=31)
+    lam = np.full(64, -20.0)
+    d = [capi.to_dev(a, "f32") for a in (x, xg, ag, gout)]
+    xr, xgr, agr, gor = (capi.to_np(t) for t in d)
+    lam_d = capi.to_dev(lam, "f32")
+    h = capi.scan_fwd(d[0], d[1], d[2], lam_d)
+    got = capi.scan_bwd(d[0], d[1], d[2], lam_d, h, d[3])
+    want = oracle.rglru_scan_bwd(xr, xgr, agr, lam, capi.to_np(h), gor)
+    for name, a, b in zip(("dx", "dxg", "dag", "dlam"), got, want):
+        assert max_rel(capi.to_np(a), b) < 1e-4, name
+
+
+@pytest.mark.parametrize(
+    "B,T,D,lo,hi",
+    [(8, 4096, 2560, 0.9, 0.999), (2, 32768, 4096, 0.99, 0.9999)],
+    ids=["scan_B8_T4096_D2560", "long_context_B2_T32768_D4096"],
+)
+def test_full_benchmark_shapes_bf16(B, T, D, lo, hi):
+    """Full benchmark sizes.  Channels are independent, so the oracle is run on a strided
+    subset of channels over all of B and T; every channel is covered by two size-independent
+    properties: linearity of h in x, and sum_t(gout*h)-style adjoint identity
+    <gout, h(x)> == <dx, x> (h is linear in x with adjoint dx for fixed gates)."""
+    rng = np.random.default_rng(7)
+    lam = np.log(np.power(rng.uniform(lo, hi, size=D), -1.0 / 8.0) - 1.0)
+    lam_d = capi.to_dev(lam, "f32")
+    g = torch.Generator(device="cuda").manual_seed(7)
+    x, xg, ag, gout = (torch.randn(B, T, D, device="cuda", generator=g).to(torch.bfloat16) for _ in range(4))
+    ws = capi.new_workspace(B, T, D, "bf16")
+    h = capi.scan_fwd(x, xg, ag, lam_d, ws)
+    dx, dxg, dag, dlam = capi.scan_bwd(x, xg, ag, lam_d, h, gout, ws)
+    torch.cuda.synchronize()
+    assert capi.workspace_flag(ws) == 0
+
+    sel = np.arange(0, D, D // 32)[:32]
+    sel_t = torch.from_numpy(sel).cuda()
+    take = lambda t: capi.to_np(t.index_select(2, sel_t))  # noqa: E731
+    xs, xgs, ags, gos = take(x), take(xg), take(ag), take(gout)
+    h_ref = oracle.rglru_scan_fwd(xs, xgs, ags, lam[sel])
+    assert max_rel(take(h), h_ref) < TOL["bf16"]
+    ref = oracle.rglru_scan_bwd(xs, xgs, ags, capi.to_np(lam_d)[sel], take(h), gos)
+    assert max_rel(take(dx), ref[0]) < TOL["bf16"]
+    assert max_rel(take(dxg), ref[1]) < TOL["bf16"]
+    assert max_rel(take(dag), ref[2]) < TOL["bf16"]
+    assert max_rel(capi.to_np(dlam)[sel], ref[3]) < TOL["bf16"]
+
+    # adjoint identity over ALL channels: <gout, h> == <dx, x> up to bf16 rounding of h, dx
+    lhs = (gout.float() * h.float()).sum(dim=(0, 1)).double()
+    rhs = (dx.float() * x.float()).sum(dim=(0, 1)).double()
+    scale = (gout.float() * h.float()).abs().sum(dim=(0, 1)).double()
+    assert float(((lhs - rhs).abs() / scale).max()) < 2e-3
+    # linearity over ALL channels: h(2x) == 2 h(x) exactly in bf16 (power-of-two scaling)
+    h2 = capi.scan_fwd((x.float() * 2).to(torch.bfloat16), xg, ag, lam_d, ws)
+    assert torch.equal(h2.float(), h.float() * 2)

@@ -1,0 +1,176 @@
+"""CPU-side checks: the C-ABI library loads and exports what the header declares, argument
+validation answers without a GPU, and the Python host mirrors upstream's surface.  No
+kernel is launched here."""
+
+import ctypes
+import math
+import os
+import re
+
+import pytest
+import torch
+
+import hawk_pytorch_amd as hk
+from hawk_pytorch_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "hawk_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(hawk_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = _lib.load()
+    names = _declared_symbols()
+    assert len(names) >= 12
+    for name in names:
+        assert hasattr(lib, name), name
+        assert name in _lib.SIGNATURES, f"{name} declared in the header but not bound"
+    assert sorted(_lib.SIGNATURES) == names
+    assert lib.hawk_version() >= 100
+
+
+def test_status_strings_are_distinct():
+    msgs = {_lib.status_string(s) for s in range(7)}
+    assert len(msgs) == 7 and _lib.status_string(0) == "ok"
+    assert "unknown" in _lib.status_string(99)
+
+
+def test_argument_validation_needs_no_gpu():
+    lib = _lib.load()
+    buf = (ctypes.c_char * 4096)()
+    p = (ctypes.addressof(buf) + 15) & ~15
+    args = [p, p, p, p, p]
+    assert lib.hawk_rglru_scan_fwd(None, p, p, p, p, 1, 8, 64, 0, None, 0, None) == _lib.HAWK_ERR_NULL_POINTER
+    assert lib.hawk_rglru_scan_fwd(*args, 1, 8, 64, 7, None, 0, None) == _lib.HAWK_ERR_BAD_DTYPE
+    assert lib.hawk_rglru_scan_fwd(*args, 0, 8, 64, 0, None, 0, None) == _lib.HAWK_ERR_BAD_SHAPE
+    assert lib.hawk_rglru_scan_fwd(*args, 1, -3, 64, 0, None, 0, None) == _lib.HAWK_ERR_BAD_SHAPE
+    assert lib.hawk_rglru_scan_fwd(p + 2, p, p, p, p, 1, 8, 64, 0, None, 0, None) == _lib.HAWK_ERR_ALIGNMENT
+    # T spans several tiles but no workspace was given
+    assert lib.hawk_rglru_scan_fwd(*args, 1, 4096, 64, 0, None, 0, None) == _lib.HAWK_ERR_WORKSPACE
+    assert lib.hawk_rglru_scan_fwd(*args, 1, 4096, 64, 0, p, 256, None) == _lib.HAWK_ERR_WORKSPACE
+    bwd = [p] * 10
+    assert lib.hawk_rglru_scan_bwd(*bwd, 1, 8, 64, 0, None, 0, None) == _lib.HAWK_ERR_WORKSPACE
+    assert lib.hawk_rglru_scan_bwd(*([None] + bwd[1:]), 1, 8, 64, 0, p, 1 << 20, None) == _lib.HAWK_ERR_NULL_POINTER
+    assert lib.hawk_conv1d_fwd(p, p, p, None, p, 1, 8, 64, 9, 0, 0, None) == _lib.HAWK_ERR_BAD_SHAPE
+    assert lib.hawk_conv1d_fwd(p, p, p, None, p, 1, 8, 64, 4, 0, 3, None) == _lib.HAWK_ERR_BAD_DTYPE
+    assert lib.hawk_conv1d_bwd(p, p, p, p, p, p, 1, 8, 64, 4, 0, 0, None, 0, None) == _lib.HAWK_ERR_WORKSPACE
+    assert lib.hawk_conv1d_step(None, p, p, p, p, 1, 64, 4, 0, 0, None) == _lib.HAWK_ERR_NULL_POINTER
+    assert lib.hawk_rglru_step(p, p, p, p, p, p, 0, 64, 0, 0, None) == _lib.HAWK_ERR_BAD_SHAPE
+    assert lib.hawk_scan_workspace_init(None, 1024, None) == _lib.HAWK_ERR_NULL_POINTER
+
+
+def test_workspace_size_queries():
+    lib = _lib.load()
+    assert lib.hawk_scan_workspace_bytes(0, 1, 1, 0) == 0
+    assert lib.hawk_scan_workspace_bytes(1, 1, 1, 5) == 0
+    small = lib.hawk_scan_workspace_bytes(1, 64, 64, 0)
+    big = lib.hawk_scan_workspace_bytes(8, 4096, 2560, 0)
+    assert 256 <= small < big
+    assert big % 256 == 0
+    # a workspace sized for a shape serves every smaller shape
+    assert lib.hawk_scan_workspace_bytes(4, 2048, 2560, 0) <= big
+    assert lib.hawk_scan_workspace_bytes(8, 4096, 1280, 1) <= lib.hawk_scan_workspace_bytes(8, 4096, 2560, 1)
+    assert lib.hawk_conv1d_bwd_workspace_bytes(8, 4096, 2560, 4) > 0
+    assert lib.hawk_conv1d_bwd_workspace_bytes(8, 4096, 2560, 9) == 0
+
+
+def test_no_cpu_fallback():
+    x = torch.randn(1, 8, 64)
+    lam = torch.randn(64)
+    with pytest.raises((NotImplementedError, RuntimeError)):
+        hk.fused_linear_scan(x, x, x, lam)
+    with pytest.raises((NotImplementedError, RuntimeError)):
+        hk.Conv1D(64, 4)(x)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        hk.rglru_step(x[:, 0], x[:, 0], x[:, 0], lam, torch.zeros(1, 64))
+
+
+def test_scan_wrapper_asserts_like_upstream():
+    x = torch.randn(1, 8, 60)
+    with pytest.raises(AssertionError, match="multiple of 64"):
+        hk.sequential_scan_forward(x, x, x, torch.randn(60))
+    y = torch.randn(1, 8, 64)
+    with pytest.raises(AssertionError):
+        hk.sequential_scan_forward(y, y[:, :4], y, torch.randn(64))
+
+
+def test_rnn_cache_matches_upstream_layout_at_batch_one():
+    c = hk.RNNCache(32, torch.device("cpu"), 4)
+    assert c.recc_state.shape == (1, 1, 32) and c.conv_state.shape == (1, 3, 32)
+    assert c.recc_state.dtype == torch.bfloat16 and c.conv_state.dtype == torch.bfloat16
+    assert torch.isnan(c.recc_state.float()).all() and torch.isnan(c.conv_state.float()).all()
+    assert c.current_cache_size == 0 and c.conv_cache_size == 3
+    c.conv_state.zero_()
+    rows = [torch.full((1, 1, 32), float(k + 1)) for k in range(4)]
+    for r in rows:
+        expect = torch.roll(c.conv_state, shifts=-1, dims=1)
+        expect[:, -1, :] = r
+        c.update_conv_cache(r)
+        assert torch.equal(c.conv_state, expect)
+    assert c.conv_state[0, :, 0].tolist() == [2.0, 3.0, 4.0]
+    c.update_cache(rows[2])
+    assert c.current_cache_size == 1 and float(c.recc_state[0, 0, 0]) == 3.0
+    with pytest.raises(AssertionError):
+        c.update_cache(torch.zeros(2, 1, 32))
+    short = torch.arange(2 * 32, dtype=torch.float32).reshape(1, 2, 32)
+    c.seed_conv_state(short)
+    assert torch.equal(c.conv_state[:, 0].float(), torch.zeros(1, 32))
+    assert torch.equal(c.conv_state[:, 1:].float(), short.bfloat16().float())
+    assert "RNNCache" in repr(c)
+
+
+def test_lambda_init_distribution():
+    t = torch.empty(200000)
+    hk.rnn_param_init(t, min_rad=0.9, max_rad=0.999)
+    a2 = torch.exp(-2.0 * torch.nn.functional.softplus(t.double()))
+    assert a2.min() >= 0.81 - 1e-6 and a2.max() <= 0.998001 + 1e-6
+    assert abs(float(a2.mean()) - (0.81 + 0.998001) / 2) < 1e-3
+
+
+def test_model_surface_and_parameter_count_of_the_readme_config():
+    cfg = hk.HawkConfig(vocab_size=32000, hidden_size=512, intermediate_size=1024, recurrent_size=512,
+                        num_hidden_layers=8, num_blocks=16, post_norm=False)
+    assert cfg.conv_width == 4
+    model = hk.HawkModel(cfg, use_cache=False)
+    assert sum(p.numel() for p in model.parameters()) == 51_945_984
+    sd = model.state_dict()
+    expect = {
+        "embed_tokens.weight": (32000, 512), "lm_head.weight": (32000, 512), "norm.weight": (512,),
+        "layers.0.input_norm.weight": (512,), "layers.0.post_recurrent_norm.weight": (512,),
+        "layers.0.recc.input_xy.weight": (1024, 512), "layers.0.recc.resid_proj.weight": (512, 512),
+        "layers.0.recc.rg_lru_input_gate.w": (16, 32, 32), "layers.0.recc.rg_lru_input_gate.b": (16, 32),
+        "layers.0.recc.rg_lru_a_gate.w": (16, 32, 32), "layers.0.recc.rg_lru_a_gate.b": (16, 32),
+        "layers.0.recc.rg_lru_a_param": (512,), "layers.0.recc.conv1d.w": (4, 512),
+        "layers.0.recc.conv1d.b": (512,), "layers.7.mlp.gate_up_proj.weight": (2048, 512),
+        "layers.7.mlp.resid_proj.weight": (512, 1024),
+    }
+    for k, shape in expect.items():
+        assert tuple(sd[k].shape) == shape, k
+    assert len(sd) == 3 + 8 * 13
+    assert sd["layers.3.recc.rg_lru_a_param"].dtype == torch.float32
+    assert float(sd["lm_head.weight"].abs().max()) == 0.0
+    assert float(sd["layers.0.recc.resid_proj.weight"].abs().max()) == 0.0
+    with pytest.raises(NotImplementedError):
+        hk.HawkConfig(10, 8, 8, 1, 8, 1, post_norm=True)
+    assert len(model.new_cache(batch_size=3)) == 8
+
+
+def test_custom_ops_have_shape_rules_for_tracing():
+    from torch._subclasses.fake_tensor import FakeTensorMode
+
+    with FakeTensorMode():
+        x = torch.empty(2, 16, 64, dtype=torch.bfloat16, device="cuda")
+        lam = torch.empty(64, device="cuda")
+        h = torch.ops.hawk_amd.rglru_scan_fwd(x, x, x, lam)
+        assert h.shape == x.shape and h.dtype == torch.bfloat16
+        dx, dxg, dag, dlam = torch.ops.hawk_amd.rglru_scan_bwd(x, x, x, lam, h, h)
+        assert dx.shape == x.shape and dlam.shape == (64,) and dlam.dtype == torch.float32
+        w = torch.empty(4, 64, device="cuda")
+        y = torch.ops.hawk_amd.conv1d_fwd(x, w, lam, None, True)
+        assert y.dtype == torch.float32 and y.shape == x.shape
+        gx, gw, gb = torch.ops.hawk_amd.conv1d_bwd(y, x, w)
+        assert gx.dtype == torch.bfloat16 and gw.shape == (4, 64) and gb.shape == (64,)
