@@ -98,6 +98,52 @@ __device__ __forceinline__ void store_raw(ET* p, typename Raw<ET, V>::type r) {
 }
 
 // ---------------------------------------------------------------------------------------
+// Buffer addressing.  A wave describes the slab of a tensor it works on with a buffer
+// resource in scalar registers (base pointer + byte size); every access is then
+// "resource + per-lane byte offset (one VGPR shared by all accesses) + scalar row offset",
+// which costs no vector address arithmetic.  The hardware range check returns zero for
+// loads and drops stores at or beyond the slab size, which is how ragged last tiles are
+// handled.
+// ---------------------------------------------------------------------------------------
+typedef __amdgpu_buffer_rsrc_t rsrc_t;
+
+__device__ __forceinline__ rsrc_t make_rsrc(const void* base, uint32_t bytes) {
+    // raw buffer: stride 0, 32-bit untyped data format
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);
+}
+
+constexpr int kAuxDefault = 0;
+constexpr int kAuxStream = 2;  // "nt": written once, not re-read by this kernel
+
+template <typename R>
+__device__ __forceinline__ R buffer_load(rsrc_t r, uint32_t lane_bytes, uint32_t row_bytes) {
+    if constexpr (sizeof(R) == 2) {
+        return __builtin_bit_cast(R, __builtin_amdgcn_raw_buffer_load_b16(r, lane_bytes, row_bytes, kAuxDefault));
+    } else if constexpr (sizeof(R) == 4) {
+        return __builtin_bit_cast(R, __builtin_amdgcn_raw_buffer_load_b32(r, lane_bytes, row_bytes, kAuxDefault));
+    } else if constexpr (sizeof(R) == 8) {
+        return __builtin_bit_cast(R, __builtin_amdgcn_raw_buffer_load_b64(r, lane_bytes, row_bytes, kAuxDefault));
+    } else {
+        static_assert(sizeof(R) == 16, "unsupported access width");
+        return __builtin_bit_cast(R, __builtin_amdgcn_raw_buffer_load_b128(r, lane_bytes, row_bytes, kAuxDefault));
+    }
+}
+
+template <typename R>
+__device__ __forceinline__ void buffer_store(R v, rsrc_t r, uint32_t lane_bytes, uint32_t row_bytes) {
+    if constexpr (sizeof(R) == 2) {
+        __builtin_amdgcn_raw_buffer_store_b16(__builtin_bit_cast(unsigned short, v), r, lane_bytes, row_bytes, kAuxStream);
+    } else if constexpr (sizeof(R) == 4) {
+        __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned int, v), r, lane_bytes, row_bytes, kAuxStream);
+    } else if constexpr (sizeof(R) == 8) {
+        __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(u32x2, v), r, lane_bytes, row_bytes, kAuxStream);
+    } else {
+        static_assert(sizeof(R) == 16, "unsupported access width");
+        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), r, lane_bytes, row_bytes, kAuxStream);
+    }
+}
+
+// ---------------------------------------------------------------------------------------
 // Transcendentals: one hardware instruction each (v_exp_f32, v_rcp_f32, v_sqrt_f32,
 // v_rsq_f32; about 1 ulp), which is what keeps the scan bandwidth-bound.
 // ---------------------------------------------------------------------------------------

@@ -28,7 +28,8 @@
 // an earlier launch can never be mistaken for a fresh one.  Tiles take their position in
 // the chain from an atomic ticket, so a tile only ever waits for tiles that have already
 // started; the wait is also bounded, and a tile that exhausts it raises the workspace's
-// error word and finishes (with a wrong carry) instead of hanging.
+// error word and finishes (with a wrong carry) instead of hanging.  Results do not depend
+// on timing: the combination order is a function of the tile position only.
 #include "hawk_scan.h"
 
 #include "hawk_device.h"
@@ -39,11 +40,20 @@ namespace {
 
 constexpr uint32_t kSpinLimit = 1u << 22;
 
-enum CtrlWord { kTicket = 0, kDone = 1, kEpoch = 2, kError = 3 };
+// Occupancy the register allocator must leave room for (waves per SIMD).
+#ifndef HAWK_FWD_WAVES_PER_SIMD
+#define HAWK_FWD_WAVES_PER_SIMD 4
+#endif
+#ifndef HAWK_BWD_WAVES_PER_SIMD
+#define HAWK_BWD_WAVES_PER_SIMD 4
+#endif
 
+// Control block at the start of the workspace:
+//   bytes 0-7   one 64-bit word: launch epoch (high half) and ticket counter (low half)
+//   bytes 8-11  error flag (a tile gave up waiting for a carry)
 struct ScanWsPtrs {
-    uint32_t* ctrl;
-    unsigned long long* incl;  // [nseg][B][D] inclusive state at the end of a tile
+    unsigned long long* ctrl;
+    unsigned long long* incl;  // [nseg][B][D] inclusive state at the end of a checkpoint tile
     unsigned long long* agg_p; // [nseg][B][D] tile aggregate: product of alpha
     unsigned long long* agg_h; // [nseg][B][D] tile aggregate: state from zero
     float* dlam_part;          // [nseg][B][D] per-tile partial sums for dLambda
@@ -59,132 +69,173 @@ __device__ __forceinline__ bool try_read(const unsigned long long* p, uint32_t t
     return (uint32_t)(w >> 32) == tag;
 }
 
-// Every kCheckpointEvery-th chain position is a checkpoint: it publishes the inclusive
-// state at its end; every other position publishes only its own aggregate.  A tile folds
-// the aggregates of its predecessors back to the nearest checkpoint and finishes with that
-// checkpoint's inclusive state.  The order of the floating-point operations is therefore
-// fixed by the position alone, never by timing, so results are bitwise reproducible, and
-// the serial dependency runs over checkpoints only (nseg / kCheckpointEvery hops).
-constexpr int kCheckpointEvery = 8;
+// Every kLookback-th chain position is a checkpoint: it publishes the inclusive state at
+// its end; every other position publishes only its own aggregate.  A tile reads the
+// aggregates of its predecessors back to the nearest checkpoint, plus that checkpoint's
+// inclusive state, all in parallel (one predecessor per wave), and folds them oldest
+// first.  The order of the floating-point operations is fixed by the position alone,
+// never by timing, so results are bitwise reproducible, and the serial dependency runs
+// over checkpoints only (nseg / kLookback hops of one memory round trip each).
+constexpr int kLookback = 8;
 
-__device__ __forceinline__ bool is_checkpoint(int pos) { return (pos % kCheckpointEvery) == 0; }
+__device__ __forceinline__ bool is_checkpoint(int pos) { return (pos % kLookback) == 0; }
+__device__ __forceinline__ int checkpoint_before(int pos) { return ((pos - 1) / kLookback) * kLookback; }
 
-// Return the state carried into chain position `pos` (pos >= 1) for one channel.  `stride`
-// is the distance in words between consecutive chain positions of the same channel.
-__device__ __forceinline__ float look_back(const ScanWsPtrs& ws, size_t idx_pos0, size_t stride,
-                                           int pos, uint32_t tag) {
-    float acc_p = 1.0f, acc_h = 0.0f;
-    int j = pos - 1;
-    uint32_t spins = 0;
-    while (true) {
+// One 64-bit atomic hands out the tile's position in the chain (ticket) together with the
+// launch tag, so a tile only ever waits for tiles that have already started.  The tile
+// that takes the last ticket re-arms the word for the next launch on this workspace
+// (epoch + 1, ticket 0) with a second atomic; nothing else ever writes it.
+__device__ __forceinline__ void take_ticket(unsigned long long* ctrl, uint32_t total, uint32_t* s_ticket,
+                                            uint32_t& ticket, uint32_t& tag) {
+    if (threadIdx.x == 0) {
+        const unsigned long long v =
+            __hip_atomic_fetch_add(ctrl, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const uint32_t t = (uint32_t)v;
+        if (t == total - 1u) {
+            __hip_atomic_fetch_add(ctrl, (1ull << 32) - (unsigned long long)total, __ATOMIC_RELAXED,
+                                   __HIP_MEMORY_SCOPE_AGENT);
+        }
+        s_ticket[0] = t;
+        s_ticket[1] = (uint32_t)(v >> 32) + 1u;
+    }
+    __syncthreads();
+    ticket = __builtin_amdgcn_readfirstlane(s_ticket[0]);
+    tag = __builtin_amdgcn_readfirstlane(s_ticket[1]);
+}
+
+// Carry into chain position `pos` for the V channels of this lane.
+//   tot_p/tot_h  aggregate of this whole tile (every wave holds it)
+//   s_prev       LDS [kLookback][CT] staging of the predecessors' words
+// Wave 0 publishes the tile's own word; wave k (k < number of predecessors) fetches
+// predecessor pos-1-k; after one barrier every wave folds the staged words.
+template <int V, int NW>
+__device__ __forceinline__ void exchange_carry(const ScanWsPtrs& ws, int pos, int nseg, size_t idx_pos0,
+                                               size_t stride, uint32_t tag, int w, int lane,
+                                               const float (&tot_p)[V], const float (&tot_h)[V],
+                                               float2 (*s_prev)[kWave * V], float (&cin)[V]) {
+    static_assert(kLookback % NW == 0 || NW % kLookback == 0, "waves must tile the look-back window");
+    const bool publishes = pos + 1 < nseg;
+    const size_t idx_self = idx_pos0 + (size_t)pos * stride;
+    if (w == 0 && publishes && !is_checkpoint(pos)) {
+#pragma unroll
+        for (int v = 0; v < V; ++v) {
+            publish(ws.agg_p + idx_self + v, tag, tot_p[v]);
+            publish(ws.agg_h + idx_self + v, tag, tot_h[v]);
+        }
+        asm volatile("" ::: "memory");
+    }
+    const int npred = (pos > 0) ? pos - checkpoint_before(pos) : 0;
+    for (int k = w; k < npred; k += NW) {
+        const int j = pos - 1 - k;
         const size_t idx = idx_pos0 + (size_t)j * stride;
-        if (is_checkpoint(j)) {
-            float vi;
-            if (try_read(ws.incl + idx, tag, vi)) return fmaf(acc_p, vi, acc_h);
-        } else {
-            float vp, vh;
-            const bool okp = try_read(ws.agg_p + idx, tag, vp);
-            const bool okh = try_read(ws.agg_h + idx, tag, vh);
-            if (okp && okh) {
-                acc_h = fmaf(acc_p, vh, acc_h);
-                acc_p *= vp;
-                --j;
-                continue;
+        const bool cp = (k == npred - 1);
+        float vp[V], vh[V];
+        bool ok = false;
+        uint32_t spins = 0;
+        while (!ok) {
+            ok = true;
+#pragma unroll
+            for (int v = 0; v < V; ++v) {
+                if (cp) {
+                    vp[v] = 0.0f;
+                    ok &= try_read(ws.incl + idx + v, tag, vh[v]);
+                } else {
+                    ok &= try_read(ws.agg_p + idx + v, tag, vp[v]);
+                    ok &= try_read(ws.agg_h + idx + v, tag, vh[v]);
+                }
+            }
+            if (!ok) {
+                if (++spins > kSpinLimit) {
+                    __hip_atomic_store(reinterpret_cast<uint32_t*>(ws.ctrl) + 2, 1u, __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+                    for (int v = 0; v < V; ++v) { vp[v] = 0.0f; vh[v] = 0.0f; }
+                    break;
+                }
+                __builtin_amdgcn_s_sleep(2);
             }
         }
-        if (++spins > kSpinLimit) {
-            __hip_atomic_store(ws.ctrl + kError, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            return acc_h;
+#pragma unroll
+        for (int v = 0; v < V; ++v) s_prev[k][lane * V + v] = make_float2(vp[v], vh[v]);
+    }
+    __syncthreads();
+#pragma unroll
+    for (int v = 0; v < V; ++v) cin[v] = 0.0f;
+    for (int k = npred - 1; k >= 0; --k) {
+#pragma unroll
+        for (int v = 0; v < V; ++v) {
+            const float2 a = s_prev[k][lane * V + v];
+            cin[v] = fmaf(a.x, cin[v], a.y);
         }
-        __builtin_amdgcn_s_sleep(4);
+    }
+    if (w == 0 && publishes && is_checkpoint(pos)) {
+#pragma unroll
+        for (int v = 0; v < V; ++v) publish(ws.incl + idx_self + v, tag, fmaf(tot_p[v], cin[v], tot_h[v]));
     }
 }
 
-// Take a ticket (chain-ordered tile index) and the launch tag.  One barrier.
-__device__ __forceinline__ void take_ticket(uint32_t* ctrl, uint32_t* s_ticket, uint32_t& ticket,
-                                            uint32_t& tag) {
-    if (threadIdx.x == 0) {
-        s_ticket[0] = __hip_atomic_fetch_add(ctrl + kTicket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        s_ticket[1] = __hip_atomic_load(ctrl + kEpoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1u;
-    }
-    __syncthreads();
-    ticket = s_ticket[0];
-    tag = s_ticket[1];
-}
-
-// Last tile out re-arms the control block for the next launch on the same workspace.
-__device__ __forceinline__ void retire(uint32_t* ctrl, uint32_t total, uint32_t tag) {
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        uint32_t d = __hip_atomic_fetch_add(ctrl + kDone, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        if (d == total - 1u) {
-            __hip_atomic_store(ctrl + kTicket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            __hip_atomic_store(ctrl + kDone, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            __hip_atomic_store(ctrl + kEpoch, tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+// Slice aggregates of the NW waves -> prefix for wave `w` and tile total, in chain order
+// (forward: wave 0 first; backward: wave NW-1 first).
+template <int V, int NW, bool REVERSE>
+__device__ __forceinline__ void combine_slices(float2 (*s_agg)[kWave * V], int w, int lane, float (&pre_p)[V],
+                                               float (&pre_h)[V], float (&tot_p)[V], float (&tot_h)[V]) {
+#pragma unroll
+    for (int v = 0; v < V; ++v) { tot_p[v] = 1.0f; tot_h[v] = 0.0f; pre_p[v] = 1.0f; pre_h[v] = 0.0f; }
+#pragma unroll
+    for (int q = 0; q < NW; ++q) {
+        const int ww = REVERSE ? NW - 1 - q : q;
+#pragma unroll
+        for (int v = 0; v < V; ++v) {
+            if (ww == w) { pre_p[v] = tot_p[v]; pre_h[v] = tot_h[v]; }
+            const float2 a = s_agg[ww][lane * V + v];
+            tot_h[v] = fmaf(a.x, tot_h[v], a.y);
+            tot_p[v] *= a.x;
         }
     }
 }
 
 // ---------------------------------------------------------------------------------------
-// Forward
+// Forward tile.  FULL: every row of the tile is inside [0, T).
 // ---------------------------------------------------------------------------------------
-template <typename ET, int V, int TC, int NW, bool PRECISE>
-__global__ __launch_bounds__(NW * kWave) void rglru_scan_fwd_kernel(
-    const ET* __restrict__ x, const ET* __restrict__ xg, const ET* __restrict__ ag,
-    const float* __restrict__ lam, ET* __restrict__ h, int B, int T, int D, int nseg, int nct,
-    ScanWsPtrs ws) {
+template <typename ET, int V, int TC, int NW, bool PRECISE, bool FULL>
+__device__ __forceinline__ void fwd_tile(const ET* __restrict__ x, const ET* __restrict__ xg,
+                                         const ET* __restrict__ ag, const float* __restrict__ lam,
+                                         ET* __restrict__ h, int B, int T, int D, int nseg, int seg, int b, int ct,
+                                         uint32_t tag, const ScanWsPtrs& ws, float2 (*s_agg)[kWave * V],
+                                         float2 (*s_prev)[kWave * V]) {
     typedef typename Raw<ET, V>::type raw_t;
     constexpr int CT = kWave * V;
     constexpr int TS = NW * TC;
 
-    __shared__ float2 s_agg[NW][CT];
-    __shared__ float s_cin[CT];
-    __shared__ uint32_t s_ticket[2];
-
-    uint32_t ticket = blockIdx.x, tag = 0;
-    const uint32_t total = (uint32_t)nseg * (uint32_t)B * (uint32_t)nct;
-    if (nseg > 1) take_ticket(ws.ctrl, s_ticket, ticket, tag);
-
-    const int per_seg = B * nct;
-    const int seg = ticket / per_seg;
-    const int rem = ticket - seg * per_seg;
-    const int b = rem / nct;
-    const int ct = rem - b * nct;
-
     const int lane = threadIdx.x & (kWave - 1);
-    const int w = threadIdx.x / kWave;
-    const int c_want = ct * CT + lane * V;
-    const bool lane_on = c_want < D;
-    const int c0 = lane_on ? c_want : D - V;  // idle lanes shadow the last valid channels
+    const int w = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    const int c_tile = ct * CT;
+    const bool lane_on = c_tile + lane * V < D;
+    const unsigned lane_off = lane_on ? lane * V : D - V - c_tile;  // idle lanes shadow the last valid channels
     const int t0 = seg * TS + w * TC;
+    const size_t tile_off = ((size_t)b * T + t0) * D + c_tile;  // wave-uniform
+    const int rows_in = FULL ? TC : __builtin_amdgcn_readfirstlane(min(max(T - t0, 0), TC));  // rows inside [0, T)
+    const uint32_t row_bytes = (uint32_t)D * sizeof(ET);
+    const uint32_t slab = (uint32_t)rows_in * row_bytes;
+    const uint32_t lane_bytes = lane_off * sizeof(ET);
+    const rsrc_t bx = make_rsrc(x + tile_off, slab), bxg = make_rsrc(xg + tile_off, slab),
+                 bag = make_rsrc(ag + tile_off, slab), bh = make_rsrc(h + tile_off, slab);
+    // idle lanes store at an offset beyond any slab, which the range check drops
+    const uint32_t store_bytes = lane_on ? lane_bytes : 0x80000000u;
 
-    const size_t base = ((size_t)b * T + t0) * D + c0;
     raw_t rx[TC], rxg[TC], rag[TC];
-    const bool full = (t0 + TC <= T);
-    if (full) {
 #pragma unroll
-        for (int j = 0; j < TC; ++j) {
-            const size_t o = base + (size_t)j * D;
-            rx[j] = load_raw<ET, V>(x + o);
-            rxg[j] = load_raw<ET, V>(xg + o);
-            rag[j] = load_raw<ET, V>(ag + o);
-        }
-    } else {
-#pragma unroll
-        for (int j = 0; j < TC; ++j) {
-            const size_t o = base + (size_t)j * D;
-            const bool ok = t0 + j < T;
-            rx[j] = ok ? load_raw<ET, V>(x + o) : raw_zero<raw_t>();
-            rxg[j] = ok ? load_raw<ET, V>(xg + o) : raw_zero<raw_t>();
-            rag[j] = ok ? load_raw<ET, V>(ag + o) : raw_zero<raw_t>();
-        }
+    for (int j = 0; j < TC; ++j) {
+        rx[j] = buffer_load<raw_t>(bx, lane_bytes, j * row_bytes);
+        rxg[j] = buffer_load<raw_t>(bxg, lane_bytes, j * row_bytes);
+        rag[j] = buffer_load<raw_t>(bag, lane_bytes, j * row_bytes);
     }
 
     // Per-channel constants: log2(alpha) = c2 * r, 2 ln(alpha) = cn * r.
     float c2[V], cn[V];
 #pragma unroll
     for (int v = 0; v < V; ++v) {
-        const float s = softplus_precise(lam[c0 + v]);
+        const float s = softplus_precise(lam[c_tile + lane_off + v]);
         c2[v] = -8.0f * kLog2e * s;
         cn[v] = -16.0f * s;
     }
@@ -200,7 +251,7 @@ __global__ __launch_bounds__(NW * kWave) void rglru_scan_fwd_kernel(
         unpack(rx[j], fx);
         unpack(rxg[j], fxg);
         unpack(rag[j], fag);
-        const bool ok = full || (t0 + j < T);
+        const bool ok = FULL || (t0 + j < T);  // wave-uniform
 #pragma unroll
         for (int v = 0; v < V; ++v) {
             const float i = sigmoid_fast(fxg[v]);
@@ -214,79 +265,63 @@ __global__ __launch_bounds__(NW * kWave) void rglru_scan_fwd_kernel(
             pj[j][v] = p_run[v];
             hj[j][v] = h_run[v];
         }
+        __builtin_amdgcn_sched_barrier(0);  // one row's temporaries live at a time
     }
 
     // 2. combine the NW time slices of this tile
 #pragma unroll
     for (int v = 0; v < V; ++v) s_agg[w][lane * V + v] = make_float2(p_run[v], h_run[v]);
     __syncthreads();
-    float p_pre[V], h_pre[V], p_tot[V], h_tot[V];
-#pragma unroll
-    for (int v = 0; v < V; ++v) { p_tot[v] = 1.0f; h_tot[v] = 0.0f; p_pre[v] = 1.0f; h_pre[v] = 0.0f; }
-#pragma unroll
-    for (int ww = 0; ww < NW; ++ww) {
-#pragma unroll
-        for (int v = 0; v < V; ++v) {
-            if (ww == w) { p_pre[v] = p_tot[v]; h_pre[v] = h_tot[v]; }
-            const float2 a = s_agg[ww][lane * V + v];
-            h_tot[v] = fmaf(a.x, h_tot[v], a.y);
-            p_tot[v] *= a.x;
-        }
-    }
+    float pre_p[V], pre_h[V], tot_p[V], tot_h[V];
+    combine_slices<V, NW, false>(s_agg, w, lane, pre_p, pre_h, tot_p, tot_h);
 
     // 3. carry across tiles
     float cin[V];
 #pragma unroll
     for (int v = 0; v < V; ++v) cin[v] = 0.0f;
     if (nseg > 1) {
-        if (w == 0) {
-            const size_t stride = (size_t)B * D;
-            const size_t idx0 = (size_t)b * D + c0;  // chain position 0 of this channel
-            const size_t idx = idx0 + (size_t)seg * stride;
-            const bool publishes = seg + 1 < nseg;
-            if (publishes && !is_checkpoint(seg)) {
-#pragma unroll
-                for (int v = 0; v < V; ++v) {
-                    publish(ws.agg_p + idx + v, tag, p_tot[v]);
-                    publish(ws.agg_h + idx + v, tag, h_tot[v]);
-                }
-                asm volatile("" ::: "memory");
-            }
-            if (seg > 0) {
-#pragma unroll
-                for (int v = 0; v < V; ++v) cin[v] = look_back(ws, idx0 + v, stride, seg, tag);
-            }
-            if (publishes && is_checkpoint(seg)) {
-#pragma unroll
-                for (int v = 0; v < V; ++v) publish(ws.incl + idx + v, tag, fmaf(p_tot[v], cin[v], h_tot[v]));
-            }
-#pragma unroll
-            for (int v = 0; v < V; ++v) s_cin[lane * V + v] = cin[v];
-        }
-        __syncthreads();
-#pragma unroll
-        for (int v = 0; v < V; ++v) cin[v] = s_cin[lane * V + v];
+        exchange_carry<V, NW>(ws, seg, nseg, (size_t)b * D + c_tile + lane_off, (size_t)B * D, tag, w, lane,
+                              tot_p, tot_h, s_prev, cin);
     }
 
     // 4. apply the carry and store
     float cw[V];
 #pragma unroll
-    for (int v = 0; v < V; ++v) cw[v] = fmaf(p_pre[v], cin[v], h_pre[v]);
-    if (lane_on) {
+    for (int v = 0; v < V; ++v) cw[v] = fmaf(pre_p[v], cin[v], pre_h[v]);
 #pragma unroll
-        for (int j = 0; j < TC; ++j) {
-            if (full || (t0 + j < T)) {
-                float out[V];
+    for (int j = 0; j < TC; ++j) {
+        float out[V];
 #pragma unroll
-                for (int v = 0; v < V; ++v) out[v] = fmaf(pj[j][v], cw[v], hj[j][v]);
-                raw_t r;
-                pack(out, r);
-                store_raw<ET, V>(h + base + (size_t)j * D, r);
-            }
-        }
+        for (int v = 0; v < V; ++v) out[v] = fmaf(pj[j][v], cw[v], hj[j][v]);
+        raw_t r;
+        pack(out, r);
+        buffer_store<raw_t>(r, bh, store_bytes, j * row_bytes);  // rows past T and idle lanes are dropped
     }
+}
 
-    if (nseg > 1) retire(ws.ctrl, total, tag);
+template <typename ET, int V, int TC, int NW, bool PRECISE>
+__global__ __launch_bounds__(NW * kWave, HAWK_FWD_WAVES_PER_SIMD) void rglru_scan_fwd_kernel(
+    const ET* __restrict__ x, const ET* __restrict__ xg, const ET* __restrict__ ag,
+    const float* __restrict__ lam, ET* __restrict__ h, int B, int T, int D, int nseg, int nct,
+    ScanWsPtrs ws) {
+    constexpr int CT = kWave * V;
+    constexpr int TS = NW * TC;
+    __shared__ float2 s_agg[NW][CT];
+    __shared__ float2 s_prev[kLookback][CT];
+    __shared__ uint32_t s_ticket[2];
+
+    uint32_t ticket = blockIdx.x, tag = 0;
+    if (nseg > 1) take_ticket(ws.ctrl, (uint32_t)nseg * (uint32_t)B * (uint32_t)nct, s_ticket, ticket, tag);
+
+    const int per_seg = B * nct;
+    const int seg = ticket / per_seg;
+    const int rem = ticket - seg * per_seg;
+    const int b = rem / nct;
+    const int ct = rem - b * nct;
+    if (seg * TS + TS <= T)
+        fwd_tile<ET, V, TC, NW, PRECISE, true>(x, xg, ag, lam, h, B, T, D, nseg, seg, b, ct, tag, ws, s_agg, s_prev);
+    else
+        fwd_tile<ET, V, TC, NW, PRECISE, false>(x, xg, ag, lam, h, B, T, D, nseg, seg, b, ct, tag, ws, s_agg, s_prev);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -295,70 +330,57 @@ __global__ __launch_bounds__(NW * kWave) void rglru_scan_fwd_kernel(
 //   dx = g K1, dx_rg_lru = g K2, da_rg_lru = g K3, dLambda += g K4 (scaled per channel later)
 //   K1 = m i;  K2 = m x i (1-i);  K4 = (h_{t-1} alpha - i x alpha^2 2 csg(1-alpha^2)) r;
 //   K3 = K4 (1-r) (-8 softplus(Lambda)).
+// FULL: every row of the tile is inside [1, T) (row 0 has no h_{t-1}).
 // ---------------------------------------------------------------------------------------
-template <typename ET, int V, int TC, int NW, bool PRECISE>
-__global__ __launch_bounds__(NW * kWave) void rglru_scan_bwd_kernel(
-    const ET* __restrict__ x, const ET* __restrict__ xg, const ET* __restrict__ ag,
-    const float* __restrict__ lam, const ET* __restrict__ hs, const ET* __restrict__ gout,
-    ET* __restrict__ dx, ET* __restrict__ dxg, ET* __restrict__ dag, int B, int T, int D, int nseg,
-    int nct, ScanWsPtrs ws) {
+template <typename ET, int V, int TC, int NW, bool PRECISE, bool FULL>
+__device__ __forceinline__ void bwd_tile(const ET* __restrict__ x, const ET* __restrict__ xg,
+                                         const ET* __restrict__ ag, const float* __restrict__ lam,
+                                         const ET* __restrict__ hs, const ET* __restrict__ gout,
+                                         ET* __restrict__ dx, ET* __restrict__ dxg, ET* __restrict__ dag, int B,
+                                         int T, int D, int nseg, int seg, int pos, int b, int ct, uint32_t tag,
+                                         const ScanWsPtrs& ws, float2 (*s_agg)[kWave * V],
+                                         float2 (*s_prev)[kWave * V], float (*s_dl)[kWave * V]) {
     typedef typename Raw<ET, V>::type raw_t;
     constexpr int CT = kWave * V;
     constexpr int TS = NW * TC;
 
-    __shared__ float2 s_agg[NW][CT];
-    __shared__ float s_cin[CT];
-    __shared__ float s_dl[NW][CT];
-    __shared__ uint32_t s_ticket[2];
-
-    uint32_t ticket = blockIdx.x, tag = 0;
-    const uint32_t total = (uint32_t)nseg * (uint32_t)B * (uint32_t)nct;
-    if (nseg > 1) take_ticket(ws.ctrl, s_ticket, ticket, tag);
-
-    const int per_seg = B * nct;
-    const int pos = ticket / per_seg;  // chain position: 0 is the LAST time tile
-    const int seg = nseg - 1 - pos;
-    const int rem = ticket - pos * per_seg;
-    const int b = rem / nct;
-    const int ct = rem - b * nct;
-
     const int lane = threadIdx.x & (kWave - 1);
-    const int w = threadIdx.x / kWave;
-    const int c_want = ct * CT + lane * V;
-    const bool lane_on = c_want < D;
-    const int c0 = lane_on ? c_want : D - V;
+    const int w = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    const int c_tile = ct * CT;
+    const bool lane_on = c_tile + lane * V < D;
+    const unsigned lane_off = lane_on ? lane * V : D - V - c_tile;
     const int t0 = seg * TS + w * TC;
+    const size_t tile_off = ((size_t)b * T + t0) * D + c_tile;
+    const int rows_in = FULL ? TC : __builtin_amdgcn_readfirstlane(min(max(T - t0, 0), TC));
+    const uint32_t row_bytes = (uint32_t)D * sizeof(ET);
+    const uint32_t slab = (uint32_t)rows_in * row_bytes;
+    const uint32_t lane_bytes = lane_off * sizeof(ET);
+    const rsrc_t bx = make_rsrc(x + tile_off, slab), bxg = make_rsrc(xg + tile_off, slab),
+                 bag = make_rsrc(ag + tile_off, slab), bgo = make_rsrc(gout + tile_off, slab),
+                 bhs = make_rsrc(hs + tile_off, slab);
+    // h_{t-1} of the slice's first row lives one row before the slab; absent at t = 0
+    const bool has_prev = FULL || (t0 > 0 && rows_in > 0);
+    const rsrc_t bhm1 = make_rsrc(has_prev ? hs + tile_off - D : hs, has_prev ? row_bytes : 0u);
+    const rsrc_t bdx = make_rsrc(dx + tile_off, slab), bdxg = make_rsrc(dxg + tile_off, slab),
+                 bdag = make_rsrc(dag + tile_off, slab);
+    // idle lanes store at an offset beyond any slab, which the range check drops
+    const uint32_t store_bytes = lane_on ? lane_bytes : 0x80000000u;
 
-    const size_t base = ((size_t)b * T + t0) * D + c0;
     raw_t rx[TC], rxg[TC], rag[TC], rgo[TC], rhp[TC];
-    const bool full = (t0 + TC <= T) && (t0 > 0);
-    if (full) {
 #pragma unroll
-        for (int j = 0; j < TC; ++j) {
-            const size_t o = base + (size_t)j * D;
-            rx[j] = load_raw<ET, V>(x + o);
-            rxg[j] = load_raw<ET, V>(xg + o);
-            rag[j] = load_raw<ET, V>(ag + o);
-            rgo[j] = load_raw<ET, V>(gout + o);
-            rhp[j] = load_raw<ET, V>(hs + o - D);
-        }
-    } else {
-#pragma unroll
-        for (int j = 0; j < TC; ++j) {
-            const size_t o = base + (size_t)j * D;
-            const bool ok = t0 + j < T;
-            rx[j] = ok ? load_raw<ET, V>(x + o) : raw_zero<raw_t>();
-            rxg[j] = ok ? load_raw<ET, V>(xg + o) : raw_zero<raw_t>();
-            rag[j] = ok ? load_raw<ET, V>(ag + o) : raw_zero<raw_t>();
-            rgo[j] = ok ? load_raw<ET, V>(gout + o) : raw_zero<raw_t>();
-            rhp[j] = (ok && t0 + j > 0) ? load_raw<ET, V>(hs + o - D) : raw_zero<raw_t>();
-        }
+    for (int j = 0; j < TC; ++j) {
+        rx[j] = buffer_load<raw_t>(bx, lane_bytes, j * row_bytes);
+        rxg[j] = buffer_load<raw_t>(bxg, lane_bytes, j * row_bytes);
+        rag[j] = buffer_load<raw_t>(bag, lane_bytes, j * row_bytes);
+        rgo[j] = buffer_load<raw_t>(bgo, lane_bytes, j * row_bytes);
+        rhp[j] = (j == 0) ? buffer_load<raw_t>(bhm1, lane_bytes, 0u)
+                          : buffer_load<raw_t>(bhs, lane_bytes, (j - 1) * row_bytes);
     }
 
     float c2[V], cs[V];
 #pragma unroll
     for (int v = 0; v < V; ++v) {
-        const float s = softplus_precise(lam[c0 + v]);
+        const float s = softplus_precise(lam[c_tile + lane_off + v]);
         c2[v] = -8.0f * kLog2e * s;
         cs[v] = -8.0f * s;
     }
@@ -376,7 +398,7 @@ __global__ __launch_bounds__(NW * kWave) void rglru_scan_bwd_kernel(
         unpack(rag[j], fag);
         unpack(rgo[j], fgo);
         unpack(rhp[j], fhp);
-        const bool ok = full || (t0 + j < T);
+        const bool ok = FULL || (t0 + j < T);
 #pragma unroll
         for (int v = 0; v < V; ++v) {
             const float i = sigmoid_fast(fxg[v]);
@@ -403,89 +425,50 @@ __global__ __launch_bounds__(NW * kWave) void rglru_scan_bwd_kernel(
             c_run[v] = alpha * g_loc;
             q_run[v] *= alpha;
         }
+        // keep one row's temporaries live at a time: the tile must fit the register file
+        __builtin_amdgcn_sched_barrier(0);
     }
 
     // 2. combine the time slices; later slices come first in the reverse chain
 #pragma unroll
     for (int v = 0; v < V; ++v) s_agg[w][lane * V + v] = make_float2(q_run[v], c_run[v]);
     __syncthreads();
-    float p_pre[V], h_pre[V], p_tot[V], h_tot[V];
-#pragma unroll
-    for (int v = 0; v < V; ++v) { p_tot[v] = 1.0f; h_tot[v] = 0.0f; p_pre[v] = 1.0f; h_pre[v] = 0.0f; }
-#pragma unroll
-    for (int ww = NW - 1; ww >= 0; --ww) {
-#pragma unroll
-        for (int v = 0; v < V; ++v) {
-            if (ww == w) { p_pre[v] = p_tot[v]; h_pre[v] = h_tot[v]; }
-            const float2 a = s_agg[ww][lane * V + v];
-            h_tot[v] = fmaf(a.x, h_tot[v], a.y);
-            p_tot[v] *= a.x;
-        }
-    }
+    float pre_p[V], pre_h[V], tot_p[V], tot_h[V];
+    combine_slices<V, NW, true>(s_agg, w, lane, pre_p, pre_h, tot_p, tot_h);
 
     // 3. carry across tiles
     float cin[V];
 #pragma unroll
     for (int v = 0; v < V; ++v) cin[v] = 0.0f;
     if (nseg > 1) {
-        if (w == 0) {
-            const size_t stride = (size_t)B * D;
-            const size_t idx0 = (size_t)b * D + c0;
-            const size_t idx = idx0 + (size_t)pos * stride;
-            const bool publishes = pos + 1 < nseg;
-            if (publishes && !is_checkpoint(pos)) {
-#pragma unroll
-                for (int v = 0; v < V; ++v) {
-                    publish(ws.agg_p + idx + v, tag, p_tot[v]);
-                    publish(ws.agg_h + idx + v, tag, h_tot[v]);
-                }
-                asm volatile("" ::: "memory");
-            }
-            if (pos > 0) {
-#pragma unroll
-                for (int v = 0; v < V; ++v) cin[v] = look_back(ws, idx0 + v, stride, pos, tag);
-            }
-            if (publishes && is_checkpoint(pos)) {
-#pragma unroll
-                for (int v = 0; v < V; ++v) publish(ws.incl + idx + v, tag, fmaf(p_tot[v], cin[v], h_tot[v]));
-            }
-#pragma unroll
-            for (int v = 0; v < V; ++v) s_cin[lane * V + v] = cin[v];
-        }
-        __syncthreads();
-#pragma unroll
-        for (int v = 0; v < V; ++v) cin[v] = s_cin[lane * V + v];
+        exchange_carry<V, NW>(ws, pos, nseg, (size_t)b * D + c_tile + lane_off, (size_t)B * D, tag, w, lane,
+                              tot_p, tot_h, s_prev, cin);
     }
 
     // 4. apply the carry, store the three gradients, reduce the dLambda partial
     float cw[V];
 #pragma unroll
     for (int v = 0; v < V; ++v) {
-        cw[v] = fmaf(p_pre[v], cin[v], h_pre[v]);
+        cw[v] = fmaf(pre_p[v], cin[v], pre_h[v]);
         s_dl[w][lane * V + v] = fmaf(cw[v], acc_q[v], acc_a[v]);
     }
-    if (lane_on) {
 #pragma unroll
-        for (int j = 0; j < TC; ++j) {
-            if (full || (t0 + j < T)) {
-                float o1[V], o2[V], o3[V];
+    for (int j = 0; j < TC; ++j) {
+        float o1[V], o2[V], o3[V];
 #pragma unroll
-                for (int v = 0; v < V; ++v) {
-                    const float g = fmaf(qn[j][v], cw[v], gl[j][v]);
-                    o1[v] = g * k1[j][v];
-                    o2[v] = g * k2[j][v];
-                    o3[v] = g * k3[j][v];
-                }
-                raw_t r1, r2, r3;
-                pack(o1, r1);
-                pack(o2, r2);
-                pack(o3, r3);
-                const size_t o = base + (size_t)j * D;
-                store_raw<ET, V>(dx + o, r1);
-                store_raw<ET, V>(dxg + o, r2);
-                store_raw<ET, V>(dag + o, r3);
-            }
+        for (int v = 0; v < V; ++v) {
+            const float g = fmaf(qn[j][v], cw[v], gl[j][v]);
+            o1[v] = g * k1[j][v];
+            o2[v] = g * k2[j][v];
+            o3[v] = g * k3[j][v];
         }
+        raw_t r1, r2, r3;
+        pack(o1, r1);
+        pack(o2, r2);
+        pack(o3, r3);
+        buffer_store<raw_t>(r1, bdx, store_bytes, j * row_bytes);
+        buffer_store<raw_t>(r2, bdxg, store_bytes, j * row_bytes);
+        buffer_store<raw_t>(r3, bdag, store_bytes, j * row_bytes);
     }
     __syncthreads();
     if (w == 0 && lane_on) {
@@ -494,11 +477,39 @@ __global__ __launch_bounds__(NW * kWave) void rglru_scan_bwd_kernel(
             float sum = 0.0f;
 #pragma unroll
             for (int ww = 0; ww < NW; ++ww) sum += s_dl[ww][lane * V + v];
-            ws.dlam_part[((size_t)seg * B + b) * D + c0 + v] = sum;
+            ws.dlam_part[((size_t)seg * B + b) * D + c_tile + lane_off + v] = sum;
         }
     }
+}
 
-    if (nseg > 1) retire(ws.ctrl, total, tag);
+template <typename ET, int V, int TC, int NW, bool PRECISE>
+__global__ __launch_bounds__(NW * kWave, HAWK_BWD_WAVES_PER_SIMD) void rglru_scan_bwd_kernel(
+    const ET* __restrict__ x, const ET* __restrict__ xg, const ET* __restrict__ ag,
+    const float* __restrict__ lam, const ET* __restrict__ hs, const ET* __restrict__ gout,
+    ET* __restrict__ dx, ET* __restrict__ dxg, ET* __restrict__ dag, int B, int T, int D, int nseg,
+    int nct, ScanWsPtrs ws) {
+    constexpr int CT = kWave * V;
+    constexpr int TS = NW * TC;
+    __shared__ float2 s_agg[NW][CT];
+    __shared__ float2 s_prev[kLookback][CT];
+    __shared__ float s_dl[NW][CT];
+    __shared__ uint32_t s_ticket[2];
+
+    uint32_t ticket = blockIdx.x, tag = 0;
+    if (nseg > 1) take_ticket(ws.ctrl, (uint32_t)nseg * (uint32_t)B * (uint32_t)nct, s_ticket, ticket, tag);
+
+    const int per_seg = B * nct;
+    const int pos = ticket / per_seg;  // chain position: 0 is the LAST time tile
+    const int seg = nseg - 1 - pos;
+    const int rem = ticket - pos * per_seg;
+    const int b = rem / nct;
+    const int ct = rem - b * nct;
+    if (seg > 0 && seg * TS + TS <= T)
+        bwd_tile<ET, V, TC, NW, PRECISE, true>(x, xg, ag, lam, hs, gout, dx, dxg, dag, B, T, D, nseg, seg, pos, b,
+                                               ct, tag, ws, s_agg, s_prev, s_dl);
+    else
+        bwd_tile<ET, V, TC, NW, PRECISE, false>(x, xg, ag, lam, hs, gout, dx, dxg, dag, B, T, D, nseg, seg, pos, b,
+                                                ct, tag, ws, s_agg, s_prev, s_dl);
 }
 
 // dLambda[c] = -8 sigmoid(Lambda_c) * sum over rows of the [rows, D] partials.
@@ -585,7 +596,7 @@ WsLayout layout_for(int B, int D, int nseg_chain, int nseg_dlam) {
 ScanWsPtrs carve(void* ws, const WsLayout& l) {
     char* p = static_cast<char*>(ws);
     ScanWsPtrs r;
-    r.ctrl = reinterpret_cast<uint32_t*>(p);
+    r.ctrl = reinterpret_cast<unsigned long long*>(p);
     r.incl = reinterpret_cast<unsigned long long*>(p + l.off_incl);
     r.agg_p = reinterpret_cast<unsigned long long*>(p + l.off_aggp);
     r.agg_h = reinterpret_cast<unsigned long long*>(p + l.off_aggh);
@@ -634,7 +645,7 @@ int workspace_init(void* ws, size_t bytes, hipStream_t st) {
 
 int workspace_status(const void* ws, hipStream_t st, int* flag) {
     uint32_t v = 0;
-    if (hipMemcpyAsync(&v, static_cast<const uint32_t*>(ws) + kError, sizeof(v), hipMemcpyDeviceToHost, st) != hipSuccess)
+    if (hipMemcpyAsync(&v, static_cast<const uint32_t*>(ws) + 2, sizeof(v), hipMemcpyDeviceToHost, st) != hipSuccess)
         return HAWK_ERR_LAUNCH;
     if (hipStreamSynchronize(st) != hipSuccess) return HAWK_ERR_LAUNCH;
     *flag = (int)v;
