@@ -184,6 +184,13 @@ __device__ __forceinline__ float sigmoid_precise(float x) {
     return e / (1.0f + e);
 }
 
+// Identity the optimiser cannot see through: stops it from keeping a value alive in a
+// register across a long region when re-evaluating it later is the cheaper choice.
+__device__ __forceinline__ float opaque(float x) {
+    asm volatile("" : "+v"(x));
+    return x;
+}
+
 __device__ __forceinline__ float clamp01(float z) { return fminf(fmaxf(z, 0.0f), 1.0f); }
 
 }  // namespace hawk

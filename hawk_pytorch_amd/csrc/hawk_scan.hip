@@ -326,10 +326,12 @@ __global__ __launch_bounds__(NW * kWave, HAWK_FWD_WAVES_PER_SIMD) void rglru_sca
 
 // ---------------------------------------------------------------------------------------
 // Backward.  Reverse chain on c_t = alpha_t (gout_t + c_{t+1}); g_t = gout_t + c_{t+1}.
-// Per element, everything that multiplies g_t is precomputed in the local pass:
-//   dx = g K1, dx_rg_lru = g K2, da_rg_lru = g K3, dLambda += g K4 (scaled per channel later)
-//   K1 = m i;  K2 = m x i (1-i);  K4 = (h_{t-1} alpha - i x alpha^2 2 csg(1-alpha^2)) r;
-//   K3 = K4 (1-r) (-8 softplus(Lambda)).
+// The chain itself needs only alpha and gout, so the local pass evaluates just those (and
+// keeps r); once the carry into the slice is known, the recurrence is replayed
+// exactly and each row's gradients are formed and stored on the spot:
+//   dx = g m i;  dx_rg_lru = g m x i (1-i);
+//   dlog_a = g (h_{t-1} alpha - i x alpha^2 2 csg(1-alpha^2));
+//   da_rg_lru = dlog_a r (1-r) (-8 softplus(Lambda));  dLambda += dlog_a r  (scaled per channel later)
 // FULL: every row of the tile is inside [1, T) (row 0 has no h_{t-1}).
 // ---------------------------------------------------------------------------------------
 template <typename ET, int V, int TC, int NW, bool PRECISE, bool FULL>
@@ -385,48 +387,27 @@ __device__ __forceinline__ void bwd_tile(const ET* __restrict__ x, const ET* __r
         cs[v] = -8.0f * s;
     }
 
-    // 1. local reverse scan from a zero carry
-    float qn[TC][V], gl[TC][V], k1[TC][V], k2[TC][V], k3[TC][V];
-    float q_run[V], c_run[V], acc_a[V], acc_q[V];
+    // 1. local reverse scan of c from a zero carry: needs only alpha and gout.  r
+    //    is kept; everything else is evaluated after the carry is known.
+    float rr[TC][V];
+    float q_run[V], c_run[V];
 #pragma unroll
-    for (int v = 0; v < V; ++v) { q_run[v] = 1.0f; c_run[v] = 0.0f; acc_a[v] = 0.0f; acc_q[v] = 0.0f; }
+    for (int v = 0; v < V; ++v) { q_run[v] = 1.0f; c_run[v] = 0.0f; }
 #pragma unroll
     for (int j = TC - 1; j >= 0; --j) {
-        float fx[V], fxg[V], fag[V], fgo[V], fhp[V];
-        unpack(rx[j], fx);
-        unpack(rxg[j], fxg);
+        float fag[V], fgo[V];
         unpack(rag[j], fag);
         unpack(rgo[j], fgo);
-        unpack(rhp[j], fhp);
         const bool ok = FULL || (t0 + j < T);
 #pragma unroll
         for (int v = 0; v < V; ++v) {
-            const float i = sigmoid_fast(fxg[v]);
             const float r = sigmoid_fast(fag[v]);
             float alpha = hw_exp2(c2[v] * r);
-            const float a2 = alpha * alpha;
-            const float z = PRECISE ? one_minus_exp(2.0f * cs[v] * r) : clamp01(1.0f - a2);
-            const float rs = hw_rsq(fmaxf(z, 1e-30f));
-            const float m = z * rs;
-            // 2 * clipped sqrt derivative: 1/sqrt(max(4z,1e-6)) = 0.5/sqrt(max(z,2.5e-7))
-            const float csg2 = (z >= 2.5e-7f) ? rs : 2000.0f;
-            const float ix = i * fx[v];
-            const float mi = m * i;
-            float k4 = fmaf(fhp[v], alpha, -(ix * a2) * csg2) * r;
-            if (!ok) { alpha = 1.0f; k4 = 0.0f; }
-            k1[j][v] = mi;
-            k2[j][v] = (m * ix) * (1.0f - i);
-            k3[j][v] = (k4 * (1.0f - r)) * cs[v];
-            const float g_loc = fgo[v] + c_run[v];
-            gl[j][v] = g_loc;
-            qn[j][v] = q_run[v];
-            acc_a[v] = fmaf(g_loc, k4, acc_a[v]);
-            acc_q[v] = fmaf(q_run[v], k4, acc_q[v]);
-            c_run[v] = alpha * g_loc;
+            if (!ok) alpha = 1.0f;  // rows past T are the identity
+            rr[j][v] = r;
+            c_run[v] = alpha * (fgo[v] + c_run[v]);
             q_run[v] *= alpha;
         }
-        // keep one row's temporaries live at a time: the tile must fit the register file
-        __builtin_amdgcn_sched_barrier(0);
     }
 
     // 2. combine the time slices; later slices come first in the reverse chain
@@ -445,22 +426,46 @@ __device__ __forceinline__ void bwd_tile(const ET* __restrict__ x, const ET* __r
                               tot_p, tot_h, s_prev, cin);
     }
 
-    // 4. apply the carry, store the three gradients, reduce the dLambda partial
-    float cw[V];
+    // 4. the exact recurrence from the true carry, with the gradients of each row computed
+    //    and stored as its g_t becomes known
+    float c_true[V], acc[V];
 #pragma unroll
     for (int v = 0; v < V; ++v) {
-        cw[v] = fmaf(pre_p[v], cin[v], pre_h[v]);
-        s_dl[w][lane * V + v] = fmaf(cw[v], acc_q[v], acc_a[v]);
+        c_true[v] = fmaf(pre_p[v], cin[v], pre_h[v]);
+        acc[v] = 0.0f;
     }
 #pragma unroll
-    for (int j = 0; j < TC; ++j) {
+    for (int j = TC - 1; j >= 0; --j) {
+        float fx[V], fxg[V], fgo[V], fhp[V];
+        unpack(rx[j], fx);
+        unpack(rxg[j], fxg);
+        unpack(rgo[j], fgo);
+        unpack(rhp[j], fhp);
+        const bool ok = FULL || (t0 + j < T);
         float o1[V], o2[V], o3[V];
 #pragma unroll
         for (int v = 0; v < V; ++v) {
-            const float g = fmaf(qn[j][v], cw[v], gl[j][v]);
-            o1[v] = g * k1[j][v];
-            o2[v] = g * k2[j][v];
-            o3[v] = g * k3[j][v];
+            const float r = opaque(rr[j][v]);
+            float alpha = hw_exp2(c2[v] * r);  // cheaper to re-evaluate than to keep in a register
+            if (!ok) alpha = 1.0f;
+            const float g = fgo[v] + c_true[v];
+            c_true[v] = alpha * g;
+            const float i = sigmoid_fast(fxg[v]);
+            const float a2 = alpha * alpha;
+            const float z = PRECISE ? one_minus_exp(2.0f * cs[v] * r) : clamp01(1.0f - a2);
+            const float rs = hw_rsq(fmaxf(z, 1e-30f));
+            const float m = z * rs;
+            // 2 * clipped sqrt derivative: 1/sqrt(max(4z,1e-6)) = 0.5/sqrt(max(z,2.5e-7))
+            const float csg2 = (z >= 2.5e-7f) ? rs : 2000.0f;
+            const float ix = i * fx[v];
+            const float gm = g * m;
+            float k4 = fmaf(fhp[v], alpha, -(ix * a2) * csg2) * r;  // dlog_a / g * r
+            if (!ok) k4 = 0.0f;
+            const float gk4 = g * k4;
+            o1[v] = gm * i;
+            o2[v] = (gm * ix) * (1.0f - i);
+            o3[v] = (gk4 * (1.0f - r)) * cs[v];
+            acc[v] += gk4;
         }
         raw_t r1, r2, r3;
         pack(o1, r1);
@@ -470,6 +475,8 @@ __device__ __forceinline__ void bwd_tile(const ET* __restrict__ x, const ET* __r
         buffer_store<raw_t>(r2, bdxg, store_bytes, j * row_bytes);
         buffer_store<raw_t>(r3, bdag, store_bytes, j * row_bytes);
     }
+#pragma unroll
+    for (int v = 0; v < V; ++v) s_dl[w][lane * V + v] = acc[v];
     __syncthreads();
     if (w == 0 && lane_on) {
 #pragma unroll
@@ -555,28 +562,17 @@ struct TileShape {
     int chans() const { return kWave * V; }
 };
 
-// Widest per-lane vector that divides D and keeps every row start aligned.
-int pick_v(int D, int dtype, int vmax) {
-    int v = vmax;
-    while (v > 1 && (D % v) != 0) v >>= 1;
-    (void)dtype;
-    return v;
-}
+// Tile shapes.  A lane moves 4 bytes per row access: two bf16 channels (one when D is
+// odd) or one fp32 channel, so a wave covers 256 contiguous bytes of a row.  The forward
+// keeps 2 floats per element across the carry exchange, the backward keeps the packed
+// inputs and one float, which sets how many rows fit in 128 VGPRs (4 waves per SIMD).
+constexpr int kFwdTC = 16, kFwdNW = 8;
+constexpr int kBwdTC = 8, kBwdNW = 8;
 
-TileShape fwd_shape(int D, int dtype) {
-    TileShape s;
-    s.V = pick_v(D, dtype, 2);
-    if (dtype == HAWK_DTYPE_BF16) { s.TC = 16; s.NW = 8; }
-    else { s.TC = 8; s.NW = 8; }
-    return s;
-}
-TileShape bwd_shape(int D, int dtype) {
-    TileShape s;
-    s.V = pick_v(D, dtype, 2);
-    s.TC = 8;
-    s.NW = 8;
-    return s;
-}
+int pick_v(int D, int dtype) { return (dtype == HAWK_DTYPE_BF16 && (D % 2) == 0) ? 2 : 1; }
+
+TileShape fwd_shape(int D, int dtype) { return TileShape{pick_v(D, dtype), kFwdTC, kFwdNW}; }
+TileShape bwd_shape(int D, int dtype) { return TileShape{pick_v(D, dtype), kBwdTC, kBwdNW}; }
 
 int ceil_div(int a, int b) { return (a + b - 1) / b; }
 
@@ -663,16 +659,12 @@ int scan_fwd(const void* x, const void* xg, const void* ag, const float* lam, vo
         if (ws == nullptr || ws_bytes < l.total) return HAWK_ERR_WORKSPACE;
         p = carve(ws, l);
     }
-#define HAWK_FWD(ET, V_, TC_, NW_, PR) \
-    return launch_fwd<ET, V_, TC_, NW_, PR>(x, xg, ag, lam, h, B, T, D, nseg, nct, p, st)
     if (dtype == HAWK_DTYPE_BF16) {
-        if (s.V == 2) HAWK_FWD(bf16_t, 2, 16, 8, false);
-        HAWK_FWD(bf16_t, 1, 16, 8, false);
-    } else {
-        if (s.V == 2) HAWK_FWD(float, 2, 8, 8, true);
-        HAWK_FWD(float, 1, 8, 8, true);
+        if (s.V == 2)
+            return launch_fwd<bf16_t, 2, kFwdTC, kFwdNW, false>(x, xg, ag, lam, h, B, T, D, nseg, nct, p, st);
+        return launch_fwd<bf16_t, 1, kFwdTC, kFwdNW, false>(x, xg, ag, lam, h, B, T, D, nseg, nct, p, st);
     }
-#undef HAWK_FWD
+    return launch_fwd<float, 1, kFwdTC, kFwdNW, true>(x, xg, ag, lam, h, B, T, D, nseg, nct, p, st);
 }
 
 int scan_bwd(const void* x, const void* xg, const void* ag, const float* lam, const void* hs, const void* gout,
@@ -685,16 +677,17 @@ int scan_bwd(const void* x, const void* xg, const void* ag, const float* lam, co
     if (ws == nullptr || ws_bytes < l.total) return HAWK_ERR_WORKSPACE;
     const ScanWsPtrs p = carve(ws, l);
     int rc;
-#define HAWK_BWD(ET, V_, TC_, NW_, PR) \
-    rc = launch_bwd<ET, V_, TC_, NW_, PR>(x, xg, ag, lam, hs, gout, dx, dxg, dag, B, T, D, nseg, nct, p, st)
     if (dtype == HAWK_DTYPE_BF16) {
-        if (s.V == 2) HAWK_BWD(bf16_t, 2, 8, 8, false);
-        else HAWK_BWD(bf16_t, 1, 8, 8, false);
+        if (s.V == 2)
+            rc = launch_bwd<bf16_t, 2, kBwdTC, kBwdNW, false>(x, xg, ag, lam, hs, gout, dx, dxg, dag, B, T, D, nseg,
+                                                              nct, p, st);
+        else
+            rc = launch_bwd<bf16_t, 1, kBwdTC, kBwdNW, false>(x, xg, ag, lam, hs, gout, dx, dxg, dag, B, T, D, nseg,
+                                                              nct, p, st);
     } else {
-        if (s.V == 2) HAWK_BWD(float, 2, 8, 8, true);
-        else HAWK_BWD(float, 1, 8, 8, true);
+        rc = launch_bwd<float, 1, kBwdTC, kBwdNW, true>(x, xg, ag, lam, hs, gout, dx, dxg, dag, B, T, D, nseg, nct, p,
+                                                        st);
     }
-#undef HAWK_BWD
     if (rc != HAWK_OK) return rc;
     hipLaunchKernelGGL(dlam_reduce_kernel, dim3((unsigned)ceil_div(D, kWave)), dim3(1024), 0, st, p.dlam_part, lam,
                        dlam, nseg * B, D);
