@@ -13,7 +13,8 @@ import threading
 import torch
 
 _CSRC = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc")
-LIB_PATH = os.path.join(_CSRC, "libhawk_hip.so")
+# HAWK_HIP_LIB selects another build of the library (e.g. one compiled with other tile shapes)
+LIB_PATH = os.environ.get("HAWK_HIP_LIB") or os.path.join(_CSRC, "libhawk_hip.so")
 
 HAWK_OK = 0
 HAWK_ERR_NULL_POINTER = 1

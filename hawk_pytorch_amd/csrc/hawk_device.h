@@ -173,8 +173,27 @@ __device__ __forceinline__ float one_minus_exp(float y) {
     return (y > -0.25f) ? series : direct;
 }
 
-// Numerically safe softplus / logistic for the per-channel Lambda (evaluated once per
-// lane, not per element, so the precise library routines are affordable here).
+// softplus(x) = log(1 + e^x) to about 1e-6 relative accuracy over the whole range
+// (Lambda is strongly negative at init, so relative accuracy for tiny results matters), in a
+// dozen instructions: it is evaluated per lane per tile, so a library-grade routine would
+// cost as much as several rows of the scan itself.
+//   u = e^x;  u < 1/16: series u (1 - u/2 + u^2/3 - u^3/4 + u^4/5);  else ln2 * log2(1 + u);
+//   x > 16: x + e^-x.
+__device__ __forceinline__ float softplus_fast(float x) {
+    const float u = hw_exp2(kLog2e * fminf(x, 16.0f));
+    float p = 0.2f;
+    p = fmaf(p, u, -0.25f);
+    p = fmaf(p, u, 1.0f / 3.0f);
+    p = fmaf(p, u, -0.5f);
+    p = fmaf(p, u, 1.0f);
+    const float small = u * p;
+    const float mid = 0.6931471805599453f * __builtin_amdgcn_logf(1.0f + u);
+    const float big = x + hw_exp2(-kLog2e * fmaxf(x, 16.0f));
+    const float lo = (u < 0.0625f) ? small : mid;
+    return (x > 16.0f) ? big : lo;
+}
+
+// Library-grade variants, for code that runs once per channel per launch.
 __device__ __forceinline__ float softplus_precise(float x) {
     return x > 20.0f ? x : log1pf(expf(x));
 }

@@ -235,7 +235,7 @@ __device__ __forceinline__ void fwd_tile(const ET* __restrict__ x, const ET* __r
     float c2[V], cn[V];
 #pragma unroll
     for (int v = 0; v < V; ++v) {
-        const float s = softplus_precise(lam[c_tile + lane_off + v]);
+        const float s = softplus_fast(lam[c_tile + lane_off + v]);
         c2[v] = -8.0f * kLog2e * s;
         cn[v] = -16.0f * s;
     }
@@ -382,7 +382,7 @@ __device__ __forceinline__ void bwd_tile(const ET* __restrict__ x, const ET* __r
     float c2[V], cs[V];
 #pragma unroll
     for (int v = 0; v < V; ++v) {
-        const float s = softplus_precise(lam[c_tile + lane_off + v]);
+        const float s = softplus_fast(lam[c_tile + lane_off + v]);
         c2[v] = -8.0f * kLog2e * s;
         cs[v] = -8.0f * s;
     }
@@ -566,8 +566,20 @@ struct TileShape {
 // odd) or one fp32 channel, so a wave covers 256 contiguous bytes of a row.  The forward
 // keeps 2 floats per element across the carry exchange, the backward keeps the packed
 // inputs and one float, which sets how many rows fit in 128 VGPRs (4 waves per SIMD).
-constexpr int kFwdTC = 16, kFwdNW = 8;
-constexpr int kBwdTC = 8, kBwdNW = 8;
+#ifndef HAWK_FWD_TC
+#define HAWK_FWD_TC 16
+#endif
+#ifndef HAWK_FWD_NW
+#define HAWK_FWD_NW 8
+#endif
+#ifndef HAWK_BWD_TC
+#define HAWK_BWD_TC 8
+#endif
+#ifndef HAWK_BWD_NW
+#define HAWK_BWD_NW 8
+#endif
+constexpr int kFwdTC = HAWK_FWD_TC, kFwdNW = HAWK_FWD_NW;
+constexpr int kBwdTC = HAWK_BWD_TC, kBwdNW = HAWK_BWD_NW;
 
 int pick_v(int D, int dtype) { return (dtype == HAWK_DTYPE_BF16 && (D % 2) == 0) ? 2 : 1; }
 
