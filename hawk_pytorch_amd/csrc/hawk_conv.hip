@@ -300,7 +300,16 @@ __global__ __launch_bounds__(1024) void colsum_kernel(const float* __restrict__ 
     const int c = blockIdx.x * kWave + lane;
     float sum = 0.0f;
     if (c < cols) {
-        for (int r = slice; r < rows; r += 16) sum += part[(size_t)r * cols + c];
+        // eight independent loads in flight per thread; the order of additions is fixed
+        int r = slice;
+        for (; r + 16 * 7 < rows; r += 16 * 8) {
+            float v[8];
+#pragma unroll
+            for (int k = 0; k < 8; ++k) v[k] = part[(size_t)(r + 16 * k) * cols + c];
+#pragma unroll
+            for (int k = 0; k < 8; ++k) sum += v[k];
+        }
+        for (; r < rows; r += 16) sum += part[(size_t)r * cols + c];
     }
     s[slice][lane] = sum;
     __syncthreads();
