@@ -37,6 +37,16 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0
 
+# HBM bytes per launch of the backward scan kernel, from rocprofv3 --pmc FETCH_SIZE and
+# WRITE_SIZE runs of this file, each scaled by what the same counter reads for a plain
+# device copy of known size in the same run (FETCH x 2.000, WRITE x 1.000 on this part).
+# Sources: profiles/rglru_scan_B8_T4096_D2560_bf16.md, profiles/rglru_scan_B2_T32768_D4096_bf16.md.
+MEASURED_BWD_TRAFFIC_BYTES = {
+    "scan": 903.6e6 + 547.5e6,
+    "scan_conv": 903.6e6 + 547.5e6,
+    "long": 2902e6 + 1754e6,
+}
+
 WORKLOADS = {
     # name: (B, T, D, a^8 range, includes conv)
     "scan": (8, 4096, 2560, (0.9, 0.999), False),
@@ -81,6 +91,10 @@ def main():
     ap.add_argument("--workload", choices=sorted(WORKLOADS), default="scan")
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibration-copy", action="store_true",
+                    help="also run three plain device-to-device copies of one activation tensor (outside the "
+                         "timed region) so that a rocprofv3 --pmc run has a kernel of known traffic to scale "
+                         "FETCH_SIZE / WRITE_SIZE by")
     args = ap.parse_args()
 
     if args.gpus != 1:
@@ -141,6 +155,11 @@ def main():
         _lib.check("conv_bwd", lib.hawk_conv1d_bwd(dx.data_ptr(), x.data_ptr(), cw.data_ptr(), du.data_ptr(),
                                                    dw.data_ptr(), db.data_ptr(), B, T, D, W, code, code,
                                                    cws.data_ptr(), cws.numel(), stream))
+
+    if args.calibration_copy:
+        for _ in range(3):
+            h.copy_(x)  # reads 2*N bytes, writes 2*N bytes
+        torch.cuda.synchronize()
 
     for _ in range(args.warmup):
         fwd()
@@ -203,7 +222,7 @@ def main():
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": bwd_gbs / HBM_PEAK_GBS,
-            "traffic": None,
+            "traffic": MEASURED_BWD_TRAFFIC_BYTES.get(args.workload),
             "algorithmic_bytes_per_launch": bwd_bytes,
             "launch_ms": bwd_ms,
         },
