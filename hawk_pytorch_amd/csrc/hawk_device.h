@@ -36,6 +36,16 @@ __device__ __forceinline__ uint16_t to_bf16_bits(float f) {
 __device__ __forceinline__ float bf16_lo(uint32_t w) { return __uint_as_float(w << 16); }
 __device__ __forceinline__ float bf16_hi(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
 
+// Two fp32 in [0,1] -> packed fp16 pair (one v_cvt_pkrtz_f16_f32) and back.  Used only for
+// running products of alpha that scale a carry: their 2^-10 relative error lands on a
+// correction term and is far below the bf16 rounding of the stored result.
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t pack_f16x2(float lo, float hi) {
+    return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(lo, hi));
+}
+__device__ __forceinline__ float f16_lo(uint32_t w) { return (float)__builtin_bit_cast(f16x2, w).x; }
+__device__ __forceinline__ float f16_hi(uint32_t w) { return (float)__builtin_bit_cast(f16x2, w).y; }
+
 // Raw register image of V consecutive elements of type ET.
 template <typename ET, int V>
 struct Raw;
