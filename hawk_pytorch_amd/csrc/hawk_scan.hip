@@ -82,7 +82,10 @@ __device__ __forceinline__ bool try_read(const unsigned long long* p, uint32_t t
 // first.  The order of the floating-point operations is fixed by the position alone,
 // never by timing, so results are bitwise reproducible, and the serial dependency runs
 // over checkpoints only (nseg / kLookback hops of one memory round trip each).
-constexpr int kLookback = 8;
+#ifndef HAWK_LOOKBACK
+#define HAWK_LOOKBACK 4
+#endif
+constexpr int kLookback = HAWK_LOOKBACK;
 
 __device__ __forceinline__ bool is_checkpoint(int pos) { return (pos % kLookback) == 0; }
 __device__ __forceinline__ int checkpoint_before(int pos) { return ((pos - 1) / kLookback) * kLookback; }
