@@ -225,6 +225,10 @@ __device__ __forceinline__ float opaque(float x) {
     asm volatile("" : "+v"(x));
     return x;
 }
+__device__ __forceinline__ uint32_t opaque(uint32_t x) {
+    asm volatile("" : "+v"(x));
+    return x;
+}
 
 __device__ __forceinline__ float clamp01(float z) { return fminf(fmaxf(z, 0.0f), 1.0f); }
 

@@ -673,15 +673,14 @@ __device__ __forceinline__ void bwd_tile(const ET* __restrict__ x, const ET* __r
     // idle lanes store at an offset beyond any slab, which the range check drops
     const uint32_t store_bytes = lane_on ? lane_bytes : 0x80000000u;
 
+    // The local pass needs only a_rg_lru and grad_out; x, x_rg_lru and h are fetched after
+    // it (their registers would otherwise sit idle through it) and arrive during the carry
+    // exchange.  This is what lets a lane own TC rows within 128 registers.
     raw_t rx[TC], rxg[TC], rag[TC], rgo[TC], rhp[TC];
 #pragma unroll
     for (int j = 0; j < TC; ++j) {
-        rx[j] = buffer_load<raw_t>(bx, lane_bytes, j * row_bytes);
-        rxg[j] = buffer_load<raw_t>(bxg, lane_bytes, j * row_bytes);
         rag[j] = buffer_load<raw_t>(bag, lane_bytes, j * row_bytes);
         rgo[j] = buffer_load<raw_t>(bgo, lane_bytes, j * row_bytes);
-        rhp[j] = (j == 0) ? buffer_load<raw_t>(bhm1, lane_bytes, 0u)
-                          : buffer_load<raw_t>(bhs, lane_bytes, (j - 1) * row_bytes);
     }
 
     float c2[V], cs[V];
@@ -694,26 +693,46 @@ __device__ __forceinline__ void bwd_tile(const ET* __restrict__ x, const ET* __r
 
     // 1. local reverse scan of c from a zero carry: needs only alpha and gout.  r
     //    is kept; everything else is evaluated after the carry is known.
-    float rr[TC][V];
+    // r is kept as an fp16 pair for bf16 activations (2^-11 relative, well inside the bf16
+    // rounding of the gradients), in fp32 otherwise.
+    constexpr bool PACK_R = (V == 2) && (sizeof(ET) == 2);
+    float rr[PACK_R ? 1 : TC][V];
+    uint32_t rrh[PACK_R ? TC : 1];
     float q_run[V], c_run[V];
 #pragma unroll
     for (int v = 0; v < V; ++v) { q_run[v] = 1.0f; c_run[v] = 0.0f; }
 #pragma unroll
     for (int j = TC - 1; j >= 0; --j) {
-        float fag[V], fgo[V];
+        float fag[V], fgo[V], rv[V];
         unpack(rag[j], fag);
         unpack(rgo[j], fgo);
         const bool ok = FULL || (t0 + j < T);
 #pragma unroll
+        for (int v = 0; v < V; ++v) rv[v] = sigmoid_fast(fag[v]);
+        if (PACK_R) {
+            // the chain must see exactly the r the replay will see
+            rrh[j] = pack_f16x2(rv[0], rv[V - 1]);
+            rv[0] = f16_lo(rrh[j]);
+            rv[V - 1] = f16_hi(rrh[j]);
+        }
+#pragma unroll
         for (int v = 0; v < V; ++v) {
-            const float r = sigmoid_fast(fag[v]);
-            float alpha = hw_exp2(c2[v] * r);
+            float alpha = hw_exp2(c2[v] * rv[v]);
             if (!ok) alpha = 1.0f;  // rows past T are the identity
-            rr[j][v] = r;
+            if (!PACK_R) rr[j][v] = rv[v];
             c_run[v] = alpha * (fgo[v] + c_run[v]);
             q_run[v] *= alpha;
         }
     }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int j = 0; j < TC; ++j) {
+        rx[j] = buffer_load<raw_t>(bx, lane_bytes, j * row_bytes);
+        rxg[j] = buffer_load<raw_t>(bxg, lane_bytes, j * row_bytes);
+        rhp[j] = (j == 0) ? buffer_load<raw_t>(bhm1, lane_bytes, 0u)
+                          : buffer_load<raw_t>(bhs, lane_bytes, (j - 1) * row_bytes);
+    }
+    __builtin_amdgcn_sched_barrier(0);
 
     // 2. combine the time slices; later slices come first in the reverse chain
 #pragma unroll
@@ -744,13 +763,19 @@ __device__ __forceinline__ void bwd_tile(const ET* __restrict__ x, const ET* __r
         float fx[V], fxg[V], fgo[V], fhp[V];
         unpack(rx[j], fx);
         unpack(rxg[j], fxg);
-        unpack(rgo[j], fgo);
+        if constexpr (sizeof(raw_t) == 4 && sizeof(ET) == 2) {
+            // unpack again rather than keep the local pass's floats alive across the exchange
+            unpack(opaque(rgo[j]), fgo);
+        } else {
+            unpack(rgo[j], fgo);
+        }
         unpack(rhp[j], fhp);
         const bool ok = FULL || (t0 + j < T);
+        const uint32_t rpair = PACK_R ? opaque(rrh[j]) : 0u;
         float o1[V], o2[V], o3[V];
 #pragma unroll
         for (int v = 0; v < V; ++v) {
-            const float r = opaque(rr[j][v]);
+            const float r = PACK_R ? (v == 0 ? f16_lo(rpair) : f16_hi(rpair)) : opaque(rr[j][v]);
             float alpha = hw_exp2(c2[v] * r);  // cheaper to re-evaluate than to keep in a register
             if (!ok) alpha = 1.0f;
             const float g = fgo[v] + c_true[v];
@@ -779,6 +804,7 @@ __device__ __forceinline__ void bwd_tile(const ET* __restrict__ x, const ET* __r
         buffer_store<raw_t>(r1, bdx, store_bytes, j * row_bytes);
         buffer_store<raw_t>(r2, bdxg, store_bytes, j * row_bytes);
         buffer_store<raw_t>(r3, bdag, store_bytes, j * row_bytes);
+        __builtin_amdgcn_sched_barrier(0);  // one row's temporaries live at a time
     }
 #pragma unroll
     for (int v = 0; v < V; ++v) s_dl[w][lane * V + v] = acc[v];
@@ -887,7 +913,7 @@ struct TileShape {
 #define HAWK_FWD_NW 8
 #endif
 #ifndef HAWK_BWD_TC
-#define HAWK_BWD_TC 8
+#define HAWK_BWD_TC 12
 #endif
 #ifndef HAWK_BWD_NW
 #define HAWK_BWD_NW 8
