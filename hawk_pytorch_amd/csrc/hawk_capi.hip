@@ -58,26 +58,35 @@ int hawk_scan_workspace_status(const void* workspace_device, void* stream, int* 
     return hawk::workspace_status(workspace_device, as_stream(stream), flag);
 }
 
-int hawk_rglru_scan_fwd(const void* x, const void* x_rg_lru, const void* a_rg_lru, const float* a_param, void* h,
-                        int B, int T, int D, int dtype, void* workspace_device, size_t workspace_bytes,
-                        void* stream) {
+int hawk_rglru_scan_fwd_mixed(const void* x, const void* x_rg_lru, const void* a_rg_lru, const float* a_param,
+                              void* h, int B, int T, int D, int in_dtype, int out_dtype, void* workspace_device,
+                              size_t workspace_bytes, void* stream) {
     if (!x || !x_rg_lru || !a_rg_lru || !a_param || !h) return HAWK_ERR_NULL_POINTER;
-    if (!dtype_ok(dtype)) return HAWK_ERR_BAD_DTYPE;
+    if (!dtype_ok(in_dtype) || !dtype_ok(out_dtype) || !hawk::scan_dtypes_supported(in_dtype, out_dtype))
+        return HAWK_ERR_BAD_DTYPE;
     if (int rc = check_scan_shape(B, T, D)) return rc;
     if (!aligned16(x) || !aligned16(x_rg_lru) || !aligned16(a_rg_lru) || !aligned16(h)) return HAWK_ERR_ALIGNMENT;
     if (workspace_device && !aligned16(workspace_device)) return HAWK_ERR_ALIGNMENT;
-    return hawk::scan_fwd(x, x_rg_lru, a_rg_lru, a_param, h, B, T, D, dtype, workspace_device, workspace_bytes,
-                          as_stream(stream));
+    return hawk::scan_fwd(x, x_rg_lru, a_rg_lru, a_param, h, B, T, D, in_dtype, out_dtype, workspace_device,
+                          workspace_bytes, as_stream(stream));
 }
 
-int hawk_rglru_scan_bwd(const void* x, const void* x_rg_lru, const void* a_rg_lru, const float* a_param,
-                        const void* h_saved, const void* grad_out, void* dx, void* dx_rg_lru, void* da_rg_lru,
-                        float* da_param, int B, int T, int D, int dtype, void* workspace_device,
-                        size_t workspace_bytes, void* stream) {
+int hawk_rglru_scan_fwd(const void* x, const void* x_rg_lru, const void* a_rg_lru, const float* a_param, void* h,
+                        int B, int T, int D, int dtype, void* workspace_device, size_t workspace_bytes,
+                        void* stream) {
+    return hawk_rglru_scan_fwd_mixed(x, x_rg_lru, a_rg_lru, a_param, h, B, T, D, dtype, dtype, workspace_device,
+                                     workspace_bytes, stream);
+}
+
+int hawk_rglru_scan_bwd_mixed(const void* x, const void* x_rg_lru, const void* a_rg_lru, const float* a_param,
+                              const void* h_saved, const void* grad_out, void* dx, void* dx_rg_lru, void* da_rg_lru,
+                              float* da_param, int B, int T, int D, int in_dtype, int state_dtype,
+                              void* workspace_device, size_t workspace_bytes, void* stream) {
     if (!x || !x_rg_lru || !a_rg_lru || !a_param || !h_saved || !grad_out || !dx || !dx_rg_lru || !da_rg_lru ||
         !da_param)
         return HAWK_ERR_NULL_POINTER;
-    if (!dtype_ok(dtype)) return HAWK_ERR_BAD_DTYPE;
+    if (!dtype_ok(in_dtype) || !dtype_ok(state_dtype) || !hawk::scan_dtypes_supported(in_dtype, state_dtype))
+        return HAWK_ERR_BAD_DTYPE;
     if (int rc = check_scan_shape(B, T, D)) return rc;
     if (!aligned16(x) || !aligned16(x_rg_lru) || !aligned16(a_rg_lru) || !aligned16(h_saved) ||
         !aligned16(grad_out) || !aligned16(dx) || !aligned16(dx_rg_lru) || !aligned16(da_rg_lru))
@@ -85,7 +94,15 @@ int hawk_rglru_scan_bwd(const void* x, const void* x_rg_lru, const void* a_rg_lr
     if (workspace_device == nullptr) return HAWK_ERR_WORKSPACE;
     if (!aligned16(workspace_device)) return HAWK_ERR_ALIGNMENT;
     return hawk::scan_bwd(x, x_rg_lru, a_rg_lru, a_param, h_saved, grad_out, dx, dx_rg_lru, da_rg_lru, da_param, B,
-                          T, D, dtype, workspace_device, workspace_bytes, as_stream(stream));
+                          T, D, in_dtype, state_dtype, workspace_device, workspace_bytes, as_stream(stream));
+}
+
+int hawk_rglru_scan_bwd(const void* x, const void* x_rg_lru, const void* a_rg_lru, const float* a_param,
+                        const void* h_saved, const void* grad_out, void* dx, void* dx_rg_lru, void* da_rg_lru,
+                        float* da_param, int B, int T, int D, int dtype, void* workspace_device,
+                        size_t workspace_bytes, void* stream) {
+    return hawk_rglru_scan_bwd_mixed(x, x_rg_lru, a_rg_lru, a_param, h_saved, grad_out, dx, dx_rg_lru, da_rg_lru,
+                                     da_param, B, T, D, dtype, dtype, workspace_device, workspace_bytes, stream);
 }
 
 int hawk_conv1d_fwd(const void* x, const float* w, const float* bias, const void* state, void* y, int B, int T,

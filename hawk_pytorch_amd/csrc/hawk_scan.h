@@ -12,11 +12,14 @@ namespace hawk {
 size_t scan_workspace_bytes(int B, int T, int D, int dtype);
 int workspace_init(void* ws, size_t bytes, hipStream_t st);
 int workspace_status(const void* ws, hipStream_t st, int* flag);
+// in_dtype: x, x_rg_lru, a_rg_lru (and, in the backward, their gradients);
+// out_dtype / state_dtype: h (and, in the backward, the saved h and grad_out).
+bool scan_dtypes_supported(int in_dtype, int state_dtype);
 int scan_fwd(const void* x, const void* xg, const void* ag, const float* lam, void* h, int B, int T, int D,
-             int dtype, void* ws, size_t ws_bytes, hipStream_t st);
+             int in_dtype, int out_dtype, void* ws, size_t ws_bytes, hipStream_t st);
 int scan_bwd(const void* x, const void* xg, const void* ag, const float* lam, const void* hs, const void* gout,
-             void* dx, void* dxg, void* dag, float* dlam, int B, int T, int D, int dtype, void* ws,
-             size_t ws_bytes, hipStream_t st);
+             void* dx, void* dxg, void* dag, float* dlam, int B, int T, int D, int in_dtype, int state_dtype,
+             void* ws, size_t ws_bytes, hipStream_t st);
 
 // hawk_conv.hip
 int conv1d_fwd(const void* x, const float* w, const float* bias, const void* state, void* y, int B, int T, int D,

@@ -44,12 +44,6 @@ constexpr uint32_t kSpinLimit = 1u << 22;
 #ifndef HAWK_FWD_WAVES_PER_SIMD
 #define HAWK_FWD_WAVES_PER_SIMD 4
 #endif
-#ifndef HAWK_FWD_PERSISTENT
-#define HAWK_FWD_PERSISTENT 0
-#endif
-#ifndef HAWK_FWD_PREFETCH_ROWS
-#define HAWK_FWD_PREFETCH_ROWS 8
-#endif
 #ifndef HAWK_BWD_WAVES_PER_SIMD
 #define HAWK_BWD_WAVES_PER_SIMD 4
 #endif
@@ -206,13 +200,14 @@ __device__ __forceinline__ void combine_slices(float2 (*s_agg)[kWave * V], int w
 // ---------------------------------------------------------------------------------------
 // Forward tile.  FULL: every row of the tile is inside [0, T).
 // ---------------------------------------------------------------------------------------
-template <typename ET, int V, int TC, int NW, bool PRECISE, bool FULL>
-__device__ __forceinline__ void fwd_tile(const ET* __restrict__ x, const ET* __restrict__ xg,
-                                         const ET* __restrict__ ag, const float* __restrict__ lam,
-                                         ET* __restrict__ h, int B, int T, int D, int nseg, int seg, int b, int ct,
+template <typename IT, typename OT, int V, int TC, int NW, bool PRECISE, bool FULL>
+__device__ __forceinline__ void fwd_tile(const IT* __restrict__ x, const IT* __restrict__ xg,
+                                         const IT* __restrict__ ag, const float* __restrict__ lam,
+                                         OT* __restrict__ h, int B, int T, int D, int nseg, int seg, int b, int ct,
                                          uint32_t tag, const ScanWsPtrs& ws, float2 (*s_agg)[kWave * V],
                                          float2 (*s_prev)[kWave * V]) {
-    typedef typename Raw<ET, V>::type raw_t;
+    typedef typename Raw<IT, V>::type raw_t;
+    typedef typename Raw<OT, V>::type out_raw_t;
     constexpr int CT = kWave * V;
     constexpr int TS = NW * TC;
 
@@ -224,13 +219,15 @@ __device__ __forceinline__ void fwd_tile(const ET* __restrict__ x, const ET* __r
     const int t0 = seg * TS + w * TC;
     const size_t tile_off = ((size_t)b * T + t0) * D + c_tile;  // wave-uniform
     const int rows_in = FULL ? TC : __builtin_amdgcn_readfirstlane(min(max(T - t0, 0), TC));  // rows inside [0, T)
-    const uint32_t row_bytes = (uint32_t)D * sizeof(ET);
+    const uint32_t row_bytes = (uint32_t)D * sizeof(IT);
+    const uint32_t out_row_bytes = (uint32_t)D * sizeof(OT);
     const uint32_t slab = (uint32_t)rows_in * row_bytes;
-    const uint32_t lane_bytes = lane_off * sizeof(ET);
+    const uint32_t lane_bytes = lane_off * sizeof(IT);
     const rsrc_t bx = make_rsrc(x + tile_off, slab), bxg = make_rsrc(xg + tile_off, slab),
-                 bag = make_rsrc(ag + tile_off, slab), bh = make_rsrc(h + tile_off, slab);
+                 bag = make_rsrc(ag + tile_off, slab),
+                 bh = make_rsrc(h + tile_off, (uint32_t)rows_in * out_row_bytes);
     // idle lanes store at an offset beyond any slab, which the range check drops
-    const uint32_t store_bytes = lane_on ? lane_bytes : 0x80000000u;
+    const uint32_t store_bytes = lane_on ? lane_off * (uint32_t)sizeof(OT) : 0x80000000u;
 
     raw_t rx[TC], rxg[TC], rag[TC];
 #pragma unroll
@@ -252,7 +249,7 @@ __device__ __forceinline__ void fwd_tile(const ET* __restrict__ x, const ET* __r
     // 1. local scan from a zero state.  Kept per row: the local state (fp32) and the
     //    running product of alpha, which for bf16 activations with two channels per lane
     //    is stored as an fp16 pair (it only ever scales the carry).
-    constexpr bool PACK_P = (V == 2) && (sizeof(ET) == 2);
+    constexpr bool PACK_P = (V == 2) && (sizeof(OT) == 2);
     float hj[TC][V];
     float pj[PACK_P ? 1 : TC][V];
     uint32_t pjh[PACK_P ? TC : 1];
@@ -313,16 +310,16 @@ __device__ __forceinline__ void fwd_tile(const ET* __restrict__ x, const ET* __r
 #pragma unroll
             for (int v = 0; v < V; ++v) out[v] = fmaf(pj[j][v], cw[v], hj[j][v]);
         }
-        raw_t r;
+        out_raw_t r;
         pack(out, r);
-        buffer_store<raw_t>(r, bh, store_bytes, j * row_bytes);  // rows past T and idle lanes are dropped
+        buffer_store<out_raw_t>(r, bh, store_bytes, j * out_row_bytes);  // rows past T and idle lanes are dropped
     }
 }
 
-template <typename ET, int V, int TC, int NW, bool PRECISE>
+template <typename IT, typename OT, int V, int TC, int NW, bool PRECISE>
 __global__ __launch_bounds__(NW * kWave, HAWK_FWD_WAVES_PER_SIMD) void rglru_scan_fwd_kernel(
-    const ET* __restrict__ x, const ET* __restrict__ xg, const ET* __restrict__ ag,
-    const float* __restrict__ lam, ET* __restrict__ h, int B, int T, int D, int nseg, int nct,
+    const IT* __restrict__ x, const IT* __restrict__ xg, const IT* __restrict__ ag,
+    const float* __restrict__ lam, OT* __restrict__ h, int B, int T, int D, int nseg, int nct,
     ScanWsPtrs ws) {
     constexpr int CT = kWave * V;
     constexpr int TS = NW * TC;
@@ -339,294 +336,9 @@ __global__ __launch_bounds__(NW * kWave, HAWK_FWD_WAVES_PER_SIMD) void rglru_sca
     const int b = rem / nct;
     const int ct = rem - b * nct;
     if (seg * TS + TS <= T)
-        fwd_tile<ET, V, TC, NW, PRECISE, true>(x, xg, ag, lam, h, B, T, D, nseg, seg, b, ct, tag, ws, s_agg, s_prev);
+        fwd_tile<IT, OT, V, TC, NW, PRECISE, true>(x, xg, ag, lam, h, B, T, D, nseg, seg, b, ct, tag, ws, s_agg, s_prev);
     else
-        fwd_tile<ET, V, TC, NW, PRECISE, false>(x, xg, ag, lam, h, B, T, D, nseg, seg, b, ct, tag, ws, s_agg, s_prev);
-}
-
-// ---------------------------------------------------------------------------------------
-// Persistent forward kernel (used whenever the scan spans more than one tile in time).
-// The grid is sized to the number of workgroups the device holds at once; each workgroup
-// draws tiles from the ticket counter until they run out.  This allows software
-// pipelining at no register cost: the raw input registers of a tile are dead once its
-// local scan is done, so the next tile's loads are issued into them right away and fly
-// while this tile waits for its carry, applies it and stores.  The next ticket itself is
-// drawn at the top of the local scan, so its latency is hidden too.
-// ---------------------------------------------------------------------------------------
-struct TileCoord {
-    int seg, b, ct;
-};
-__device__ __forceinline__ TileCoord tile_coord(uint32_t ticket, int B, int nct) {
-    TileCoord t;
-    const int per_seg = B * nct;
-    t.seg = ticket / per_seg;
-    const int rem = ticket - t.seg * per_seg;
-    t.b = rem / nct;
-    t.ct = rem - t.b * nct;
-    return t;
-}
-
-// One draw from the control word.  `draws` is the number of draws the whole launch makes
-// (tiles + one terminating draw per workgroup); whoever makes the last one re-arms the word.
-__device__ __forceinline__ unsigned long long draw_ticket(unsigned long long* ctrl) {
-    return __hip_atomic_fetch_add(ctrl, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-__device__ __forceinline__ void rearm_if_last(unsigned long long* ctrl, uint32_t ticket, uint32_t draws) {
-    if (ticket == draws - 1u) {
-        __hip_atomic_fetch_add(ctrl, (1ull << 32) - (unsigned long long)draws, __ATOMIC_RELAXED,
-                               __HIP_MEMORY_SCOPE_AGENT);
-    }
-}
-
-template <typename ET, int V, int TC, int NW, bool PRECISE, bool FULL>
-__device__ __forceinline__ void fwd_local_scan(const typename Raw<ET, V>::type (&rx)[TC],
-                                               const typename Raw<ET, V>::type (&rxg)[TC],
-                                               const typename Raw<ET, V>::type (&rag)[TC], const float (&c2)[V],
-                                               const float (&cn)[V], int t0, int T, float (&pj)[TC][V],
-                                               float (&hj)[TC][V], float (&p_run)[V], float (&h_run)[V]) {
-#pragma unroll
-    for (int v = 0; v < V; ++v) { p_run[v] = 1.0f; h_run[v] = 0.0f; }
-#pragma unroll
-    for (int j = 0; j < TC; ++j) {
-        float fx[V], fxg[V], fag[V];
-        unpack(rx[j], fx);
-        unpack(rxg[j], fxg);
-        unpack(rag[j], fag);
-        const bool ok = FULL || (t0 + j < T);  // wave-uniform
-#pragma unroll
-        for (int v = 0; v < V; ++v) {
-            const float i = sigmoid_fast(fxg[v]);
-            const float r = sigmoid_fast(fag[v]);
-            float alpha = hw_exp2(c2[v] * r);
-            const float z = PRECISE ? one_minus_exp(cn[v] * r) : clamp01(fmaf(-alpha, alpha, 1.0f));
-            float beta = hw_sqrt(z) * (i * fx[v]);
-            if (!ok) { alpha = 1.0f; beta = 0.0f; }  // rows past T are the identity
-            h_run[v] = fmaf(alpha, h_run[v], beta);
-            p_run[v] *= alpha;
-            pj[j][v] = p_run[v];
-            hj[j][v] = h_run[v];
-        }
-        __builtin_amdgcn_sched_barrier(0);  // one row's temporaries live at a time
-    }
-}
-
-// RAGGED: T is not a multiple of the tile height, so rows past T must be neutralised.
-template <typename ET, int V, int TC, int NW, bool PRECISE, bool RAGGED>
-__global__ __launch_bounds__(NW * kWave, HAWK_FWD_WAVES_PER_SIMD) void rglru_scan_fwd_persistent_kernel(
-    const ET* __restrict__ x, const ET* __restrict__ xg, const ET* __restrict__ ag,
-    const float* __restrict__ lam, ET* __restrict__ h, int B, int T, int D, int nseg, int nct,
-    ScanWsPtrs ws, uint32_t total) {
-    typedef typename Raw<ET, V>::type raw_t;
-    constexpr int CT = kWave * V;
-    constexpr int TS = NW * TC;
-    __shared__ float2 s_agg[NW][CT];
-    __shared__ float2 s_prev[kLookback][CT];
-    __shared__ uint32_t s_tk[2];
-
-    const int lane = threadIdx.x & (kWave - 1);
-    const int w = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
-    const uint32_t draws = total + gridDim.x;
-    const uint32_t row_bytes = (uint32_t)D * sizeof(ET);
-    const size_t stride = (size_t)B * D;
-
-    if (threadIdx.x == 0) {
-        const unsigned long long v = draw_ticket(ws.ctrl);
-        rearm_if_last(ws.ctrl, (uint32_t)v, draws);
-        s_tk[0] = (uint32_t)v;
-        s_tk[1] = (uint32_t)(v >> 32) + 1u;
-    }
-    __syncthreads();
-    uint32_t cur = __builtin_amdgcn_readfirstlane(s_tk[0]);
-    const uint32_t tag = __builtin_amdgcn_readfirstlane(s_tk[1]);
-    if (cur >= total) return;
-
-    // geometry of the current tile, and its loads
-    TileCoord tc = tile_coord(cur, B, nct);
-    int c_tile = tc.ct * CT;
-    bool lane_on = c_tile + lane * V < D;
-    unsigned lane_off = lane_on ? lane * V : D - V - c_tile;  // idle lanes shadow the last valid channels
-    int t0 = tc.seg * TS + w * TC;
-    size_t tile_off = ((size_t)tc.b * T + t0) * D + c_tile;
-    int rows_in = __builtin_amdgcn_readfirstlane(min(max(T - t0, 0), TC));
-
-    // Rows [0, PF) of a tile are fetched ahead of time (while the previous tile finishes),
-    // rows [PF, TC) at the top of the tile's own turn; they arrive while the first rows are
-    // being scanned.  Prefetching everything would need TC more registers than there are.
-    constexpr int PF = HAWK_FWD_PREFETCH_ROWS < TC ? HAWK_FWD_PREFETCH_ROWS : TC;
-    raw_t rx[TC], rxg[TC], rag[TC];
-    rsrc_t bx, bxg, bag;
-    {
-        const uint32_t slab = (uint32_t)rows_in * row_bytes;
-        bx = make_rsrc(x + tile_off, slab);
-        bxg = make_rsrc(xg + tile_off, slab);
-        bag = make_rsrc(ag + tile_off, slab);
-#pragma unroll
-        for (int j = 0; j < PF; ++j) {
-            rx[j] = buffer_load<raw_t>(bx, lane_off * sizeof(ET), j * row_bytes);
-            rxg[j] = buffer_load<raw_t>(bxg, lane_off * sizeof(ET), j * row_bytes);
-            rag[j] = buffer_load<raw_t>(bag, lane_off * sizeof(ET), j * row_bytes);
-        }
-    }
-
-    while (true) {
-#pragma unroll
-        for (int j = PF; j < TC; ++j) {
-            rx[j] = buffer_load<raw_t>(bx, lane_off * sizeof(ET), j * row_bytes);
-            rxg[j] = buffer_load<raw_t>(bxg, lane_off * sizeof(ET), j * row_bytes);
-            rag[j] = buffer_load<raw_t>(bag, lane_off * sizeof(ET), j * row_bytes);
-        }
-        // next ticket: drawn now, looked at after the local scan
-        unsigned long long next_word = 0ull;
-        if (threadIdx.x == 0) next_word = draw_ticket(ws.ctrl);
-
-        float c2[V], cn[V];
-#pragma unroll
-        for (int v = 0; v < V; ++v) {
-            const float s = softplus_fast(lam[c_tile + lane_off + v]);
-            c2[v] = -8.0f * kLog2e * s;
-            cn[v] = -16.0f * s;
-        }
-
-        // 1. local scan from a zero state
-        float pj[TC][V], hj[TC][V], p_run[V], h_run[V];
-        fwd_local_scan<ET, V, TC, NW, PRECISE, !RAGGED>(rx, rxg, rag, c2, cn, t0, T, pj, hj, p_run, h_run);
-
-        // 2. combine the NW time slices; hand the next ticket to all waves
-#pragma unroll
-        for (int v = 0; v < V; ++v) s_agg[w][lane * V + v] = make_float2(p_run[v], h_run[v]);
-        if (threadIdx.x == 0) {
-            rearm_if_last(ws.ctrl, (uint32_t)next_word, draws);
-            s_tk[0] = (uint32_t)next_word;
-        }
-        __syncthreads();
-        const uint32_t nxt = __builtin_amdgcn_readfirstlane(s_tk[0]);
-        float pre_p[V], pre_h[V], tot_p[V], tot_h[V];
-        combine_slices<V, NW, false>(s_agg, w, lane, pre_p, pre_h, tot_p, tot_h);
-
-        // output view of the current tile (needed after the inputs' geometry is overwritten)
-        const rsrc_t bh = make_rsrc(h + tile_off, (uint32_t)rows_in * row_bytes);
-        const uint32_t store_bytes = lane_on ? lane_off * (uint32_t)sizeof(ET) : 0x80000000u;
-        const int pos = tc.seg;
-        const size_t idx_pos0 = (size_t)tc.b * D + c_tile + lane_off;
-
-        // 3a. publish this tile's aggregate, fetch the predecessors' words
-        const bool publishes = pos + 1 < nseg;
-        const size_t idx_self = idx_pos0 + (size_t)pos * stride;
-        if (w == 0 && publishes && !is_checkpoint(pos)) {
-#pragma unroll
-            for (int v = 0; v < V; ++v) {
-                publish(ws.agg_p + idx_self + v, tag, tot_p[v]);
-                publish(ws.agg_h + idx_self + v, tag, tot_h[v]);
-            }
-            asm volatile("" ::: "memory");
-        }
-        const int npred = (pos > 0) ? pos - checkpoint_before(pos) : 0;
-        const bool mine = w < npred;
-        const bool cp = (w == npred - 1);
-        const size_t idx_pred = idx_pos0 + (size_t)(mine ? pos - 1 - w : 0) * stride;
-        unsigned long long wp[V], wh[V];
-        if (mine) {
-#pragma unroll
-            for (int v = 0; v < V; ++v) {
-                wh[v] = __hip_atomic_load((cp ? ws.incl : ws.agg_h) + idx_pred + v, __ATOMIC_RELAXED,
-                                          __HIP_MEMORY_SCOPE_AGENT);
-                wp[v] = cp ? 0ull
-                           : __hip_atomic_load(ws.agg_p + idx_pred + v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            }
-        }
-
-        // 3b. the next tile's loads go out now, into the registers the local scan has freed
-        if (nxt < total) {
-            tc = tile_coord(nxt, B, nct);
-            c_tile = tc.ct * CT;
-            lane_on = c_tile + lane * V < D;
-            lane_off = lane_on ? lane * V : D - V - c_tile;
-            t0 = tc.seg * TS + w * TC;
-            tile_off = ((size_t)tc.b * T + t0) * D + c_tile;
-            rows_in = __builtin_amdgcn_readfirstlane(min(max(T - t0, 0), TC));
-            const uint32_t slab = (uint32_t)rows_in * row_bytes;
-            bx = make_rsrc(x + tile_off, slab);
-            bxg = make_rsrc(xg + tile_off, slab);
-            bag = make_rsrc(ag + tile_off, slab);
-#pragma unroll
-            for (int j = 0; j < PF; ++j) {
-                rx[j] = buffer_load<raw_t>(bx, lane_off * sizeof(ET), j * row_bytes);
-                rxg[j] = buffer_load<raw_t>(bxg, lane_off * sizeof(ET), j * row_bytes);
-                rag[j] = buffer_load<raw_t>(bag, lane_off * sizeof(ET), j * row_bytes);
-            }
-        }
-
-        // 3c. wait for the predecessors' words (bounded), stage them, fold
-        if (mine) {
-            float vp[V], vh[V];
-            uint32_t spins = 0;
-            while (true) {
-                bool ok = true;
-#pragma unroll
-                for (int v = 0; v < V; ++v) {
-                    ok &= (uint32_t)(wh[v] >> 32) == tag;
-                    vh[v] = __uint_as_float((uint32_t)wh[v]);
-                    if (cp) {
-                        vp[v] = 0.0f;
-                    } else {
-                        ok &= (uint32_t)(wp[v] >> 32) == tag;
-                        vp[v] = __uint_as_float((uint32_t)wp[v]);
-                    }
-                }
-                if (__all(ok)) break;
-                if (++spins > kSpinLimit) {
-                    __hip_atomic_store(reinterpret_cast<uint32_t*>(ws.ctrl) + 2, 1u, __ATOMIC_RELAXED,
-                                       __HIP_MEMORY_SCOPE_AGENT);
-#pragma unroll
-                    for (int v = 0; v < V; ++v) { vp[v] = 0.0f; vh[v] = 0.0f; }
-                    break;
-                }
-                __builtin_amdgcn_s_sleep(2);
-#pragma unroll
-                for (int v = 0; v < V; ++v) {
-                    wh[v] = __hip_atomic_load((cp ? ws.incl : ws.agg_h) + idx_pred + v, __ATOMIC_RELAXED,
-                                              __HIP_MEMORY_SCOPE_AGENT);
-                    wp[v] = cp ? 0ull
-                               : __hip_atomic_load(ws.agg_p + idx_pred + v, __ATOMIC_RELAXED,
-                                                   __HIP_MEMORY_SCOPE_AGENT);
-                }
-            }
-#pragma unroll
-            for (int v = 0; v < V; ++v) s_prev[w][lane * V + v] = make_float2(vp[v], vh[v]);
-        }
-        __syncthreads();
-        float cin[V];
-#pragma unroll
-        for (int v = 0; v < V; ++v) cin[v] = 0.0f;
-        for (int k = npred - 1; k >= 0; --k) {
-#pragma unroll
-            for (int v = 0; v < V; ++v) {
-                const float2 a = s_prev[k][lane * V + v];
-                cin[v] = fmaf(a.x, cin[v], a.y);
-            }
-        }
-        if (w == 0 && publishes && is_checkpoint(pos)) {
-#pragma unroll
-            for (int v = 0; v < V; ++v) publish(ws.incl + idx_self + v, tag, fmaf(tot_p[v], cin[v], tot_h[v]));
-        }
-
-        // 4. apply the carry and store
-        float cw[V];
-#pragma unroll
-        for (int v = 0; v < V; ++v) cw[v] = fmaf(pre_p[v], cin[v], pre_h[v]);
-#pragma unroll
-        for (int j = 0; j < TC; ++j) {
-            float out[V];
-#pragma unroll
-            for (int v = 0; v < V; ++v) out[v] = fmaf(pj[j][v], cw[v], hj[j][v]);
-            raw_t r;
-            pack(out, r);
-            buffer_store<raw_t>(r, bh, store_bytes, j * row_bytes);  // rows past T and idle lanes are dropped
-        }
-
-        if (nxt >= total) break;
-        cur = nxt;
-    }
+        fwd_tile<IT, OT, V, TC, NW, PRECISE, false>(x, xg, ag, lam, h, B, T, D, nseg, seg, b, ct, tag, ws, s_agg, s_prev);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -639,15 +351,16 @@ __global__ __launch_bounds__(NW * kWave, HAWK_FWD_WAVES_PER_SIMD) void rglru_sca
 //   da_rg_lru = dlog_a r (1-r) (-8 softplus(Lambda));  dLambda += dlog_a r  (scaled per channel later)
 // FULL: every row of the tile is inside [1, T) (row 0 has no h_{t-1}).
 // ---------------------------------------------------------------------------------------
-template <typename ET, int V, int TC, int NW, bool PRECISE, bool FULL>
-__device__ __forceinline__ void bwd_tile(const ET* __restrict__ x, const ET* __restrict__ xg,
-                                         const ET* __restrict__ ag, const float* __restrict__ lam,
-                                         const ET* __restrict__ hs, const ET* __restrict__ gout,
-                                         ET* __restrict__ dx, ET* __restrict__ dxg, ET* __restrict__ dag, int B,
+template <typename IT, typename ST, int V, int TC, int NW, bool PRECISE, bool FULL>
+__device__ __forceinline__ void bwd_tile(const IT* __restrict__ x, const IT* __restrict__ xg,
+                                         const IT* __restrict__ ag, const float* __restrict__ lam,
+                                         const ST* __restrict__ hs, const ST* __restrict__ gout,
+                                         IT* __restrict__ dx, IT* __restrict__ dxg, IT* __restrict__ dag, int B,
                                          int T, int D, int nseg, int seg, int pos, int b, int ct, uint32_t tag,
                                          const ScanWsPtrs& ws, float2 (*s_agg)[kWave * V],
                                          float2 (*s_prev)[kWave * V], float (*s_dl)[kWave * V]) {
-    typedef typename Raw<ET, V>::type raw_t;
+    typedef typename Raw<IT, V>::type raw_t;      // x, x_rg_lru, a_rg_lru and the three gradients
+    typedef typename Raw<ST, V>::type sraw_t;     // saved h and grad_out
     constexpr int CT = kWave * V;
     constexpr int TS = NW * TC;
 
@@ -659,15 +372,18 @@ __device__ __forceinline__ void bwd_tile(const ET* __restrict__ x, const ET* __r
     const int t0 = seg * TS + w * TC;
     const size_t tile_off = ((size_t)b * T + t0) * D + c_tile;
     const int rows_in = FULL ? TC : __builtin_amdgcn_readfirstlane(min(max(T - t0, 0), TC));
-    const uint32_t row_bytes = (uint32_t)D * sizeof(ET);
+    const uint32_t row_bytes = (uint32_t)D * sizeof(IT);
+    const uint32_t srow_bytes = (uint32_t)D * sizeof(ST);
     const uint32_t slab = (uint32_t)rows_in * row_bytes;
-    const uint32_t lane_bytes = lane_off * sizeof(ET);
+    const uint32_t lane_bytes = lane_off * sizeof(IT);
+    const uint32_t slane_bytes = lane_off * sizeof(ST);
     const rsrc_t bx = make_rsrc(x + tile_off, slab), bxg = make_rsrc(xg + tile_off, slab),
-                 bag = make_rsrc(ag + tile_off, slab), bgo = make_rsrc(gout + tile_off, slab),
-                 bhs = make_rsrc(hs + tile_off, slab);
+                 bag = make_rsrc(ag + tile_off, slab),
+                 bgo = make_rsrc(gout + tile_off, (uint32_t)rows_in * srow_bytes),
+                 bhs = make_rsrc(hs + tile_off, (uint32_t)rows_in * srow_bytes);
     // h_{t-1} of the slice's first row lives one row before the slab; absent at t = 0
     const bool has_prev = FULL || (t0 > 0 && rows_in > 0);
-    const rsrc_t bhm1 = make_rsrc(has_prev ? hs + tile_off - D : hs, has_prev ? row_bytes : 0u);
+    const rsrc_t bhm1 = make_rsrc(has_prev ? hs + tile_off - D : hs, has_prev ? srow_bytes : 0u);
     const rsrc_t bdx = make_rsrc(dx + tile_off, slab), bdxg = make_rsrc(dxg + tile_off, slab),
                  bdag = make_rsrc(dag + tile_off, slab);
     // idle lanes store at an offset beyond any slab, which the range check drops
@@ -676,11 +392,12 @@ __device__ __forceinline__ void bwd_tile(const ET* __restrict__ x, const ET* __r
     // The local pass needs only a_rg_lru and grad_out; x, x_rg_lru and h are fetched after
     // it (their registers would otherwise sit idle through it) and arrive during the carry
     // exchange.  This is what lets a lane own TC rows within 128 registers.
-    raw_t rx[TC], rxg[TC], rag[TC], rgo[TC], rhp[TC];
+    raw_t rx[TC], rxg[TC], rag[TC];
+    sraw_t rgo[TC], rhp[TC];
 #pragma unroll
     for (int j = 0; j < TC; ++j) {
         rag[j] = buffer_load<raw_t>(bag, lane_bytes, j * row_bytes);
-        rgo[j] = buffer_load<raw_t>(bgo, lane_bytes, j * row_bytes);
+        rgo[j] = buffer_load<sraw_t>(bgo, slane_bytes, j * srow_bytes);
     }
 
     float c2[V], cs[V];
@@ -695,7 +412,7 @@ __device__ __forceinline__ void bwd_tile(const ET* __restrict__ x, const ET* __r
     //    is kept; everything else is evaluated after the carry is known.
     // r is kept as an fp16 pair for bf16 activations (2^-11 relative, well inside the bf16
     // rounding of the gradients), in fp32 otherwise.
-    constexpr bool PACK_R = (V == 2) && (sizeof(ET) == 2);
+    constexpr bool PACK_R = (V == 2) && (sizeof(IT) == 2);
     float rr[PACK_R ? 1 : TC][V];
     uint32_t rrh[PACK_R ? TC : 1];
     float q_run[V], c_run[V];
@@ -729,8 +446,8 @@ __device__ __forceinline__ void bwd_tile(const ET* __restrict__ x, const ET* __r
     for (int j = 0; j < TC; ++j) {
         rx[j] = buffer_load<raw_t>(bx, lane_bytes, j * row_bytes);
         rxg[j] = buffer_load<raw_t>(bxg, lane_bytes, j * row_bytes);
-        rhp[j] = (j == 0) ? buffer_load<raw_t>(bhm1, lane_bytes, 0u)
-                          : buffer_load<raw_t>(bhs, lane_bytes, (j - 1) * row_bytes);
+        rhp[j] = (j == 0) ? buffer_load<sraw_t>(bhm1, slane_bytes, 0u)
+                          : buffer_load<sraw_t>(bhs, slane_bytes, (j - 1) * srow_bytes);
     }
     __builtin_amdgcn_sched_barrier(0);
 
@@ -763,7 +480,7 @@ __device__ __forceinline__ void bwd_tile(const ET* __restrict__ x, const ET* __r
         float fx[V], fxg[V], fgo[V], fhp[V];
         unpack(rx[j], fx);
         unpack(rxg[j], fxg);
-        if constexpr (sizeof(raw_t) == 4 && sizeof(ET) == 2) {
+        if constexpr (sizeof(sraw_t) == 4 && sizeof(ST) == 2) {
             // unpack again rather than keep the local pass's floats alive across the exchange
             unpack(opaque(rgo[j]), fgo);
         } else {
@@ -820,11 +537,11 @@ __device__ __forceinline__ void bwd_tile(const ET* __restrict__ x, const ET* __r
     }
 }
 
-template <typename ET, int V, int TC, int NW, bool PRECISE>
+template <typename IT, typename ST, int V, int TC, int NW, bool PRECISE>
 __global__ __launch_bounds__(NW * kWave, HAWK_BWD_WAVES_PER_SIMD) void rglru_scan_bwd_kernel(
-    const ET* __restrict__ x, const ET* __restrict__ xg, const ET* __restrict__ ag,
-    const float* __restrict__ lam, const ET* __restrict__ hs, const ET* __restrict__ gout,
-    ET* __restrict__ dx, ET* __restrict__ dxg, ET* __restrict__ dag, int B, int T, int D, int nseg,
+    const IT* __restrict__ x, const IT* __restrict__ xg, const IT* __restrict__ ag,
+    const float* __restrict__ lam, const ST* __restrict__ hs, const ST* __restrict__ gout,
+    IT* __restrict__ dx, IT* __restrict__ dxg, IT* __restrict__ dag, int B, int T, int D, int nseg,
     int nct, ScanWsPtrs ws) {
     constexpr int CT = kWave * V;
     constexpr int TS = NW * TC;
@@ -843,10 +560,10 @@ __global__ __launch_bounds__(NW * kWave, HAWK_BWD_WAVES_PER_SIMD) void rglru_sca
     const int b = rem / nct;
     const int ct = rem - b * nct;
     if (seg > 0 && seg * TS + TS <= T)
-        bwd_tile<ET, V, TC, NW, PRECISE, true>(x, xg, ag, lam, hs, gout, dx, dxg, dag, B, T, D, nseg, seg, pos, b,
+        bwd_tile<IT, ST, V, TC, NW, PRECISE, true>(x, xg, ag, lam, hs, gout, dx, dxg, dag, B, T, D, nseg, seg, pos, b,
                                                ct, tag, ws, s_agg, s_prev, s_dl);
     else
-        bwd_tile<ET, V, TC, NW, PRECISE, false>(x, xg, ag, lam, hs, gout, dx, dxg, dag, B, T, D, nseg, seg, pos, b,
+        bwd_tile<IT, ST, V, TC, NW, PRECISE, false>(x, xg, ag, lam, hs, gout, dx, dxg, dag, B, T, D, nseg, seg, pos, b,
                                                 ct, tag, ws, s_agg, s_prev, s_dl);
 }
 
@@ -955,47 +672,25 @@ ScanWsPtrs carve(void* ws, const WsLayout& l) {
     return r;
 }
 
-// Workgroups the device holds at once for a kernel (CUs x resident workgroups per CU).
-template <typename K>
-unsigned resident_workgroups(K kernel, int block_threads) {
-    int dev = 0, cus = 0, per_cu = 0;
-    if (hipGetDevice(&dev) != hipSuccess) return 0;
-    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, block_threads, 0) != hipSuccess) return 0;
-    return (unsigned)(cus > 0 && per_cu > 0 ? cus * per_cu : 0);
-}
-
-template <typename ET, int V, int TC, int NW, bool PRECISE>
+template <typename IT, typename OT, int V, int TC, int NW, bool PRECISE>
 int launch_fwd(const void* x, const void* xg, const void* ag, const float* lam, void* h, int B, int T,
                int D, int nseg, int nct, ScanWsPtrs ws, hipStream_t st) {
-    const unsigned total = (unsigned)nseg * B * nct;
-    if (HAWK_FWD_PERSISTENT && nseg > 1) {
-        const bool ragged = (T % (TC * NW)) != 0;
-        auto kernel = ragged ? rglru_scan_fwd_persistent_kernel<ET, V, TC, NW, PRECISE, true>
-                             : rglru_scan_fwd_persistent_kernel<ET, V, TC, NW, PRECISE, false>;
-        unsigned grid = resident_workgroups(kernel, NW * kWave);
-        if (grid == 0) return HAWK_ERR_LAUNCH;
-        if (grid > total) grid = total;
-        hipLaunchKernelGGL(kernel, dim3(grid), dim3(NW * kWave), 0, st, static_cast<const ET*>(x),
-                           static_cast<const ET*>(xg), static_cast<const ET*>(ag), lam, static_cast<ET*>(h), B, T, D,
-                           nseg, nct, ws, total);
-        return hipGetLastError() == hipSuccess ? HAWK_OK : HAWK_ERR_LAUNCH;
-    }
-    hipLaunchKernelGGL((rglru_scan_fwd_kernel<ET, V, TC, NW, PRECISE>), dim3(total), dim3(NW * kWave), 0, st,
-                       static_cast<const ET*>(x), static_cast<const ET*>(xg), static_cast<const ET*>(ag), lam,
-                       static_cast<ET*>(h), B, T, D, nseg, nct, ws);
+    const unsigned grid = (unsigned)nseg * B * nct;
+    hipLaunchKernelGGL((rglru_scan_fwd_kernel<IT, OT, V, TC, NW, PRECISE>), dim3(grid), dim3(NW * kWave), 0, st,
+                       static_cast<const IT*>(x), static_cast<const IT*>(xg), static_cast<const IT*>(ag), lam,
+                       static_cast<OT*>(h), B, T, D, nseg, nct, ws);
     return hipGetLastError() == hipSuccess ? HAWK_OK : HAWK_ERR_LAUNCH;
 }
 
-template <typename ET, int V, int TC, int NW, bool PRECISE>
+template <typename IT, typename ST, int V, int TC, int NW, bool PRECISE>
 int launch_bwd(const void* x, const void* xg, const void* ag, const float* lam, const void* hs,
                const void* gout, void* dx, void* dxg, void* dag, int B, int T, int D, int nseg, int nct,
                ScanWsPtrs ws, hipStream_t st) {
     const unsigned grid = (unsigned)nseg * B * nct;
-    hipLaunchKernelGGL((rglru_scan_bwd_kernel<ET, V, TC, NW, PRECISE>), dim3(grid), dim3(NW * kWave), 0, st,
-                       static_cast<const ET*>(x), static_cast<const ET*>(xg), static_cast<const ET*>(ag), lam,
-                       static_cast<const ET*>(hs), static_cast<const ET*>(gout), static_cast<ET*>(dx),
-                       static_cast<ET*>(dxg), static_cast<ET*>(dag), B, T, D, nseg, nct, ws);
+    hipLaunchKernelGGL((rglru_scan_bwd_kernel<IT, ST, V, TC, NW, PRECISE>), dim3(grid), dim3(NW * kWave), 0, st,
+                       static_cast<const IT*>(x), static_cast<const IT*>(xg), static_cast<const IT*>(ag), lam,
+                       static_cast<const ST*>(hs), static_cast<const ST*>(gout), static_cast<IT*>(dx),
+                       static_cast<IT*>(dxg), static_cast<IT*>(dag), B, T, D, nseg, nct, ws);
     return hipGetLastError() == hipSuccess ? HAWK_OK : HAWK_ERR_LAUNCH;
 }
 
@@ -1025,9 +720,14 @@ int workspace_status(const void* ws, hipStream_t st, int* flag) {
     return HAWK_OK;
 }
 
+bool scan_dtypes_supported(int in_dtype, int state_dtype) {
+    if (in_dtype == HAWK_DTYPE_BF16) return state_dtype == HAWK_DTYPE_BF16;
+    return in_dtype == HAWK_DTYPE_F32 && (state_dtype == HAWK_DTYPE_F32 || state_dtype == HAWK_DTYPE_BF16);
+}
+
 int scan_fwd(const void* x, const void* xg, const void* ag, const float* lam, void* h, int B, int T, int D,
-             int dtype, void* ws, size_t ws_bytes, hipStream_t st) {
-    const TileShape s = fwd_shape(D, dtype);
+             int in_dtype, int out_dtype, void* ws, size_t ws_bytes, hipStream_t st) {
+    const TileShape s = fwd_shape(D, in_dtype);
     const int nseg = ceil_div(T, s.rows());
     const int nct = ceil_div(D, s.chans());
     ScanWsPtrs p = {};
@@ -1036,34 +736,39 @@ int scan_fwd(const void* x, const void* xg, const void* ag, const float* lam, vo
         if (ws == nullptr || ws_bytes < l.total) return HAWK_ERR_WORKSPACE;
         p = carve(ws, l);
     }
-    if (dtype == HAWK_DTYPE_BF16) {
+    if (in_dtype == HAWK_DTYPE_BF16) {
         if (s.V == 2)
-            return launch_fwd<bf16_t, 2, kFwdTC, kFwdNW, false>(x, xg, ag, lam, h, B, T, D, nseg, nct, p, st);
-        return launch_fwd<bf16_t, 1, kFwdTC, kFwdNW, false>(x, xg, ag, lam, h, B, T, D, nseg, nct, p, st);
+            return launch_fwd<bf16_t, bf16_t, 2, kFwdTC, kFwdNW, false>(x, xg, ag, lam, h, B, T, D, nseg, nct, p, st);
+        return launch_fwd<bf16_t, bf16_t, 1, kFwdTC, kFwdNW, false>(x, xg, ag, lam, h, B, T, D, nseg, nct, p, st);
     }
-    return launch_fwd<float, 1, kFwdTC, kFwdNW, true>(x, xg, ag, lam, h, B, T, D, nseg, nct, p, st);
+    if (out_dtype == HAWK_DTYPE_BF16)
+        return launch_fwd<float, bf16_t, 1, kFwdTC, kFwdNW, false>(x, xg, ag, lam, h, B, T, D, nseg, nct, p, st);
+    return launch_fwd<float, float, 1, kFwdTC, kFwdNW, true>(x, xg, ag, lam, h, B, T, D, nseg, nct, p, st);
 }
 
 int scan_bwd(const void* x, const void* xg, const void* ag, const float* lam, const void* hs, const void* gout,
-             void* dx, void* dxg, void* dag, float* dlam, int B, int T, int D, int dtype, void* ws,
-             size_t ws_bytes, hipStream_t st) {
-    const TileShape s = bwd_shape(D, dtype);
+             void* dx, void* dxg, void* dag, float* dlam, int B, int T, int D, int in_dtype, int state_dtype,
+             void* ws, size_t ws_bytes, hipStream_t st) {
+    const TileShape s = bwd_shape(D, in_dtype);
     const int nseg = ceil_div(T, s.rows());
     const int nct = ceil_div(D, s.chans());
     const WsLayout l = layout_for(B, D, nseg, nseg);
     if (ws == nullptr || ws_bytes < l.total) return HAWK_ERR_WORKSPACE;
     const ScanWsPtrs p = carve(ws, l);
     int rc;
-    if (dtype == HAWK_DTYPE_BF16) {
+    if (in_dtype == HAWK_DTYPE_BF16) {
         if (s.V == 2)
-            rc = launch_bwd<bf16_t, 2, kBwdTC, kBwdNW, false>(x, xg, ag, lam, hs, gout, dx, dxg, dag, B, T, D, nseg,
-                                                              nct, p, st);
+            rc = launch_bwd<bf16_t, bf16_t, 2, kBwdTC, kBwdNW, false>(x, xg, ag, lam, hs, gout, dx, dxg, dag, B, T, D,
+                                                                      nseg, nct, p, st);
         else
-            rc = launch_bwd<bf16_t, 1, kBwdTC, kBwdNW, false>(x, xg, ag, lam, hs, gout, dx, dxg, dag, B, T, D, nseg,
-                                                              nct, p, st);
+            rc = launch_bwd<bf16_t, bf16_t, 1, kBwdTC, kBwdNW, false>(x, xg, ag, lam, hs, gout, dx, dxg, dag, B, T, D,
+                                                                      nseg, nct, p, st);
+    } else if (state_dtype == HAWK_DTYPE_BF16) {
+        rc = launch_bwd<float, bf16_t, 1, kBwdTC, kBwdNW, false>(x, xg, ag, lam, hs, gout, dx, dxg, dag, B, T, D, nseg,
+                                                                 nct, p, st);
     } else {
-        rc = launch_bwd<float, 1, kBwdTC, kBwdNW, true>(x, xg, ag, lam, hs, gout, dx, dxg, dag, B, T, D, nseg, nct, p,
-                                                        st);
+        rc = launch_bwd<float, float, 1, kBwdTC, kBwdNW, true>(x, xg, ag, lam, hs, gout, dx, dxg, dag, B, T, D, nseg,
+                                                               nct, p, st);
     }
     if (rc != HAWK_OK) return rc;
     hipLaunchKernelGGL(dlam_reduce_kernel, dim3((unsigned)ceil_div(D, kWave)), dim3(1024), 0, st, p.dlam_part, lam,

@@ -10,6 +10,9 @@ Public surface mirrors the upstream operator boundary (hawk/scan_fused.py:319-44
 
 Differences from upstream, all deliberate:
 
+* Under autocast, fp32 activations are NOT first cast to bf16 by three extra kernels
+  (upstream: ``custom_fwd(cast_inputs=bfloat16)``, scan_fused.py:428): mixed-precision
+  kernels read fp32, keep fp32 state, write bf16 ``h``, and return fp32 gradients.
 * Lambda (``a_param``) and its gradient stay fp32 even under autocast (upstream's
   ``custom_fwd(cast_inputs=bfloat16)`` rounds Lambda to bf16 too, scan_fused.py:428).
 * fp32 activations are stored as fp32 (upstream rounds every store through bf16,
@@ -37,21 +40,22 @@ def _prepare(*tensors: torch.Tensor):
     return tuple(t if t.is_contiguous() else t.contiguous() for t in tensors)
 
 
-def _launch_scan_fwd(x, x_rg_lru, a_rg_lru, a_param) -> torch.Tensor:
+def _launch_scan_fwd(x, x_rg_lru, a_rg_lru, a_param, h_bf16: bool) -> torch.Tensor:
     dev = _lib.require_cuda(x, x_rg_lru, a_rg_lru, a_param)
     x, x_rg_lru, a_rg_lru, a_param = (_lib.dense16(t) for t in (x, x_rg_lru, a_rg_lru, a_param))
     b, sq, d = x.shape
-    code = _lib.dtype_code(x.dtype)
+    in_code = _lib.dtype_code(x.dtype)
+    out_dtype = torch.bfloat16 if h_bf16 else x.dtype
     lib = _lib.load()
-    h = torch.empty_like(x)
-    nbytes = lib.hawk_scan_workspace_bytes(b, sq, d, code)
+    h = torch.empty((b, sq, d), dtype=out_dtype, device=dev)
+    nbytes = lib.hawk_scan_workspace_bytes(b, sq, d, in_code)
     ws = _lib.scan_workspace(dev, nbytes)
     with torch.cuda.device(dev):
-        status = lib.hawk_rglru_scan_fwd(
+        status = lib.hawk_rglru_scan_fwd_mixed(
             x.data_ptr(), x_rg_lru.data_ptr(), a_rg_lru.data_ptr(), a_param.data_ptr(), h.data_ptr(),
-            b, sq, d, code, ws.data_ptr(), ws.numel(), _lib.stream_ptr(dev),
+            b, sq, d, in_code, _lib.dtype_code(out_dtype), ws.data_ptr(), ws.numel(), _lib.stream_ptr(dev),
         )
-    _lib.check("hawk_rglru_scan_fwd", status)
+    _lib.check("hawk_rglru_scan_fwd_mixed", status)
     return h
 
 
@@ -61,37 +65,41 @@ def _launch_scan_bwd(x, x_rg_lru, a_rg_lru, a_param, h_saved, grad_out):
         _lib.dense16(t) for t in (x, x_rg_lru, a_rg_lru, a_param, h_saved, grad_out)
     )
     b, sq, d = x.shape
-    code = _lib.dtype_code(x.dtype)
+    in_code = _lib.dtype_code(x.dtype)
     lib = _lib.load()
     dx = torch.empty_like(x)
     dxg = torch.empty_like(x)
     dag = torch.empty_like(x)
     dlam = torch.empty(d, dtype=torch.float32, device=dev)
-    nbytes = lib.hawk_scan_workspace_bytes(b, sq, d, code)
+    nbytes = lib.hawk_scan_workspace_bytes(b, sq, d, in_code)
     ws = _lib.scan_workspace(dev, nbytes)
     with torch.cuda.device(dev):
-        status = lib.hawk_rglru_scan_bwd(
+        status = lib.hawk_rglru_scan_bwd_mixed(
             x.data_ptr(), x_rg_lru.data_ptr(), a_rg_lru.data_ptr(), a_param.data_ptr(),
             h_saved.data_ptr(), grad_out.data_ptr(), dx.data_ptr(), dxg.data_ptr(), dag.data_ptr(),
-            dlam.data_ptr(), b, sq, d, code, ws.data_ptr(), ws.numel(), _lib.stream_ptr(dev),
+            dlam.data_ptr(), b, sq, d, in_code, _lib.dtype_code(h_saved.dtype),
+            ws.data_ptr(), ws.numel(), _lib.stream_ptr(dev),
         )
-    _lib.check("hawk_rglru_scan_bwd", status)
+    _lib.check("hawk_rglru_scan_bwd_mixed", status)
     return dx, dxg, dag, dlam
 
 
 # ---------------------------------------------------------------------------------------
-# torch.library registration (opaque to Dynamo, with shape/dtype propagation rules)
+# torch.library registration (opaque to Dynamo, with shape/dtype propagation rules).
+# x, x_rg_lru, a_rg_lru share a dtype (bf16 or fp32); h is bf16 when h_bf16 is set, else
+# that same dtype; in the backward h_saved and grad_out share h's dtype and the three
+# activation gradients come back in the inputs' dtype.
 # ---------------------------------------------------------------------------------------
 @torch.library.custom_op("hawk_amd::rglru_scan_fwd", mutates_args=(), device_types="cuda")
 def _rglru_scan_fwd_op(
-    x: torch.Tensor, x_rg_lru: torch.Tensor, a_rg_lru: torch.Tensor, a_param: torch.Tensor
+    x: torch.Tensor, x_rg_lru: torch.Tensor, a_rg_lru: torch.Tensor, a_param: torch.Tensor, h_bf16: bool
 ) -> torch.Tensor:
-    return _launch_scan_fwd(x, x_rg_lru, a_rg_lru, a_param)
+    return _launch_scan_fwd(x, x_rg_lru, a_rg_lru, a_param, h_bf16)
 
 
 @_rglru_scan_fwd_op.register_fake
-def _(x, x_rg_lru, a_rg_lru, a_param):
-    return torch.empty_like(x, memory_format=torch.contiguous_format)
+def _(x, x_rg_lru, a_rg_lru, a_param, h_bf16):
+    return torch.empty(x.shape, dtype=torch.bfloat16 if h_bf16 else x.dtype, device=x.device)
 
 
 @torch.library.custom_op("hawk_amd::rglru_scan_bwd", mutates_args=(), device_types="cuda")
@@ -134,16 +142,21 @@ def sequential_scan_forward(
     x_rg_lru: torch.Tensor,
     a_rg_lru: torch.Tensor,  # [b,sq,d]
     a_param: torch.Tensor,  # [d]
+    out_dtype: torch.dtype | None = None,
 ) -> torch.Tensor:
     """Forward pass of the RG-LRU scan (drop-in for hawk/scan_fused.py:319-360).
 
     Non-contiguous inputs are silently copied, as upstream does; D must be a multiple of
     64, as upstream asserts.  ``a_param`` is used in fp32 whatever dtype it arrives in.
+    ``out_dtype=torch.bfloat16`` with fp32 inputs selects the mixed-precision kernel
+    (fp32 read, bf16 h) that replaces upstream's cast-then-scan sequence.
     """
     _check_shapes(x, x_rg_lru, a_rg_lru, a_param)
     x, x_rg_lru, a_rg_lru = _prepare(x, x_rg_lru, a_rg_lru)
     a_param = a_param.float().contiguous()
-    return _rglru_scan_fwd_op(x, x_rg_lru, a_rg_lru, a_param)
+    h_bf16 = out_dtype == torch.bfloat16 or (out_dtype is None and x.dtype == torch.bfloat16)
+    assert out_dtype in (None, x.dtype, torch.bfloat16), f"unsupported h dtype {out_dtype} for {x.dtype} inputs"
+    return _rglru_scan_fwd_op(x, x_rg_lru, a_rg_lru, a_param, h_bf16)
 
 
 def sequential_scan_backward(
@@ -156,8 +169,10 @@ def sequential_scan_backward(
 ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
     """Backward pass of the RG-LRU scan (drop-in for hawk/scan_fused.py:363-424).
 
-    Returns (dx, dx_rg_lru, da_rg_lru, da_param[D]); da_param is fp32 and already summed
-    over the batch.  A non-contiguous ``grad_out`` is copied with a warning, as upstream.
+    Returns (dx, dx_rg_lru, da_rg_lru, da_param[D]); the three activation gradients have
+    the dtype of the saved inputs, da_param is fp32 and already summed over the batch.
+    ``h_saved`` may be bf16 while the inputs are fp32 (mixed-precision forward).  A
+    non-contiguous ``grad_out`` is copied with a warning, as upstream.
     """
     _check_shapes(x_saved, x_rg_lru_saved, a_rg_lru_saved, a_param_saved)
     assert h_saved.shape == x_saved.shape and grad_out.shape == x_saved.shape
@@ -167,10 +182,10 @@ def sequential_scan_backward(
             "`grad_out` tensor is not contiguous. Setting to contiguous and attempting to continue. "
             "This may impact runtime."
         )
-    if grad_out.dtype != x_saved.dtype:
-        grad_out = grad_out.to(x_saved.dtype)
-    if h_saved.dtype != x_saved.dtype:
+    if h_saved.dtype not in (x_saved.dtype, torch.bfloat16):
         h_saved = h_saved.to(x_saved.dtype)
+    if grad_out.dtype != h_saved.dtype:
+        grad_out = grad_out.to(h_saved.dtype)
     x_saved, x_rg_lru_saved, a_rg_lru_saved, h_saved, grad_out = _prepare(
         x_saved, x_rg_lru_saved, a_rg_lru_saved, h_saved, grad_out
     )
@@ -178,13 +193,10 @@ def sequential_scan_backward(
     return _rglru_scan_bwd_op(x_saved, x_rg_lru_saved, a_rg_lru_saved, a_param_saved, h_saved, grad_out)
 
 
-def _activation_dtype(x: torch.Tensor) -> torch.dtype:
-    """dtype the scan runs in: bf16 under CUDA autocast (as upstream's custom_fwd), else
-    bf16 or fp32 as given; other floating dtypes are computed in fp32."""
-    if torch.is_autocast_enabled("cuda"):
+def _common_input_dtype(*tensors: torch.Tensor) -> torch.dtype:
+    """bf16 only if every activation already is bf16; fp32 otherwise (fp16/fp64 compute in fp32)."""
+    if all(t.dtype == torch.bfloat16 for t in tensors):
         return torch.bfloat16
-    if x.dtype in (torch.bfloat16, torch.float32):
-        return x.dtype
     return torch.float32
 
 
@@ -192,19 +204,22 @@ class DiagonalRecurrence(Function):
     """h = scan(x, x_rg_lru, a_rg_lru, a_param) with the hand-written reverse-time backward.
 
     Same four positional tensor arguments and four gradients as upstream
-    (hawk/scan_fused.py:426-442).  Under CUDA autocast the three activation tensors are
-    cast to bf16, which is what upstream's ``custom_fwd(cast_inputs=torch.bfloat16)`` does
-    to them; Lambda is kept in fp32.
+    (hawk/scan_fused.py:426-442).  Under CUDA autocast h is bf16, as with upstream's
+    ``custom_fwd(cast_inputs=torch.bfloat16)``, but fp32 activations are not cast first:
+    the mixed-precision kernels read them as fp32 and round in registers, and the backward
+    writes their gradients directly in fp32.  Lambda is always used in fp32.
     """
 
     @staticmethod
     def forward(ctx, x, x_rg_lru, a_rg_lru, a_param) -> torch.Tensor:
-        run_dtype = _activation_dtype(x)
-        out_dtype = run_dtype if run_dtype == torch.bfloat16 or x.dtype == torch.float32 else x.dtype
-        xc, xgc, agc = (t.to(run_dtype) for t in (x, x_rg_lru, a_rg_lru))
-        h = sequential_scan_forward(xc, xgc, agc, a_param)
+        in_dtype = _common_input_dtype(x, x_rg_lru, a_rg_lru)
+        xc, xgc, agc = (t if t.dtype == in_dtype else t.to(in_dtype) for t in (x, x_rg_lru, a_rg_lru))
+        autocast = torch.is_autocast_enabled("cuda")
+        h = sequential_scan_forward(xc, xgc, agc, a_param, torch.bfloat16 if autocast else None)
         ctx.save_for_backward(xc, xgc, agc, a_param, h)
-        return h if h.dtype == out_dtype else h.to(out_dtype)
+        if not autocast and x.dtype not in (torch.bfloat16, torch.float32):
+            return h.to(x.dtype)
+        return h
 
     @staticmethod
     def backward(ctx, grad_output):  # type: ignore[override]

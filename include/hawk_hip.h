@@ -84,6 +84,24 @@ int hawk_rglru_scan_bwd(const void* x, const void* x_rg_lru, const void* a_rg_lr
                         int T, int D, int dtype, void* workspace_device,
                         size_t workspace_bytes, void* stream);
 
+/* Mixed-precision variants of the two scan entry points: x, x_rg_lru, a_rg_lru (and, in
+ * the backward, their three gradients) have in_dtype; h (and, in the backward, h_saved and
+ * grad_out) have out_dtype / state_dtype.  Supported pairs: (bf16, bf16), (f32, f32) and
+ * (f32, bf16).  The last one is what the model produces under autocast (fp32 conv output
+ * and gate logits, bf16 h): upstream first casts all inputs to bf16 with three extra
+ * kernels (custom_fwd(cast_inputs=bfloat16), hawk/scan_fused.py:428) and autograd casts the
+ * three gradients back to fp32 with three more; here the rounding happens in registers.
+ * The plain entry points above are these with both dtypes equal. */
+int hawk_rglru_scan_fwd_mixed(const void* x, const void* x_rg_lru, const void* a_rg_lru,
+                              const float* a_param, void* h, int B, int T, int D, int in_dtype,
+                              int out_dtype, void* workspace_device, size_t workspace_bytes,
+                              void* stream);
+int hawk_rglru_scan_bwd_mixed(const void* x, const void* x_rg_lru, const void* a_rg_lru,
+                              const float* a_param, const void* h_saved, const void* grad_out,
+                              void* dx, void* dx_rg_lru, void* da_rg_lru, float* da_param,
+                              int B, int T, int D, int in_dtype, int state_dtype,
+                              void* workspace_device, size_t workspace_bytes, void* stream);
+
 /* ---------------------------------------------------------------------------------------
  * Temporal causal depthwise conv1d.
  *   y[b,t,c] = bias[c] + sum_{s<W} w[W-1-s,c] x[b,t-s,c]

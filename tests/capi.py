@@ -56,6 +56,34 @@ def scan_fwd(x, xg, ag, lam, ws=None):
     return h
 
 
+def scan_fwd_mixed(x, xg, ag, lam, out_dtype, ws=None):
+    """Inputs in x.dtype, h in out_dtype (the (f32, bf16) pair is the interesting one)."""
+    B, T, D = x.shape
+    h = torch.empty((B, T, D), dtype=out_dtype, device="cuda")
+    if ws is None:
+        ws = new_workspace(B, T, D, "bf16" if x.dtype == torch.bfloat16 else "f32")
+    rc = _lib.load().hawk_rglru_scan_fwd_mixed(
+        x.data_ptr(), xg.data_ptr(), ag.data_ptr(), lam.data_ptr(), h.data_ptr(), B, T, D,
+        _lib.dtype_code(x.dtype), _lib.dtype_code(out_dtype), ws.data_ptr(), ws.numel(), _stream())
+    _lib.check("hawk_rglru_scan_fwd_mixed", rc)
+    return h
+
+
+def scan_bwd_mixed(x, xg, ag, lam, h, gout, ws=None):
+    """x, xg, ag and the returned gradients in x.dtype; h and gout in h.dtype."""
+    B, T, D = x.shape
+    dx, dxg, dag = torch.empty_like(x), torch.empty_like(x), torch.empty_like(x)
+    dlam = torch.empty(D, dtype=torch.float32, device="cuda")
+    if ws is None:
+        ws = new_workspace(B, T, D, "bf16" if x.dtype == torch.bfloat16 else "f32")
+    rc = _lib.load().hawk_rglru_scan_bwd_mixed(
+        x.data_ptr(), xg.data_ptr(), ag.data_ptr(), lam.data_ptr(), h.data_ptr(), gout.data_ptr(),
+        dx.data_ptr(), dxg.data_ptr(), dag.data_ptr(), dlam.data_ptr(), B, T, D,
+        _lib.dtype_code(x.dtype), _lib.dtype_code(h.dtype), ws.data_ptr(), ws.numel(), _stream())
+    _lib.check("hawk_rglru_scan_bwd_mixed", rc)
+    return dx, dxg, dag, dlam
+
+
 def scan_bwd(x, xg, ag, lam, h, gout, ws=None):
     B, T, D = x.shape
     dx, dxg, dag = torch.empty_like(x), torch.empty_like(x), torch.empty_like(x)

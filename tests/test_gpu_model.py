@@ -41,16 +41,26 @@ def test_fused_linear_scan_autograd(dtype):
         assert max_rel(capi.to_np(t.grad), want) < TOL[dtype]
 
 
-def test_fused_linear_scan_under_autocast_casts_activations_not_lambda():
+def test_fused_linear_scan_under_autocast_bf16_state_fp32_inputs_and_lambda():
     (x, xg, ag), lam, gout = _leaves(1, 130, 64, "f32", seed=2)
     with torch.autocast(device_type="cuda", dtype=torch.bfloat16):
         h = hk.fused_linear_scan(x, xg, ag, lam)
     assert h.dtype == torch.bfloat16  # as upstream's custom_fwd(cast_inputs=bfloat16)
     h.backward(gout.to(torch.bfloat16))
     assert x.grad.dtype == torch.float32 and lam.grad.dtype == torch.float32
-    xr, xgr, agr = (capi.to_np(t.detach().to(torch.bfloat16)) for t in (x, xg, ag))
-    h_ref = oracle.rglru_scan_fwd(xr, xgr, agr, capi.to_np(lam))  # Lambda NOT rounded to bf16
+    # inputs are read as fp32 (no bf16 rounding of x or of the gate logits) and Lambda is not rounded
+    xr, xgr, agr = (capi.to_np(t) for t in (x, xg, ag))
+    h_ref = oracle.rglru_scan_fwd(xr, xgr, agr, capi.to_np(lam))
     assert max_rel(capi.to_np(h), h_ref) < TOL["bf16"]
+    ref = oracle.rglru_scan_bwd(xr, xgr, agr, capi.to_np(lam), capi.to_np(h), capi.to_np(gout.bfloat16()))
+    for t, want in zip((x, xg, ag, lam), ref):
+        assert max_rel(capi.to_np(t.grad), want) < TOL["bf16"]
+    # bf16 inputs under autocast take the all-bf16 kernels
+    xb, xgb, agb = (t.detach().bfloat16().requires_grad_(True) for t in (x, xg, ag))
+    with torch.autocast(device_type="cuda", dtype=torch.bfloat16):
+        hb = hk.fused_linear_scan(xb, xgb, agb, lam)
+    hb.backward(gout.bfloat16())
+    assert hb.dtype == torch.bfloat16 and xb.grad.dtype == torch.bfloat16
 
 
 def test_scan_wrapper_contract_errors_and_copies():

@@ -77,6 +77,42 @@ def test_many_tiles_long_memory(dtype):
     _run_case(1, 8192, 128, dtype, seed=5, lo=0.99, hi=0.9999)
 
 
+@pytest.mark.parametrize("shape", [(1, 256, 512), (2, 1000, 192), (1, 1, 64), (2, 97, 65), (1, 4096, 128)])
+def test_mixed_precision_entry_fp32_inputs_bf16_state(shape):
+    """fp32 x / gate logits, bf16 h and grad_out, fp32 gradients: what the model feeds the
+    scan under autocast.  The oracle sees the exact fp32 inputs; tolerance is the bf16 one
+    because h and grad_out are bf16."""
+    B, T, D = shape
+    x, xg, ag, lam, gout = make_scan_inputs(B, T, D, seed=T + D)
+    (dx_, dxg_, dag_), (xr, xgr, agr) = _round_inputs((x, xg, ag), "f32")
+    go_d = capi.to_dev(gout, "bf16")
+    gor = capi.to_np(go_d)
+    lam_d = capi.to_dev(lam, "f32")
+    lam_r = capi.to_np(lam_d)
+    h = capi.scan_fwd_mixed(dx_, dxg_, dag_, lam_d, torch.bfloat16)
+    assert h.dtype == torch.bfloat16
+    h_ref = oracle.rglru_scan_fwd(xr, xgr, agr, lam_r)
+    assert max_rel(capi.to_np(h), h_ref) < TOL["bf16"]
+    grads = capi.scan_bwd_mixed(dx_, dxg_, dag_, lam_d, h, go_d)
+    assert all(g.dtype == torch.float32 for g in grads)
+    ref = oracle.rglru_scan_bwd(xr, xgr, agr, lam_r, capi.to_np(h), gor)
+    for name, got, want in zip(("dx", "dx_rg_lru", "da_rg_lru", "da_param"), grads, ref):
+        assert max_rel(capi.to_np(got), want) < TOL["bf16"], name
+    # the mixed forward must agree with "cast inputs to bf16, then scan" up to input rounding,
+    # and be closer to the exact-input oracle than that path is
+    h_cast = capi.scan_fwd(dx_.bfloat16(), dxg_.bfloat16(), dag_.bfloat16(), lam_d)
+    err_mixed = np.abs(capi.to_np(h) - h_ref).mean()
+    err_cast = np.abs(capi.to_np(h_cast) - h_ref).mean()
+    assert err_mixed <= err_cast * 1.05
+
+
+def test_unsupported_dtype_pairs_are_refused():
+    x = torch.zeros(1, 8, 64, device="cuda", dtype=torch.bfloat16)
+    lam = torch.zeros(64, device="cuda")
+    with pytest.raises(Exception, match="dtype"):
+        capi.scan_fwd_mixed(x, x, x, lam, torch.float32)  # bf16 inputs with fp32 state: not offered
+
+
 def test_workspace_reuse_across_shapes_and_launches():
     """One workspace serves repeated launches and smaller shapes; tags of earlier launches
     must never be taken for fresh ones."""

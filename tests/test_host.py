@@ -61,6 +61,10 @@ def test_argument_validation_needs_no_gpu():
     assert lib.hawk_conv1d_step(None, p, p, p, p, 1, 64, 4, 0, 0, None) == _lib.HAWK_ERR_NULL_POINTER
     assert lib.hawk_rglru_step(p, p, p, p, p, p, 0, 64, 0, 0, None) == _lib.HAWK_ERR_BAD_SHAPE
     assert lib.hawk_scan_workspace_init(None, 1024, None) == _lib.HAWK_ERR_NULL_POINTER
+    # mixed entry points: bf16 inputs with fp32 state is not an offered pair
+    assert lib.hawk_rglru_scan_fwd_mixed(*args, 1, 8, 64, 0, 1, None, 0, None) == _lib.HAWK_ERR_BAD_DTYPE
+    assert lib.hawk_rglru_scan_bwd_mixed(*bwd, 1, 8, 64, 0, 1, p, 1 << 20, None) == _lib.HAWK_ERR_BAD_DTYPE
+    assert lib.hawk_rglru_scan_bwd_mixed(*bwd, 1, 8, 64, 1, 0, None, 0, None) == _lib.HAWK_ERR_WORKSPACE
 
 
 def test_workspace_size_queries():
@@ -165,8 +169,13 @@ def test_custom_ops_have_shape_rules_for_tracing():
     with FakeTensorMode():
         x = torch.empty(2, 16, 64, dtype=torch.bfloat16, device="cuda")
         lam = torch.empty(64, device="cuda")
-        h = torch.ops.hawk_amd.rglru_scan_fwd(x, x, x, lam)
+        h = torch.ops.hawk_amd.rglru_scan_fwd(x, x, x, lam, False)
         assert h.shape == x.shape and h.dtype == torch.bfloat16
+        xf = torch.empty(2, 16, 64, device="cuda")
+        hm = torch.ops.hawk_amd.rglru_scan_fwd(xf, xf, xf, lam, True)
+        assert hm.dtype == torch.bfloat16
+        gm = torch.ops.hawk_amd.rglru_scan_bwd(xf, xf, xf, lam, hm, hm)
+        assert gm[0].dtype == torch.float32
         dx, dxg, dag, dlam = torch.ops.hawk_amd.rglru_scan_bwd(x, x, x, lam, h, h)
         assert dx.shape == x.shape and dlam.shape == (64,) and dlam.dtype == torch.float32
         w = torch.empty(4, 64, device="cuda")
