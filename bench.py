@@ -42,9 +42,9 @@ HBM_PEAK_GBS = 8000.0
 # device copy of known size in the same run (FETCH x 2.000, WRITE x 1.000 on this part).
 # Sources: profiles/rglru_scan_B8_T4096_D2560_bf16.md, profiles/rglru_scan_B2_T32768_D4096_bf16.md.
 MEASURED_BWD_TRAFFIC_BYTES = {
-    "scan": 903.6e6 + 547.5e6,
-    "scan_conv": 903.6e6 + 547.5e6,
-    "long": 2902e6 + 1754e6,
+    "scan": 865.4e6 + 533.0e6,
+    "scan_conv": 865.4e6 + 533.0e6,
+    "long": 2776.5e6 + 1711.7e6,
 }
 
 WORKLOADS = {
