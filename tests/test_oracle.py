@@ -3,7 +3,8 @@
 Upstream holds no tests, fixtures or golden vectors, so each function of the oracle is
 pinned by mathematics: closed forms, a library routine, an independent derivation by
 automatic differentiation, finite differences, and special cases, chosen so that a dropped
-term, a wrong sign or an off-by-one time index fails at least one of them.
+term, a wrong sign or an off-by-one time index fails at least one of them.  A fixture written
+by an unrelated third-party implementation is checked in test_golden.py.
 """
 
 import numpy as np
