@@ -14,7 +14,9 @@ from .external import (
 from .hawk import Hawk, HawkConfig, HawkModel, MLP, RMSNorm, RNNLayer
 from .scan_fused import (
     DiagonalRecurrence,
+    GatedDiagonalRecurrence,
     fused_linear_scan,
+    fused_linear_scan_gated,
     sequential_scan_backward,
     sequential_scan_forward,
 )
@@ -23,6 +25,7 @@ __all__ = [
     "BlockDiagonalLinear",
     "Conv1D",
     "DiagonalRecurrence",
+    "GatedDiagonalRecurrence",
     "Hawk",
     "HawkConfig",
     "HawkModel",
@@ -31,6 +34,7 @@ __all__ = [
     "RNNCache",
     "RNNLayer",
     "fused_linear_scan",
+    "fused_linear_scan_gated",
     "rglru_step",
     "rnn_param_init",
     "sequential_scan_backward",

@@ -42,6 +42,15 @@ SIGNATURES = {
     "hawk_rglru_scan_bwd": (_c_int, [_c_void_p] * 10 + [_c_int] * 4 + [_c_void_p, _c_size_t, _c_void_p]),
     "hawk_rglru_scan_fwd_mixed": (_c_int, [_c_void_p] * 5 + [_c_int] * 5 + [_c_void_p, _c_size_t, _c_void_p]),
     "hawk_rglru_scan_bwd_mixed": (_c_int, [_c_void_p] * 10 + [_c_int] * 5 + [_c_void_p, _c_size_t, _c_void_p]),
+    "hawk_rglru_scan_gated_fwd": (
+        _c_int,
+        [_c_void_p] * 5 + [ctypes.c_longlong] + [_c_void_p] * 3 + [_c_int] * 5 + [_c_void_p, _c_size_t, _c_void_p],
+    ),
+    "hawk_rglru_scan_gated_bwd": (
+        _c_int,
+        [_c_void_p] * 5 + [ctypes.c_longlong] + [_c_void_p] * 6 + [ctypes.c_longlong] + [_c_void_p]
+        + [_c_int] * 5 + [_c_void_p, _c_size_t, _c_void_p],
+    ),
     "hawk_conv1d_fwd": (_c_int, [_c_void_p] * 5 + [_c_int] * 6 + [_c_void_p]),
     "hawk_conv1d_bwd_workspace_bytes": (_c_size_t, [_c_int] * 4),
     "hawk_conv1d_bwd": (_c_int, [_c_void_p] * 6 + [_c_int] * 6 + [_c_void_p, _c_size_t, _c_void_p]),

@@ -9,10 +9,15 @@ namespace {
 
 inline bool dtype_ok(int d) { return d == HAWK_DTYPE_BF16 || d == HAWK_DTYPE_F32; }
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+// y and dy of the gated scan may be slices of wider tensors: element alignment is enough
+inline bool aligned_elem(const void* p, int dtype) {
+    return (reinterpret_cast<uintptr_t>(p) & (dtype == HAWK_DTYPE_F32 ? 3u : 1u)) == 0;
+}
 inline hipStream_t as_stream(void* s) { return static_cast<hipStream_t>(s); }
 
 constexpr int kMaxGridY = 65535;
 constexpr long long kMaxTiles = 0x7fffffffLL;
+constexpr long long kMaxRowStride = 1LL << 24;  // elements; keeps 16 rows of any dtype within 32-bit byte offsets
 
 int check_scan_shape(int B, int T, int D) {
     if (B < 1 || T < 1 || D < 1) return HAWK_ERR_BAD_SHAPE;
@@ -103,6 +108,46 @@ int hawk_rglru_scan_bwd(const void* x, const void* x_rg_lru, const void* a_rg_lr
                         size_t workspace_bytes, void* stream) {
     return hawk_rglru_scan_bwd_mixed(x, x_rg_lru, a_rg_lru, a_param, h_saved, grad_out, dx, dx_rg_lru, da_rg_lru,
                                      da_param, B, T, D, dtype, dtype, workspace_device, workspace_bytes, stream);
+}
+
+int hawk_rglru_scan_gated_fwd(const void* x, const void* x_rg_lru, const void* a_rg_lru, const float* a_param,
+                              const void* y, long long ldy, void* h, void* out, void* h_last, int B, int T, int D,
+                              int in_dtype, int out_dtype, void* workspace_device, size_t workspace_bytes,
+                              void* stream) {
+    if (!x || !x_rg_lru || !a_rg_lru || !a_param || !y || !out) return HAWK_ERR_NULL_POINTER;
+    if (!dtype_ok(in_dtype) || !dtype_ok(out_dtype) || !hawk::scan_dtypes_supported(in_dtype, out_dtype))
+        return HAWK_ERR_BAD_DTYPE;
+    if (int rc = check_scan_shape(B, T, D)) return rc;
+    if (ldy < D || ldy > kMaxRowStride) return HAWK_ERR_BAD_SHAPE;
+    if (!aligned16(x) || !aligned16(x_rg_lru) || !aligned16(a_rg_lru) || !aligned_elem(y, out_dtype) ||
+        !aligned16(out) || (h && !aligned16(h)) || (h_last && !aligned16(h_last)))
+        return HAWK_ERR_ALIGNMENT;
+    if (workspace_device && !aligned16(workspace_device)) return HAWK_ERR_ALIGNMENT;
+    return hawk::scan_gated_fwd(x, x_rg_lru, a_rg_lru, a_param, y, ldy, h, out, h_last, B, T, D, in_dtype, out_dtype,
+                                workspace_device, workspace_bytes, as_stream(stream));
+}
+
+int hawk_rglru_scan_gated_bwd(const void* x, const void* x_rg_lru, const void* a_rg_lru, const float* a_param,
+                              const void* y, long long ldy, const void* h_saved, const void* grad_out, void* dx,
+                              void* dx_rg_lru, void* da_rg_lru, void* dy, long long lddy, float* da_param, int B,
+                              int T, int D, int in_dtype, int state_dtype, void* workspace_device,
+                              size_t workspace_bytes, void* stream) {
+    if (!x || !x_rg_lru || !a_rg_lru || !a_param || !y || !h_saved || !grad_out || !dx || !dx_rg_lru || !da_rg_lru ||
+        !dy || !da_param)
+        return HAWK_ERR_NULL_POINTER;
+    if (!dtype_ok(in_dtype) || !dtype_ok(state_dtype) || !hawk::scan_dtypes_supported(in_dtype, state_dtype))
+        return HAWK_ERR_BAD_DTYPE;
+    if (int rc = check_scan_shape(B, T, D)) return rc;
+    if (ldy < D || ldy > kMaxRowStride || lddy < D || lddy > kMaxRowStride) return HAWK_ERR_BAD_SHAPE;
+    if (!aligned16(x) || !aligned16(x_rg_lru) || !aligned16(a_rg_lru) || !aligned_elem(y, state_dtype) ||
+        !aligned16(h_saved) || !aligned16(grad_out) || !aligned16(dx) || !aligned16(dx_rg_lru) ||
+        !aligned16(da_rg_lru) || !aligned_elem(dy, state_dtype))
+        return HAWK_ERR_ALIGNMENT;
+    if (workspace_device == nullptr) return HAWK_ERR_WORKSPACE;
+    if (!aligned16(workspace_device)) return HAWK_ERR_ALIGNMENT;
+    return hawk::scan_gated_bwd(x, x_rg_lru, a_rg_lru, a_param, y, ldy, h_saved, grad_out, dx, dx_rg_lru, da_rg_lru,
+                                dy, lddy, da_param, B, T, D, in_dtype, state_dtype, workspace_device, workspace_bytes,
+                                as_stream(stream));
 }
 
 int hawk_conv1d_fwd(const void* x, const float* w, const float* bias, const void* state, void* y, int B, int T,

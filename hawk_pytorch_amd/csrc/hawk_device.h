@@ -232,4 +232,43 @@ __device__ __forceinline__ uint32_t opaque(uint32_t x) {
 
 __device__ __forceinline__ float clamp01(float z) { return fminf(fmaxf(z, 0.0f), 1.0f); }
 
+// Standard normal CDF Phi(y) and e = exp(-y^2 / 2), the two pieces of the exact (erf) GELU:
+//   gelu(y) = y Phi(y),   gelu'(y) = Phi(y) + y e / sqrt(2 pi).
+// Phi comes from erfc(|y| / sqrt 2), so the negative tail keeps its relative accuracy.
+//   PRECISE: t exp(-x^2 + P9(t)), t = 1 / (1 + x/2)   (Numerical Recipes' erfcc; relative
+//            error 1.2e-7 in exact arithmetic, about 4e-6 in fp32)
+//   else:    t P4(t) exp(-x^2), t = 1 / (1 + 0.3275911 x)   (Abramowitz & Stegun 7.1.26;
+//            absolute error 1.5e-7, far below bf16 rounding)
+template <bool PRECISE>
+__device__ __forceinline__ void normal_cdf(float y, float& cdf, float& e) {
+    const float ax = fabsf(y) * 0.70710678118654752f;
+    const float nx2 = -ax * ax;
+    e = hw_exp2(nx2 * kLog2e);
+    float half_erfc;
+    if (PRECISE) {
+        const float t = hw_rcp(fmaf(0.5f, ax, 1.0f));
+        float p = 0.17087277f;
+        p = fmaf(p, t, -0.82215223f);
+        p = fmaf(p, t, 1.48851587f);
+        p = fmaf(p, t, -1.13520398f);
+        p = fmaf(p, t, 0.27886807f);
+        p = fmaf(p, t, -0.18628806f);
+        p = fmaf(p, t, 0.09678418f);
+        p = fmaf(p, t, 0.37409196f);
+        p = fmaf(p, t, 1.00002368f);
+        p = fmaf(p, t, -1.26551223f);
+        half_erfc = (0.5f * t) * hw_exp2((nx2 + p) * kLog2e);
+    } else {
+        const float t = hw_rcp(fmaf(0.3275911f, ax, 1.0f));
+        float p = 1.061405429f;
+        p = fmaf(p, t, -1.453152027f);
+        p = fmaf(p, t, 1.421413741f);
+        p = fmaf(p, t, -0.284496736f);
+        p = fmaf(p, t, 0.254829592f);
+        half_erfc = (0.5f * t) * (p * e);
+    }
+    cdf = (y < 0.0f) ? half_erfc : 1.0f - half_erfc;
+}
+constexpr float kInvSqrt2Pi = 0.39894228040143268f;
+
 }  // namespace hawk

@@ -32,6 +32,8 @@
 // on timing: the combination order is a function of the tile position only.
 #include "hawk_scan.h"
 
+#include <stdint.h>
+
 #include "hawk_device.h"
 
 namespace hawk {
@@ -179,7 +181,8 @@ __device__ __forceinline__ void exchange_carry(const ScanWsPtrs& ws, int pos, in
 
 // Slice aggregates of the NW waves -> prefix for wave `w` and tile total, in chain order
 // (forward: wave 0 first; backward: wave NW-1 first).
-template <int V, int NW, bool REVERSE>
+// LEAN: read the staged aggregates four at a time instead of all at once (fewer registers).
+template <int V, int NW, bool REVERSE, bool LEAN = false>
 __device__ __forceinline__ void combine_slices(float2 (*s_agg)[kWave * V], int w, int lane, float (&pre_p)[V],
                                                float (&pre_h)[V], float (&tot_p)[V], float (&tot_h)[V]) {
 #pragma unroll
@@ -194,18 +197,42 @@ __device__ __forceinline__ void combine_slices(float2 (*s_agg)[kWave * V], int w
             tot_h[v] = fmaf(a.x, tot_h[v], a.y);
             tot_p[v] *= a.x;
         }
+        if (LEAN && (q % 4) == 3) __builtin_amdgcn_sched_barrier(0);
     }
+}
+
+// Operands of the gated variants (out = gelu(y) * h, the step that follows the scan in a
+// Hawk block).  y and dy are [B, T, D] views whose rows may be further apart than D
+// elements (y is one half of a wider projection); batches are T rows apart.
+template <typename OT>
+struct GateFwdArgs {
+    const OT* y;      // gate input
+    OT* out;          // gelu(y) * h, dense [B, T, D]
+    OT* h_last;       // optional [B, D]: h at t = T-1 (the decode cache's recurrent state)
+    uint32_t ldy;     // elements between consecutive rows of y
+};
+template <typename ST>
+struct GateBwdArgs {
+    const ST* y;
+    ST* dy;
+    uint32_t ldy, lddy;
+};
+
+// Bytes of a [rows, D - c_tile] window of a row-strided tensor, for its buffer resource.
+__device__ __forceinline__ uint32_t strided_window_bytes(int rows, uint32_t row_bytes, uint32_t last_row_bytes) {
+    return rows > 0 ? (uint32_t)(rows - 1) * row_bytes + last_row_bytes : 0u;
 }
 
 // ---------------------------------------------------------------------------------------
 // Forward tile.  FULL: every row of the tile is inside [0, T).
+// GATED: also reads y and writes out = gelu(y) * h; h itself is stored only if h != nullptr.
 // ---------------------------------------------------------------------------------------
-template <typename IT, typename OT, int V, int TC, int NW, bool PRECISE, bool FULL>
+template <typename IT, typename OT, int V, int TC, int NW, bool PRECISE, bool FULL, bool GATED, bool STORE_H>
 __device__ __forceinline__ void fwd_tile(const IT* __restrict__ x, const IT* __restrict__ xg,
                                          const IT* __restrict__ ag, const float* __restrict__ lam,
-                                         OT* __restrict__ h, int B, int T, int D, int nseg, int seg, int b, int ct,
-                                         uint32_t tag, const ScanWsPtrs& ws, float2 (*s_agg)[kWave * V],
-                                         float2 (*s_prev)[kWave * V]) {
+                                         OT* __restrict__ h, const GateFwdArgs<OT>& gate, int B, int T, int D,
+                                         int nseg, int seg, int b, int ct, uint32_t tag, const ScanWsPtrs& ws,
+                                         float2 (*s_agg)[kWave * V], float2 (*s_prev)[kWave * V]) {
     typedef typename Raw<IT, V>::type raw_t;
     typedef typename Raw<OT, V>::type out_raw_t;
     constexpr int CT = kWave * V;
@@ -224,8 +251,8 @@ __device__ __forceinline__ void fwd_tile(const IT* __restrict__ x, const IT* __r
     const uint32_t slab = (uint32_t)rows_in * row_bytes;
     const uint32_t lane_bytes = lane_off * sizeof(IT);
     const rsrc_t bx = make_rsrc(x + tile_off, slab), bxg = make_rsrc(xg + tile_off, slab),
-                 bag = make_rsrc(ag + tile_off, slab),
-                 bh = make_rsrc(h + tile_off, (uint32_t)rows_in * out_row_bytes);
+                 bag = make_rsrc(ag + tile_off, slab);
+    const rsrc_t bh = make_rsrc(STORE_H ? h + tile_off : nullptr, STORE_H ? (uint32_t)rows_in * out_row_bytes : 0u);
     // idle lanes store at an offset beyond any slab, which the range check drops
     const uint32_t store_bytes = lane_on ? lane_off * (uint32_t)sizeof(OT) : 0x80000000u;
 
@@ -280,12 +307,25 @@ __device__ __forceinline__ void fwd_tile(const IT* __restrict__ x, const IT* __r
         __builtin_amdgcn_sched_barrier(0);  // one row's temporaries live at a time
     }
 
+    // The gate rows are fetched now, into registers the raw inputs occupied until here,
+    // and arrive during the carry exchange.
+    out_raw_t ry[GATED ? TC : 1];
+    if constexpr (GATED) {
+        __builtin_amdgcn_sched_barrier(0);  // not before the local pass has freed the inputs' registers
+        const uint32_t y_row_bytes = gate.ldy * (uint32_t)sizeof(OT);
+        const rsrc_t by = make_rsrc(gate.y + ((size_t)b * T + t0) * gate.ldy + c_tile,
+                                    strided_window_bytes(rows_in, y_row_bytes, (uint32_t)(D - c_tile) * sizeof(OT)));
+#pragma unroll
+        for (int j = 0; j < TC; ++j)
+            ry[j] = buffer_load<out_raw_t>(by, lane_off * (uint32_t)sizeof(OT), j * y_row_bytes);
+    }
+
     // 2. combine the NW time slices of this tile
 #pragma unroll
     for (int v = 0; v < V; ++v) s_agg[w][lane * V + v] = make_float2(p_run[v], h_run[v]);
     __syncthreads();
     float pre_p[V], pre_h[V], tot_p[V], tot_h[V];
-    combine_slices<V, NW, false>(s_agg, w, lane, pre_p, pre_h, tot_p, tot_h);
+    combine_slices<V, NW, false, GATED>(s_agg, w, lane, pre_p, pre_h, tot_p, tot_h);
 
     // 3. carry across tiles
     float cin[V];
@@ -300,6 +340,9 @@ __device__ __forceinline__ void fwd_tile(const IT* __restrict__ x, const IT* __r
     float cw[V];
 #pragma unroll
     for (int v = 0; v < V; ++v) cw[v] = fmaf(pre_p[v], cin[v], pre_h[v]);
+    const rsrc_t bout = make_rsrc(GATED ? gate.out + tile_off : nullptr, GATED ? (uint32_t)rows_in * out_row_bytes : 0u);
+    const int j_last = T - 1 - t0;  // row of this slice that is t = T-1, if any (wave-uniform)
+    out_raw_t r_last = raw_zero<out_raw_t>();
 #pragma unroll
     for (int j = 0; j < TC; ++j) {
         float out[V];
@@ -312,15 +355,42 @@ __device__ __forceinline__ void fwd_tile(const IT* __restrict__ x, const IT* __r
         }
         out_raw_t r;
         pack(out, r);
-        buffer_store<out_raw_t>(r, bh, store_bytes, j * out_row_bytes);  // rows past T and idle lanes are dropped
+        if constexpr (GATED) {
+            float fy[V], o[V];
+            if constexpr (sizeof(out_raw_t) == 4) {
+                unpack(opaque(ry[j]), fy);  // keeps the gate's arithmetic below the exchange, one row at a time
+            } else {
+                unpack(ry[j], fy);
+            }
+#pragma unroll
+            for (int v = 0; v < V; ++v) {
+                float cdf, e;
+                normal_cdf<PRECISE>(fy[v], cdf, e);
+                o[v] = (fy[v] * cdf) * out[v];
+            }
+            out_raw_t ro;
+            pack(o, ro);
+            buffer_store<out_raw_t>(ro, bout, store_bytes, j * out_row_bytes);
+            if constexpr (STORE_H) buffer_store<out_raw_t>(r, bh, store_bytes, j * out_row_bytes);
+            r_last = (j == j_last) ? r : r_last;
+            __builtin_amdgcn_sched_barrier(0);  // one row's temporaries live at a time
+        } else {
+            buffer_store<out_raw_t>(r, bh, store_bytes, j * out_row_bytes);  // rows past T and idle lanes are dropped
+        }
+    }
+    if constexpr (GATED) {
+        if (gate.h_last != nullptr && j_last >= 0 && j_last < TC) {
+            const rsrc_t bl = make_rsrc(gate.h_last + (size_t)b * D + c_tile, (uint32_t)(D - c_tile) * sizeof(OT));
+            buffer_store<out_raw_t>(r_last, bl, store_bytes, 0u);
+        }
     }
 }
 
-template <typename IT, typename OT, int V, int TC, int NW, bool PRECISE>
+template <typename IT, typename OT, int V, int TC, int NW, bool PRECISE, bool GATED, bool STORE_H>
 __global__ __launch_bounds__(NW * kWave, HAWK_FWD_WAVES_PER_SIMD) void rglru_scan_fwd_kernel(
     const IT* __restrict__ x, const IT* __restrict__ xg, const IT* __restrict__ ag,
-    const float* __restrict__ lam, OT* __restrict__ h, int B, int T, int D, int nseg, int nct,
-    ScanWsPtrs ws) {
+    const float* __restrict__ lam, OT* __restrict__ h, GateFwdArgs<OT> gate, int B, int T, int D, int nseg,
+    int nct, ScanWsPtrs ws) {
     constexpr int CT = kWave * V;
     constexpr int TS = NW * TC;
     __shared__ float2 s_agg[NW][CT];
@@ -336,9 +406,11 @@ __global__ __launch_bounds__(NW * kWave, HAWK_FWD_WAVES_PER_SIMD) void rglru_sca
     const int b = rem / nct;
     const int ct = rem - b * nct;
     if (seg * TS + TS <= T)
-        fwd_tile<IT, OT, V, TC, NW, PRECISE, true>(x, xg, ag, lam, h, B, T, D, nseg, seg, b, ct, tag, ws, s_agg, s_prev);
+        fwd_tile<IT, OT, V, TC, NW, PRECISE, true, GATED, STORE_H>(x, xg, ag, lam, h, gate, B, T, D, nseg, seg, b, ct,
+                                                                   tag, ws, s_agg, s_prev);
     else
-        fwd_tile<IT, OT, V, TC, NW, PRECISE, false>(x, xg, ag, lam, h, B, T, D, nseg, seg, b, ct, tag, ws, s_agg, s_prev);
+        fwd_tile<IT, OT, V, TC, NW, PRECISE, false, GATED, STORE_H>(x, xg, ag, lam, h, gate, B, T, D, nseg, seg, b, ct,
+                                                                    tag, ws, s_agg, s_prev);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -350,15 +422,18 @@ __global__ __launch_bounds__(NW * kWave, HAWK_FWD_WAVES_PER_SIMD) void rglru_sca
 //   dlog_a = g (h_{t-1} alpha - i x alpha^2 2 csg(1-alpha^2));
 //   da_rg_lru = dlog_a r (1-r) (-8 softplus(Lambda));  dLambda += dlog_a r  (scaled per channel later)
 // FULL: every row of the tile is inside [1, T) (row 0 has no h_{t-1}).
+// GATED: gout is the gradient of out = gelu(y) * h; the gradient reaching h is
+//   gout gelu(y), and dy = gout h_t gelu'(y) is stored as a fourth output.
 // ---------------------------------------------------------------------------------------
-template <typename IT, typename ST, int V, int TC, int NW, bool PRECISE, bool FULL>
+template <typename IT, typename ST, int V, int TC, int NW, bool PRECISE, bool FULL, bool GATED>
 __device__ __forceinline__ void bwd_tile(const IT* __restrict__ x, const IT* __restrict__ xg,
                                          const IT* __restrict__ ag, const float* __restrict__ lam,
                                          const ST* __restrict__ hs, const ST* __restrict__ gout,
-                                         IT* __restrict__ dx, IT* __restrict__ dxg, IT* __restrict__ dag, int B,
-                                         int T, int D, int nseg, int seg, int pos, int b, int ct, uint32_t tag,
-                                         const ScanWsPtrs& ws, float2 (*s_agg)[kWave * V],
-                                         float2 (*s_prev)[kWave * V], float (*s_dl)[kWave * V]) {
+                                         IT* __restrict__ dx, IT* __restrict__ dxg, IT* __restrict__ dag,
+                                         const GateBwdArgs<ST>& gate, int B, int T, int D, int nseg, int seg, int pos,
+                                         int b, int ct, uint32_t tag, const ScanWsPtrs& ws,
+                                         float2 (*s_agg)[kWave * V], float2 (*s_prev)[kWave * V],
+                                         float (*s_dl)[kWave * V]) {
     typedef typename Raw<IT, V>::type raw_t;      // x, x_rg_lru, a_rg_lru and the three gradients
     typedef typename Raw<ST, V>::type sraw_t;     // saved h and grad_out
     constexpr int CT = kWave * V;
@@ -394,10 +469,22 @@ __device__ __forceinline__ void bwd_tile(const IT* __restrict__ x, const IT* __r
     // exchange.  This is what lets a lane own TC rows within 128 registers.
     raw_t rx[TC], rxg[TC], rag[TC];
     sraw_t rgo[TC], rhp[TC];
+    sraw_t ry[GATED ? TC : 1], rh_end = raw_zero<sraw_t>();
+    const uint32_t y_row_bytes = GATED ? gate.ldy * (uint32_t)sizeof(ST) : 0u;
+    const uint32_t dy_row_bytes = GATED ? gate.lddy * (uint32_t)sizeof(ST) : 0u;
+    rsrc_t by, bdy;
+    if constexpr (GATED) {
+        const uint32_t last = (uint32_t)(D - c_tile) * sizeof(ST);
+        by = make_rsrc(gate.y + ((size_t)b * T + t0) * gate.ldy + c_tile,
+                       strided_window_bytes(rows_in, y_row_bytes, last));
+        bdy = make_rsrc(gate.dy + ((size_t)b * T + t0) * gate.lddy + c_tile,
+                        strided_window_bytes(rows_in, dy_row_bytes, last));
+    }
 #pragma unroll
     for (int j = 0; j < TC; ++j) {
         rag[j] = buffer_load<raw_t>(bag, lane_bytes, j * row_bytes);
         rgo[j] = buffer_load<sraw_t>(bgo, slane_bytes, j * srow_bytes);
+        if constexpr (GATED) ry[j] = buffer_load<sraw_t>(by, slane_bytes, j * y_row_bytes);
     }
 
     float c2[V], cs[V];
@@ -423,6 +510,16 @@ __device__ __forceinline__ void bwd_tile(const IT* __restrict__ x, const IT* __r
         float fag[V], fgo[V], rv[V];
         unpack(rag[j], fag);
         unpack(rgo[j], fgo);
+        if constexpr (GATED) {
+            float fy[V];
+            unpack(ry[j], fy);
+#pragma unroll
+            for (int v = 0; v < V; ++v) {
+                float cdf, e;
+                normal_cdf<PRECISE>(fy[v], cdf, e);
+                fgo[v] *= fy[v] * cdf;
+            }
+        }
         const bool ok = FULL || (t0 + j < T);
 #pragma unroll
         for (int v = 0; v < V; ++v) rv[v] = sigmoid_fast(fag[v]);
@@ -449,6 +546,7 @@ __device__ __forceinline__ void bwd_tile(const IT* __restrict__ x, const IT* __r
         rhp[j] = (j == 0) ? buffer_load<sraw_t>(bhm1, slane_bytes, 0u)
                           : buffer_load<sraw_t>(bhs, slane_bytes, (j - 1) * srow_bytes);
     }
+    if constexpr (GATED) rh_end = buffer_load<sraw_t>(bhs, slane_bytes, (TC - 1) * srow_bytes);
     __builtin_amdgcn_sched_barrier(0);
 
     // 2. combine the time slices; later slices come first in the reverse chain
@@ -487,6 +585,25 @@ __device__ __forceinline__ void bwd_tile(const IT* __restrict__ x, const IT* __r
             unpack(rgo[j], fgo);
         }
         unpack(rhp[j], fhp);
+        float o4[V];
+        if constexpr (GATED) {
+            // gelu(y) again (cheaper than a register per element across the exchange), its
+            // derivative, and h_t, which is the next row's h_{t-1}
+            float fy[V], fh[V];
+            if constexpr (sizeof(sraw_t) == 4 && sizeof(ST) == 2) {
+                unpack(opaque(ry[j]), fy);
+            } else {
+                unpack(ry[j], fy);
+            }
+            unpack(j == TC - 1 ? rh_end : rhp[j == TC - 1 ? j : j + 1], fh);
+#pragma unroll
+            for (int v = 0; v < V; ++v) {
+                float cdf, e;
+                normal_cdf<PRECISE>(fy[v], cdf, e);
+                o4[v] = (fgo[v] * fh[v]) * fmaf(fy[v] * kInvSqrt2Pi, e, cdf);
+                fgo[v] *= fy[v] * cdf;
+            }
+        }
         const bool ok = FULL || (t0 + j < T);
         const uint32_t rpair = PACK_R ? opaque(rrh[j]) : 0u;
         float o1[V], o2[V], o3[V];
@@ -521,6 +638,11 @@ __device__ __forceinline__ void bwd_tile(const IT* __restrict__ x, const IT* __r
         buffer_store<raw_t>(r1, bdx, store_bytes, j * row_bytes);
         buffer_store<raw_t>(r2, bdxg, store_bytes, j * row_bytes);
         buffer_store<raw_t>(r3, bdag, store_bytes, j * row_bytes);
+        if constexpr (GATED) {
+            sraw_t r4;
+            pack(o4, r4);
+            buffer_store<sraw_t>(r4, bdy, lane_on ? slane_bytes : 0x80000000u, j * dy_row_bytes);
+        }
         __builtin_amdgcn_sched_barrier(0);  // one row's temporaries live at a time
     }
 #pragma unroll
@@ -537,12 +659,12 @@ __device__ __forceinline__ void bwd_tile(const IT* __restrict__ x, const IT* __r
     }
 }
 
-template <typename IT, typename ST, int V, int TC, int NW, bool PRECISE>
+template <typename IT, typename ST, int V, int TC, int NW, bool PRECISE, bool GATED>
 __global__ __launch_bounds__(NW * kWave, HAWK_BWD_WAVES_PER_SIMD) void rglru_scan_bwd_kernel(
     const IT* __restrict__ x, const IT* __restrict__ xg, const IT* __restrict__ ag,
     const float* __restrict__ lam, const ST* __restrict__ hs, const ST* __restrict__ gout,
-    IT* __restrict__ dx, IT* __restrict__ dxg, IT* __restrict__ dag, int B, int T, int D, int nseg,
-    int nct, ScanWsPtrs ws) {
+    IT* __restrict__ dx, IT* __restrict__ dxg, IT* __restrict__ dag, GateBwdArgs<ST> gate, int B, int T, int D,
+    int nseg, int nct, ScanWsPtrs ws) {
     constexpr int CT = kWave * V;
     constexpr int TS = NW * TC;
     __shared__ float2 s_agg[NW][CT];
@@ -560,11 +682,11 @@ __global__ __launch_bounds__(NW * kWave, HAWK_BWD_WAVES_PER_SIMD) void rglru_sca
     const int b = rem / nct;
     const int ct = rem - b * nct;
     if (seg > 0 && seg * TS + TS <= T)
-        bwd_tile<IT, ST, V, TC, NW, PRECISE, true>(x, xg, ag, lam, hs, gout, dx, dxg, dag, B, T, D, nseg, seg, pos, b,
-                                               ct, tag, ws, s_agg, s_prev, s_dl);
+        bwd_tile<IT, ST, V, TC, NW, PRECISE, true, GATED>(x, xg, ag, lam, hs, gout, dx, dxg, dag, gate, B, T, D, nseg,
+                                                          seg, pos, b, ct, tag, ws, s_agg, s_prev, s_dl);
     else
-        bwd_tile<IT, ST, V, TC, NW, PRECISE, false>(x, xg, ag, lam, hs, gout, dx, dxg, dag, B, T, D, nseg, seg, pos, b,
-                                                ct, tag, ws, s_agg, s_prev, s_dl);
+        bwd_tile<IT, ST, V, TC, NW, PRECISE, false, GATED>(x, xg, ag, lam, hs, gout, dx, dxg, dag, gate, B, T, D, nseg,
+                                                           seg, pos, b, ct, tag, ws, s_agg, s_prev, s_dl);
 }
 
 // dLambda[c] = -8 sigmoid(Lambda_c) * sum over rows of the [rows, D] partials.
@@ -635,8 +757,20 @@ struct TileShape {
 #ifndef HAWK_BWD_NW
 #define HAWK_BWD_NW 8
 #endif
+#ifndef HAWK_FWD_GATED_TC
+#define HAWK_FWD_GATED_TC 12
+#endif
+#ifndef HAWK_BWD_GATED_TC
+#define HAWK_BWD_GATED_TC 10
+#endif
+#ifndef HAWK_BWD_GATED_TC1
+#define HAWK_BWD_GATED_TC1 8
+#endif
 constexpr int kFwdTC = HAWK_FWD_TC, kFwdNW = HAWK_FWD_NW;
 constexpr int kBwdTC = HAWK_BWD_TC, kBwdNW = HAWK_BWD_NW;
+// the gate adds a register per row and lane (two channels per lane), or two (one channel)
+constexpr int kBwdGatedTC = HAWK_BWD_GATED_TC, kBwdGatedTC1 = HAWK_BWD_GATED_TC1;
+constexpr int kFwdGatedTC = HAWK_FWD_GATED_TC;  // two channels per lane; one channel keeps kFwdTC
 
 #ifndef HAWK_MAX_V
 #define HAWK_MAX_V 2
@@ -645,6 +779,8 @@ int pick_v(int D, int dtype) { return (HAWK_MAX_V >= 2 && dtype == HAWK_DTYPE_BF
 
 TileShape fwd_shape(int D, int dtype) { return TileShape{pick_v(D, dtype), kFwdTC, kFwdNW}; }
 TileShape bwd_shape(int D, int dtype) { return TileShape{pick_v(D, dtype), kBwdTC, kBwdNW}; }
+TileShape fwd_gated_shape(int V) { return TileShape{V, V == 2 ? kFwdGatedTC : kFwdTC, kFwdNW}; }
+TileShape bwd_gated_shape(int V) { return TileShape{V, V == 2 ? kBwdGatedTC : kBwdGatedTC1, kBwdNW}; }
 
 int ceil_div(int a, int b) { return (a + b - 1) / b; }
 
@@ -672,34 +808,131 @@ ScanWsPtrs carve(void* ws, const WsLayout& l) {
     return r;
 }
 
-template <typename IT, typename OT, int V, int TC, int NW, bool PRECISE>
-int launch_fwd(const void* x, const void* xg, const void* ag, const float* lam, void* h, int B, int T,
-               int D, int nseg, int nct, ScanWsPtrs ws, hipStream_t st) {
+// Type-erased gate operands as they arrive from the C ABI; y == nullptr means "not gated".
+struct GateFwdHost {
+    const void* y = nullptr;
+    void* out = nullptr;
+    void* h_last = nullptr;
+    uint32_t ldy = 0;
+};
+struct GateBwdHost {
+    const void* y = nullptr;
+    void* dy = nullptr;
+    uint32_t ldy = 0, lddy = 0;
+};
+
+template <typename IT, typename OT, int V, int TC, int NW, bool PRECISE, bool GATED>
+int launch_fwd(const void* x, const void* xg, const void* ag, const float* lam, void* h, const GateFwdHost& g,
+               int B, int T, int D, int nseg, int nct, ScanWsPtrs ws, hipStream_t st) {
     const unsigned grid = (unsigned)nseg * B * nct;
-    hipLaunchKernelGGL((rglru_scan_fwd_kernel<IT, OT, V, TC, NW, PRECISE>), dim3(grid), dim3(NW * kWave), 0, st,
-                       static_cast<const IT*>(x), static_cast<const IT*>(xg), static_cast<const IT*>(ag), lam,
-                       static_cast<OT*>(h), B, T, D, nseg, nct, ws);
+    const GateFwdArgs<OT> gate = {static_cast<const OT*>(g.y), static_cast<OT*>(g.out), static_cast<OT*>(g.h_last),
+                                  g.ldy};
+    if constexpr (!GATED) {
+        hipLaunchKernelGGL((rglru_scan_fwd_kernel<IT, OT, V, TC, NW, PRECISE, false, true>), dim3(grid),
+                           dim3(NW * kWave), 0, st, static_cast<const IT*>(x), static_cast<const IT*>(xg),
+                           static_cast<const IT*>(ag), lam, static_cast<OT*>(h), gate, B, T, D, nseg, nct, ws);
+    } else if (h != nullptr) {
+        hipLaunchKernelGGL((rglru_scan_fwd_kernel<IT, OT, V, TC, NW, PRECISE, GATED, true>), dim3(grid),
+                           dim3(NW * kWave), 0, st, static_cast<const IT*>(x), static_cast<const IT*>(xg),
+                           static_cast<const IT*>(ag), lam, static_cast<OT*>(h), gate, B, T, D, nseg, nct, ws);
+    } else {
+        hipLaunchKernelGGL((rglru_scan_fwd_kernel<IT, OT, V, TC, NW, PRECISE, GATED, false>), dim3(grid),
+                           dim3(NW * kWave), 0, st, static_cast<const IT*>(x), static_cast<const IT*>(xg),
+                           static_cast<const IT*>(ag), lam, static_cast<OT*>(h), gate, B, T, D, nseg, nct, ws);
+    }
     return hipGetLastError() == hipSuccess ? HAWK_OK : HAWK_ERR_LAUNCH;
 }
 
-template <typename IT, typename ST, int V, int TC, int NW, bool PRECISE>
+template <typename IT, typename ST, int V, int TC, int NW, bool PRECISE, bool GATED>
 int launch_bwd(const void* x, const void* xg, const void* ag, const float* lam, const void* hs,
-               const void* gout, void* dx, void* dxg, void* dag, int B, int T, int D, int nseg, int nct,
-               ScanWsPtrs ws, hipStream_t st) {
+               const void* gout, void* dx, void* dxg, void* dag, const GateBwdHost& g, int B, int T, int D,
+               int nseg, int nct, ScanWsPtrs ws, hipStream_t st) {
     const unsigned grid = (unsigned)nseg * B * nct;
-    hipLaunchKernelGGL((rglru_scan_bwd_kernel<IT, ST, V, TC, NW, PRECISE>), dim3(grid), dim3(NW * kWave), 0, st,
-                       static_cast<const IT*>(x), static_cast<const IT*>(xg), static_cast<const IT*>(ag), lam,
+    const GateBwdArgs<ST> gate = {static_cast<const ST*>(g.y), static_cast<ST*>(g.dy), g.ldy, g.lddy};
+    hipLaunchKernelGGL((rglru_scan_bwd_kernel<IT, ST, V, TC, NW, PRECISE, GATED>), dim3(grid), dim3(NW * kWave), 0,
+                       st, static_cast<const IT*>(x), static_cast<const IT*>(xg), static_cast<const IT*>(ag), lam,
                        static_cast<const ST*>(hs), static_cast<const ST*>(gout), static_cast<IT*>(dx),
-                       static_cast<IT*>(dxg), static_cast<IT*>(dag), B, T, D, nseg, nct, ws);
+                       static_cast<IT*>(dxg), static_cast<IT*>(dag), gate, B, T, D, nseg, nct, ws);
+    return hipGetLastError() == hipSuccess ? HAWK_OK : HAWK_ERR_LAUNCH;
+}
+
+template <bool GATED>
+int scan_fwd_impl(const void* x, const void* xg, const void* ag, const float* lam, void* h, const GateFwdHost& g,
+                  int B, int T, int D, int in_dtype, int out_dtype, void* ws, size_t ws_bytes, hipStream_t st) {
+    TileShape s = fwd_shape(D, in_dtype);
+    // a lane's pair of bf16 must stay 4-byte aligned in every row of y
+    if (GATED) s = fwd_gated_shape(((g.ldy % 2) != 0 || (reinterpret_cast<uintptr_t>(g.y) & 3u) != 0) ? 1 : s.V);
+    constexpr int TC2 = GATED ? kFwdGatedTC : kFwdTC;
+    const int nseg = ceil_div(T, s.rows());
+    const int nct = ceil_div(D, s.chans());
+    ScanWsPtrs p = {};
+    if (nseg > 1) {
+        const WsLayout l = layout_for(B, D, nseg, 0);
+        if (ws == nullptr || ws_bytes < l.total) return HAWK_ERR_WORKSPACE;
+        p = carve(ws, l);
+    }
+    if (in_dtype == HAWK_DTYPE_BF16) {
+        if (s.V == 2)
+            return launch_fwd<bf16_t, bf16_t, 2, TC2, kFwdNW, false, GATED>(x, xg, ag, lam, h, g, B, T, D, nseg, nct,
+                                                                               p, st);
+        return launch_fwd<bf16_t, bf16_t, 1, kFwdTC, kFwdNW, false, GATED>(x, xg, ag, lam, h, g, B, T, D, nseg, nct, p,
+                                                                           st);
+    }
+    if (out_dtype == HAWK_DTYPE_BF16)
+        return launch_fwd<float, bf16_t, 1, kFwdTC, kFwdNW, false, GATED>(x, xg, ag, lam, h, g, B, T, D, nseg, nct, p,
+                                                                          st);
+    return launch_fwd<float, float, 1, kFwdTC, kFwdNW, true, GATED>(x, xg, ag, lam, h, g, B, T, D, nseg, nct, p, st);
+}
+
+template <bool GATED>
+int scan_bwd_impl(const void* x, const void* xg, const void* ag, const float* lam, const void* hs, const void* gout,
+                  void* dx, void* dxg, void* dag, float* dlam, const GateBwdHost& g, int B, int T, int D,
+                  int in_dtype, int state_dtype, void* ws, size_t ws_bytes, hipStream_t st) {
+    constexpr int TC2 = GATED ? kBwdGatedTC : kBwdTC, TC1 = GATED ? kBwdGatedTC1 : kBwdTC;
+    TileShape s = bwd_shape(D, in_dtype);
+    if (GATED) {
+        const bool pairs_aligned = (g.ldy % 2) == 0 && (g.lddy % 2) == 0 &&
+                                   ((reinterpret_cast<uintptr_t>(g.y) | reinterpret_cast<uintptr_t>(g.dy)) & 3u) == 0;
+        s = bwd_gated_shape(pairs_aligned ? s.V : 1);
+    }
+    const int nseg = ceil_div(T, s.rows());
+    const int nct = ceil_div(D, s.chans());
+    const WsLayout l = layout_for(B, D, nseg, nseg);
+    if (ws == nullptr || ws_bytes < l.total) return HAWK_ERR_WORKSPACE;
+    const ScanWsPtrs p = carve(ws, l);
+    int rc;
+    if (in_dtype == HAWK_DTYPE_BF16) {
+        if (s.V == 2)
+            rc = launch_bwd<bf16_t, bf16_t, 2, TC2, kBwdNW, false, GATED>(x, xg, ag, lam, hs, gout, dx, dxg, dag, g, B, T,
+                                                                         D, nseg, nct, p, st);
+        else
+            rc = launch_bwd<bf16_t, bf16_t, 1, TC1, kBwdNW, false, GATED>(x, xg, ag, lam, hs, gout, dx, dxg, dag, g, B, T,
+                                                                         D, nseg, nct, p, st);
+    } else if (state_dtype == HAWK_DTYPE_BF16) {
+        rc = launch_bwd<float, bf16_t, 1, TC1, kBwdNW, false, GATED>(x, xg, ag, lam, hs, gout, dx, dxg, dag, g, B, T, D,
+                                                                    nseg, nct, p, st);
+    } else {
+        rc = launch_bwd<float, float, 1, TC1, kBwdNW, true, GATED>(x, xg, ag, lam, hs, gout, dx, dxg, dag, g, B, T, D,
+                                                                  nseg, nct, p, st);
+    }
+    if (rc != HAWK_OK) return rc;
+    hipLaunchKernelGGL(dlam_reduce_kernel, dim3((unsigned)ceil_div(D, kWave)), dim3(1024), 0, st, p.dlam_part, lam,
+                       dlam, nseg * B, D);
     return hipGetLastError() == hipSuccess ? HAWK_OK : HAWK_ERR_LAUNCH;
 }
 
 }  // namespace
 
 size_t scan_workspace_bytes(int B, int T, int D, int dtype) {
-    const TileShape f = fwd_shape(D, dtype), r = bwd_shape(D, dtype);
-    const int nf = ceil_div(T, f.rows()), nr = ceil_div(T, r.rows());
-    return layout_for(B, D, nf > nr ? nf : nr, nr).total;
+    // one size serves every scan entry point: the longest chain (shortest tile) decides
+    const int rows[3] = {fwd_shape(D, dtype).rows(), bwd_shape(D, dtype).rows(), bwd_gated_shape(1).rows()};
+    int n_chain = 0, n_dlam = 0;
+    for (int k = 0; k < 3; ++k) {
+        const int n = ceil_div(T, rows[k]);
+        if (n > n_chain) n_chain = n;
+        if (k > 0 && n > n_dlam) n_dlam = n;
+    }
+    return layout_for(B, D, n_chain, n_dlam).total;
 }
 
 int workspace_init(void* ws, size_t bytes, hipStream_t st) {
@@ -727,53 +960,38 @@ bool scan_dtypes_supported(int in_dtype, int state_dtype) {
 
 int scan_fwd(const void* x, const void* xg, const void* ag, const float* lam, void* h, int B, int T, int D,
              int in_dtype, int out_dtype, void* ws, size_t ws_bytes, hipStream_t st) {
-    const TileShape s = fwd_shape(D, in_dtype);
-    const int nseg = ceil_div(T, s.rows());
-    const int nct = ceil_div(D, s.chans());
-    ScanWsPtrs p = {};
-    if (nseg > 1) {
-        const WsLayout l = layout_for(B, D, nseg, 0);
-        if (ws == nullptr || ws_bytes < l.total) return HAWK_ERR_WORKSPACE;
-        p = carve(ws, l);
-    }
-    if (in_dtype == HAWK_DTYPE_BF16) {
-        if (s.V == 2)
-            return launch_fwd<bf16_t, bf16_t, 2, kFwdTC, kFwdNW, false>(x, xg, ag, lam, h, B, T, D, nseg, nct, p, st);
-        return launch_fwd<bf16_t, bf16_t, 1, kFwdTC, kFwdNW, false>(x, xg, ag, lam, h, B, T, D, nseg, nct, p, st);
-    }
-    if (out_dtype == HAWK_DTYPE_BF16)
-        return launch_fwd<float, bf16_t, 1, kFwdTC, kFwdNW, false>(x, xg, ag, lam, h, B, T, D, nseg, nct, p, st);
-    return launch_fwd<float, float, 1, kFwdTC, kFwdNW, true>(x, xg, ag, lam, h, B, T, D, nseg, nct, p, st);
+    return scan_fwd_impl<false>(x, xg, ag, lam, h, GateFwdHost{}, B, T, D, in_dtype, out_dtype, ws, ws_bytes, st);
 }
 
 int scan_bwd(const void* x, const void* xg, const void* ag, const float* lam, const void* hs, const void* gout,
              void* dx, void* dxg, void* dag, float* dlam, int B, int T, int D, int in_dtype, int state_dtype,
              void* ws, size_t ws_bytes, hipStream_t st) {
-    const TileShape s = bwd_shape(D, in_dtype);
-    const int nseg = ceil_div(T, s.rows());
-    const int nct = ceil_div(D, s.chans());
-    const WsLayout l = layout_for(B, D, nseg, nseg);
-    if (ws == nullptr || ws_bytes < l.total) return HAWK_ERR_WORKSPACE;
-    const ScanWsPtrs p = carve(ws, l);
-    int rc;
-    if (in_dtype == HAWK_DTYPE_BF16) {
-        if (s.V == 2)
-            rc = launch_bwd<bf16_t, bf16_t, 2, kBwdTC, kBwdNW, false>(x, xg, ag, lam, hs, gout, dx, dxg, dag, B, T, D,
-                                                                      nseg, nct, p, st);
-        else
-            rc = launch_bwd<bf16_t, bf16_t, 1, kBwdTC, kBwdNW, false>(x, xg, ag, lam, hs, gout, dx, dxg, dag, B, T, D,
-                                                                      nseg, nct, p, st);
-    } else if (state_dtype == HAWK_DTYPE_BF16) {
-        rc = launch_bwd<float, bf16_t, 1, kBwdTC, kBwdNW, false>(x, xg, ag, lam, hs, gout, dx, dxg, dag, B, T, D, nseg,
-                                                                 nct, p, st);
-    } else {
-        rc = launch_bwd<float, float, 1, kBwdTC, kBwdNW, true>(x, xg, ag, lam, hs, gout, dx, dxg, dag, B, T, D, nseg,
-                                                               nct, p, st);
-    }
-    if (rc != HAWK_OK) return rc;
-    hipLaunchKernelGGL(dlam_reduce_kernel, dim3((unsigned)ceil_div(D, kWave)), dim3(1024), 0, st, p.dlam_part, lam,
-                       dlam, nseg * B, D);
-    return hipGetLastError() == hipSuccess ? HAWK_OK : HAWK_ERR_LAUNCH;
+    return scan_bwd_impl<false>(x, xg, ag, lam, hs, gout, dx, dxg, dag, dlam, GateBwdHost{}, B, T, D, in_dtype,
+                                state_dtype, ws, ws_bytes, st);
+}
+
+int scan_gated_fwd(const void* x, const void* xg, const void* ag, const float* lam, const void* y, long long ldy,
+                   void* h, void* out, void* h_last, int B, int T, int D, int in_dtype, int out_dtype, void* ws,
+                   size_t ws_bytes, hipStream_t st) {
+    GateFwdHost g;
+    g.y = y;
+    g.out = out;
+    g.h_last = h_last;
+    g.ldy = (uint32_t)ldy;
+    return scan_fwd_impl<true>(x, xg, ag, lam, h, g, B, T, D, in_dtype, out_dtype, ws, ws_bytes, st);
+}
+
+int scan_gated_bwd(const void* x, const void* xg, const void* ag, const float* lam, const void* y, long long ldy,
+                   const void* hs, const void* gout, void* dx, void* dxg, void* dag, void* dy, long long lddy,
+                   float* dlam, int B, int T, int D, int in_dtype, int state_dtype, void* ws, size_t ws_bytes,
+                   hipStream_t st) {
+    GateBwdHost g;
+    g.y = y;
+    g.dy = dy;
+    g.ldy = (uint32_t)ldy;
+    g.lddy = (uint32_t)lddy;
+    return scan_bwd_impl<true>(x, xg, ag, lam, hs, gout, dx, dxg, dag, dlam, g, B, T, D, in_dtype, state_dtype, ws,
+                               ws_bytes, st);
 }
 
 }  // namespace hawk

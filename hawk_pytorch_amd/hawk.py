@@ -8,7 +8,9 @@ PyTorch-ROCm modules (library GEMMs); the loss is plain ``F.cross_entropy``.
 
 What differs from upstream is confined to the recurrent block:
 
-* prefill and training call ``Conv1D`` and ``fused_linear_scan`` from this package;
+* prefill and training call ``Conv1D`` and the scan from this package; with
+  ``HawkConfig.fused_epilogue`` (default) the scan kernel also applies the block's gate,
+  ``gelu(y) * h``, and its backward also produces the gate's gradient;
 * decode (``use_cache=True`` with a warm ``RNNCache``) issues two fused kernels per layer
   (conv window roll + conv, RG-LRU state update) instead of about thirty eager ones, works
   for any batch size, and evaluates the two gate projections once instead of twice.
@@ -26,7 +28,7 @@ import torch.nn.functional as F
 
 from .cache import RNNCache
 from .external import BlockDiagonalLinear, Conv1D, rglru_step, rnn_param_init
-from .scan_fused import fused_linear_scan
+from .scan_fused import fused_linear_scan, fused_linear_scan_gated
 
 
 @dataclass
@@ -40,6 +42,8 @@ class HawkConfig:
     conv_width: int = 4
     # accepted for compatibility with upstream's README snippet; only False is implemented
     post_norm: bool = False
+    # not an upstream field: apply gelu(y) * h inside the scan kernels (hawk/hawk.py:134-135)
+    fused_epilogue: bool = True
 
     def __post_init__(self):
         if self.post_norm:
@@ -122,11 +126,16 @@ class Hawk(nn.Module):
                 assert layer_past is not None, "use_cache=True needs one RNNCache per layer in layer_past"
                 layer_past.seed_conv_state(branch)
             u = self.conv1d(branch)
-            h = fused_linear_scan(u, self.rg_lru_input_gate(u), self.rg_lru_a_gate(u), self.rg_lru_a_param.float())
-            cache = None
+            gates = (self.rg_lru_input_gate(u), self.rg_lru_a_gate(u), self.rg_lru_a_param.float())
+            cache = layer_past if self.use_cache else None
+            if self.config.fused_epilogue:
+                gated, h_last = fused_linear_scan_gated(u, *gates, gate_branch, return_last_state=True)
+                if self.use_cache:
+                    layer_past.update_cache(h_last)
+                return self.resid_proj(gated), cache
+            h = fused_linear_scan(u, *gates)
             if self.use_cache:
                 layer_past.update_cache(h[:, -1:, :])
-                cache = layer_past
 
         return self.resid_proj(F.gelu(gate_branch) * h), cache
 

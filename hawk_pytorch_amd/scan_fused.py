@@ -8,6 +8,10 @@ Public surface mirrors the upstream operator boundary (hawk/scan_fused.py:319-44
     DiagonalRecurrence            torch.autograd.Function
     fused_linear_scan             = DiagonalRecurrence.apply
 
+and, beyond upstream, the scan fused with the block's gate (hawk/hawk.py:134-135, :186):
+
+    fused_linear_scan_gated(x, x_rg_lru, a_rg_lru, a_param, y) -> gelu(y) * h
+
 Differences from upstream, all deliberate:
 
 * Under autocast, fp32 activations are NOT first cast to bf16 by three extra kernels
@@ -231,3 +235,187 @@ class DiagonalRecurrence(Function):
 
 
 fused_linear_scan = DiagonalRecurrence.apply
+
+
+# ---------------------------------------------------------------------------------------
+# Scan fused with the block's gate: out = gelu(y) * h  (hawk/hawk.py:134-135 applied to the
+# scan's result, :186).  y is usually one half of a wider projection, so it is taken in
+# place when its rows are evenly spaced.
+# ---------------------------------------------------------------------------------------
+def _row_stride(t: torch.Tensor):
+    """Elements between consecutive rows of a [B, T, D] tensor whose row r = b*T + t starts at
+    r * stride, or None when t is not laid out that way."""
+    b, sq, d = t.shape
+    if t.stride(2) != 1 and d > 1:
+        return None
+    if sq > 1:
+        ld = t.stride(1)
+    elif b > 1:
+        ld = t.stride(0)
+    else:
+        ld = d
+    if ld < d or (b > 1 and t.stride(0) != sq * ld):
+        return None
+    return ld
+
+
+def _launch_scan_gated_fwd(x, x_rg_lru, a_rg_lru, a_param, y, h_bf16: bool, want_h: bool, want_last: bool):
+    dev = _lib.require_cuda(x, x_rg_lru, a_rg_lru, a_param, y)
+    x, x_rg_lru, a_rg_lru, a_param = (_lib.dense16(t) for t in (x, x_rg_lru, a_rg_lru, a_param))
+    b, sq, d = x.shape
+    in_code = _lib.dtype_code(x.dtype)
+    out_dtype = torch.bfloat16 if h_bf16 else x.dtype
+    if y.dtype != out_dtype:
+        y = y.to(out_dtype)
+    ldy = _row_stride(y)
+    if ldy is None:
+        y = _lib.dense16(y)
+        ldy = d
+    lib = _lib.load()
+    out = torch.empty((b, sq, d), dtype=out_dtype, device=dev)
+    h = torch.empty((b, sq, d) if want_h else (0,), dtype=out_dtype, device=dev)
+    h_last = torch.empty((b, 1, d) if want_last else (0,), dtype=out_dtype, device=dev)
+    nbytes = lib.hawk_scan_workspace_bytes(b, sq, d, in_code)
+    ws = _lib.scan_workspace(dev, nbytes)
+    with torch.cuda.device(dev):
+        status = lib.hawk_rglru_scan_gated_fwd(
+            x.data_ptr(), x_rg_lru.data_ptr(), a_rg_lru.data_ptr(), a_param.data_ptr(), y.data_ptr(), ldy,
+            h.data_ptr() if want_h else None, out.data_ptr(), h_last.data_ptr() if want_last else None,
+            b, sq, d, in_code, _lib.dtype_code(out_dtype), ws.data_ptr(), ws.numel(), _lib.stream_ptr(dev),
+        )
+    _lib.check("hawk_rglru_scan_gated_fwd", status)
+    return out, h, h_last
+
+
+def _launch_scan_gated_bwd(x, x_rg_lru, a_rg_lru, a_param, y, h_saved, grad_out):
+    dev = _lib.require_cuda(x, x_rg_lru, a_rg_lru, a_param, y, h_saved, grad_out)
+    x, x_rg_lru, a_rg_lru, a_param, h_saved, grad_out = (
+        _lib.dense16(t) for t in (x, x_rg_lru, a_rg_lru, a_param, h_saved, grad_out)
+    )
+    b, sq, d = x.shape
+    in_code = _lib.dtype_code(x.dtype)
+    if y.dtype != h_saved.dtype:
+        y = y.to(h_saved.dtype)
+    ldy = _row_stride(y)
+    if ldy is None:
+        y = _lib.dense16(y)
+        ldy = d
+    lib = _lib.load()
+    dx = torch.empty_like(x)
+    dxg = torch.empty_like(x)
+    dag = torch.empty_like(x)
+    dy = torch.empty((b, sq, d), dtype=h_saved.dtype, device=dev)
+    dlam = torch.empty(d, dtype=torch.float32, device=dev)
+    nbytes = lib.hawk_scan_workspace_bytes(b, sq, d, in_code)
+    ws = _lib.scan_workspace(dev, nbytes)
+    with torch.cuda.device(dev):
+        status = lib.hawk_rglru_scan_gated_bwd(
+            x.data_ptr(), x_rg_lru.data_ptr(), a_rg_lru.data_ptr(), a_param.data_ptr(), y.data_ptr(), ldy,
+            h_saved.data_ptr(), grad_out.data_ptr(), dx.data_ptr(), dxg.data_ptr(), dag.data_ptr(),
+            dy.data_ptr(), d, dlam.data_ptr(), b, sq, d, in_code, _lib.dtype_code(h_saved.dtype),
+            ws.data_ptr(), ws.numel(), _lib.stream_ptr(dev),
+        )
+    _lib.check("hawk_rglru_scan_gated_bwd", status)
+    return dx, dxg, dag, dlam, dy
+
+
+@torch.library.custom_op("hawk_amd::rglru_scan_gated_fwd", mutates_args=(), device_types="cuda")
+def _rglru_scan_gated_fwd_op(
+    x: torch.Tensor,
+    x_rg_lru: torch.Tensor,
+    a_rg_lru: torch.Tensor,
+    a_param: torch.Tensor,
+    y: torch.Tensor,
+    h_bf16: bool,
+    want_h: bool,
+    want_last: bool,
+) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    return _launch_scan_gated_fwd(x, x_rg_lru, a_rg_lru, a_param, y, h_bf16, want_h, want_last)
+
+
+@_rglru_scan_gated_fwd_op.register_fake
+def _(x, x_rg_lru, a_rg_lru, a_param, y, h_bf16, want_h, want_last):
+    dt = torch.bfloat16 if h_bf16 else x.dtype
+    b, sq, d = x.shape
+    return (
+        torch.empty((b, sq, d), dtype=dt, device=x.device),
+        torch.empty((b, sq, d) if want_h else (0,), dtype=dt, device=x.device),
+        torch.empty((b, 1, d) if want_last else (0,), dtype=dt, device=x.device),
+    )
+
+
+@torch.library.custom_op("hawk_amd::rglru_scan_gated_bwd", mutates_args=(), device_types="cuda")
+def _rglru_scan_gated_bwd_op(
+    x: torch.Tensor,
+    x_rg_lru: torch.Tensor,
+    a_rg_lru: torch.Tensor,
+    a_param: torch.Tensor,
+    y: torch.Tensor,
+    h_saved: torch.Tensor,
+    grad_out: torch.Tensor,
+) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+    return _launch_scan_gated_bwd(x, x_rg_lru, a_rg_lru, a_param, y, h_saved, grad_out)
+
+
+@_rglru_scan_gated_bwd_op.register_fake
+def _(x, x_rg_lru, a_rg_lru, a_param, y, h_saved, grad_out):
+    e = lambda: torch.empty_like(x, memory_format=torch.contiguous_format)  # noqa: E731
+    return (
+        e(), e(), e(),
+        torch.empty(x.shape[-1], dtype=torch.float32, device=x.device),
+        torch.empty(x.shape, dtype=h_saved.dtype, device=x.device),
+    )
+
+
+class GatedDiagonalRecurrence(Function):
+    """(out, h_last) = (gelu(y) * h, h[:, -1:]) with h = scan(x, x_rg_lru, a_rg_lru, a_param).
+
+    One kernel per direction instead of the scan, a GELU and a product (and their three
+    autograd mirrors).  Dtype rules are DiagonalRecurrence's; y and out have h's dtype.
+    The state sequence h is written only when a gradient will be asked for; h_last (what
+    the decode cache keeps, hawk/hawk.py:190) is not differentiable.
+    """
+
+    @staticmethod
+    def forward(ctx, x, x_rg_lru, a_rg_lru, a_param, y, want_last):
+        in_dtype = _common_input_dtype(x, x_rg_lru, a_rg_lru)
+        xc, xgc, agc = (t if t.dtype == in_dtype else t.to(in_dtype) for t in (x, x_rg_lru, a_rg_lru))
+        autocast = torch.is_autocast_enabled("cuda")
+        _check_shapes(xc, xgc, agc, a_param)
+        assert y.shape == x.shape, f"Error: expected y of shape {tuple(x.shape)}, got {tuple(y.shape)}"
+        xc, xgc, agc = _prepare(xc, xgc, agc)
+        lam = a_param.float().contiguous()
+        h_bf16 = autocast or in_dtype == torch.bfloat16
+        want_h = any(ctx.needs_input_grad[:5])
+        out, h, h_last = _rglru_scan_gated_fwd_op(xc, xgc, agc, lam, y, h_bf16, want_h, bool(want_last))
+        if want_h:
+            ctx.save_for_backward(xc, xgc, agc, a_param, y, h)
+        ctx.y_dtype = y.dtype
+        ctx.mark_non_differentiable(h_last)
+        if not autocast and x.dtype not in (torch.bfloat16, torch.float32):
+            out, h_last = out.to(x.dtype), h_last.to(x.dtype)
+        return out, h_last
+
+    @staticmethod
+    def backward(ctx, grad_out, _grad_last):  # type: ignore[override]
+        (x, x_rg_lru, a_rg_lru, a_param, y, h_saved) = ctx.saved_tensors
+        if not grad_out.is_contiguous():
+            grad_out = grad_out.contiguous()
+        if grad_out.dtype != h_saved.dtype:
+            grad_out = grad_out.to(h_saved.dtype)
+        dx, dxg, dag, dlam, dy = _rglru_scan_gated_bwd_op(
+            x, x_rg_lru, a_rg_lru, a_param.float().contiguous(), y, h_saved, grad_out
+        )
+        if dy.dtype != ctx.y_dtype:
+            dy = dy.to(ctx.y_dtype)
+        return dx, dxg, dag, dlam.to(a_param.dtype), dy, None
+
+
+def fused_linear_scan_gated(x, x_rg_lru, a_rg_lru, a_param, y, return_last_state: bool = False):
+    """gelu(y) * fused_linear_scan(x, x_rg_lru, a_rg_lru, a_param) in one kernel per direction.
+
+    With ``return_last_state`` also returns h[:, -1:, :] (shape [B, 1, D]), the recurrent
+    state a decode cache keeps after prefill.
+    """
+    out, h_last = GatedDiagonalRecurrence.apply(x, x_rg_lru, a_rg_lru, a_param, y, return_last_state)
+    return (out, h_last) if return_last_state else out

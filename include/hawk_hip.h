@@ -102,6 +102,37 @@ int hawk_rglru_scan_bwd_mixed(const void* x, const void* x_rg_lru, const void* a
                               int B, int T, int D, int in_dtype, int state_dtype,
                               void* workspace_device, size_t workspace_bytes, void* stream);
 
+/* Scan fused with the step that follows it in a Hawk block, out = gelu(y) * h with the
+ * exact (erf) GELU (Hawk.epilogue before its projection, hawk/hawk.py:134-135, applied to
+ * the scan's result at hawk/hawk.py:186).  Dtypes as in the mixed variants; y, out, h_last
+ * and dy have the out / state dtype.
+ *   y        [B,T,D] gate input; rows are ldy >= D elements apart and batches T rows apart,
+ *            so the second half of the fused projection of hawk/hawk.py:164-166 can be
+ *            passed in place (ldy = 2 D).  y and dy need only be aligned to their element
+ *            size; 4-byte alignment and even row strides let bf16 move as pairs.
+ *   h        [B,T,D] dense, or NULL when the state sequence is not needed (no backward)
+ *   out      [B,T,D] dense
+ *   h_last   [B,D] or NULL: h at t = T-1, what RNNCache.update_cache keeps (hawk.py:190)
+ * Forward: reads 4 tensors, writes 1 or 2, where the unfused sequence reads 5 and writes 2. */
+int hawk_rglru_scan_gated_fwd(const void* x, const void* x_rg_lru, const void* a_rg_lru,
+                              const float* a_param, const void* y, long long ldy, void* h,
+                              void* out, void* h_last, int B, int T, int D, int in_dtype,
+                              int out_dtype, void* workspace_device, size_t workspace_bytes,
+                              void* stream);
+
+/* Backward of the above.  grad_out is the gradient of `out`; dy [B,T,D] (rows lddy >= D
+ * elements apart) receives grad_out * h * gelu'(y); the other outputs are as in
+ * hawk_rglru_scan_bwd.  Replaces the autograd of gelu and of the product together with
+ * sequential_scan_backward (hawk/scan_fused.py:363-424): reads 6 tensors and writes 4
+ * where the unfused sequence reads 8 and writes 5. */
+int hawk_rglru_scan_gated_bwd(const void* x, const void* x_rg_lru, const void* a_rg_lru,
+                              const float* a_param, const void* y, long long ldy,
+                              const void* h_saved, const void* grad_out, void* dx,
+                              void* dx_rg_lru, void* da_rg_lru, void* dy, long long lddy,
+                              float* da_param, int B, int T, int D, int in_dtype,
+                              int state_dtype, void* workspace_device, size_t workspace_bytes,
+                              void* stream);
+
 /* ---------------------------------------------------------------------------------------
  * Temporal causal depthwise conv1d.
  *   y[b,t,c] = bias[c] + sum_{s<W} w[W-1-s,c] x[b,t-s,c]

@@ -137,3 +137,42 @@ def conv1d_step(conv_state, x_new, w, b, precision: str = "f64"):
     fn = getattr(_load(), f"oracle_conv1d_step_{precision}")
     fn(_ptr(st), _ptr(xn), _ptr(w), _ptr(b), _ptr(y), B, D, W)
     return y, st
+
+
+# ---------------------------------------------------------------------------------------
+# Scan followed by the block's gate, out = gelu(y) * h (restates Hawk.epilogue before its
+# projection, hawk/hawk.py:134-135: F.gelu with its default, the exact erf form).
+# ---------------------------------------------------------------------------------------
+def gelu(y):
+    """y * Phi(y), Phi the standard normal CDF (= 0.5 (1 + erf(y / sqrt 2)))."""
+    from scipy.special import ndtr
+
+    y = np.asarray(y, dtype=np.float64)
+    return y * ndtr(y)
+
+
+def gelu_grad(y):
+    """d gelu / dy = Phi(y) + y exp(-y^2 / 2) / sqrt(2 pi)."""
+    from scipy.special import ndtr
+
+    y = np.asarray(y, dtype=np.float64)
+    return ndtr(y) + y * np.exp(-0.5 * y * y) / np.sqrt(2.0 * np.pi)
+
+
+def rglru_scan_gated_fwd(x, x_rg_lru, a_rg_lru, a_param, y):
+    """(h, out) with out = gelu(y) * h; fp64."""
+    h = rglru_scan_fwd(x, x_rg_lru, a_rg_lru, a_param)
+    return h, gelu(y) * h
+
+
+def rglru_scan_gated_bwd(x, x_rg_lru, a_rg_lru, a_param, y, h_saved, grad_out):
+    """(dx, dx_rg_lru, da_rg_lru, dLambda, dy) for out = gelu(y) * h; fp64.
+
+    The product rule in front of rglru_scan_bwd: the gradient reaching h is
+    grad_out * gelu(y), and dy = grad_out * h * gelu'(y) with the saved h.
+    """
+    go = np.asarray(grad_out, dtype=np.float64)
+    hs = np.asarray(h_saved, dtype=np.float64)
+    dy = go * hs * gelu_grad(y)
+    dx, dxg, dag, dlam = rglru_scan_bwd(x, x_rg_lru, a_rg_lru, a_param, hs, go * gelu(y))
+    return dx, dxg, dag, dlam, dy

@@ -146,3 +146,44 @@ def rglru_step(x, xg, ag, lam, state):
         _lib.dtype_code(x.dtype), _lib.dtype_code(state.dtype), _stream())
     _lib.check("hawk_rglru_step", rc)
     return h
+
+
+def scan_gated_fwd(x, xg, ag, lam, y, out_dtype=None, want_h=True, want_last=True, ws=None):
+    """y: [B,T,D] view with unit channel stride and evenly spaced rows (may be a slice of a
+    wider tensor).  Returns (out, h or None, h_last or None)."""
+    B, T, D = x.shape
+    out_dtype = out_dtype or x.dtype
+    assert y.dtype == out_dtype and y.stride(2) == 1
+    ldy = y.stride(1) if T > 1 else (y.stride(0) if B > 1 else D)
+    assert B == 1 or y.stride(0) == T * ldy
+    out = torch.empty((B, T, D), dtype=out_dtype, device="cuda")
+    h = torch.empty((B, T, D), dtype=out_dtype, device="cuda") if want_h else None
+    h_last = torch.full((B, D), float("nan"), dtype=out_dtype, device="cuda") if want_last else None
+    if ws is None:
+        ws = new_workspace(B, T, D, "bf16" if x.dtype == torch.bfloat16 else "f32")
+    rc = _lib.load().hawk_rglru_scan_gated_fwd(
+        x.data_ptr(), xg.data_ptr(), ag.data_ptr(), lam.data_ptr(), y.data_ptr(), ldy,
+        _lib.ptr(h), out.data_ptr(), _lib.ptr(h_last), B, T, D, _lib.dtype_code(x.dtype),
+        _lib.dtype_code(out_dtype), ws.data_ptr(), ws.numel(), _stream())
+    _lib.check("hawk_rglru_scan_gated_fwd", rc)
+    return out, h, h_last
+
+
+def scan_gated_bwd(x, xg, ag, lam, y, h, gout, dy=None, ws=None):
+    """dy: optional preallocated [B,T,D] view with evenly spaced rows to receive the gate's gradient."""
+    B, T, D = x.shape
+    assert y.dtype == h.dtype and gout.dtype == h.dtype
+    ldy = y.stride(1) if T > 1 else (y.stride(0) if B > 1 else D)
+    dx, dxg, dag = torch.empty_like(x), torch.empty_like(x), torch.empty_like(x)
+    if dy is None:
+        dy = torch.empty((B, T, D), dtype=h.dtype, device="cuda")
+    lddy = dy.stride(1) if T > 1 else (dy.stride(0) if B > 1 else D)
+    dlam = torch.empty(D, dtype=torch.float32, device="cuda")
+    if ws is None:
+        ws = new_workspace(B, T, D, "bf16" if x.dtype == torch.bfloat16 else "f32")
+    rc = _lib.load().hawk_rglru_scan_gated_bwd(
+        x.data_ptr(), xg.data_ptr(), ag.data_ptr(), lam.data_ptr(), y.data_ptr(), ldy, h.data_ptr(),
+        gout.data_ptr(), dx.data_ptr(), dxg.data_ptr(), dag.data_ptr(), dy.data_ptr(), lddy, dlam.data_ptr(),
+        B, T, D, _lib.dtype_code(x.dtype), _lib.dtype_code(h.dtype), ws.data_ptr(), ws.numel(), _stream())
+    _lib.check("hawk_rglru_scan_gated_bwd", rc)
+    return dx, dxg, dag, dlam, dy

@@ -63,6 +63,50 @@ def test_fused_linear_scan_under_autocast_bf16_state_fp32_inputs_and_lambda():
     assert hb.dtype == torch.bfloat16 and xb.grad.dtype == torch.bfloat16
 
 
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_fused_linear_scan_gated_autograd_with_y_as_half_of_a_projection(dtype):
+    (x, xg, ag), lam, gout = _leaves(2, 300, 128, dtype, seed=6)
+    wide = torch.randn(2, 300, 256, device="cuda").to(x.dtype).requires_grad_(True)
+    y = wide.chunk(2, dim=-1)[1]  # strided view, as hawk/hawk.py:166 hands it over
+    out, h_last = hk.fused_linear_scan_gated(x, xg, ag, lam, y, return_last_state=True)
+    assert out.dtype == x.dtype and out.shape == x.shape and h_last.shape == (2, 1, 128)
+    assert not h_last.requires_grad
+    out.backward(gout)
+    xr, xgr, agr, yr = (capi.to_np(t) for t in (x, xg, ag, y))
+    h_ref, out_ref = oracle.rglru_scan_gated_fwd(xr, xgr, agr, capi.to_np(lam), yr)
+    assert max_rel(capi.to_np(out), out_ref) < TOL[dtype]
+    assert max_rel(capi.to_np(h_last), h_ref[:, -1:, :]) < TOL[dtype]
+    h_saved = capi.to_np(hk.fused_linear_scan(x.detach(), xg.detach(), ag.detach(), lam.detach()))
+    ref = oracle.rglru_scan_gated_bwd(xr, xgr, agr, capi.to_np(lam), yr, h_saved, capi.to_np(gout))
+    for t, want in zip((x, xg, ag, lam), ref[:4]):
+        assert t.grad is not None and t.grad.dtype == t.dtype
+        assert max_rel(capi.to_np(t.grad), want) < TOL[dtype]
+    assert max_rel(capi.to_np(wide.grad[..., 128:]), ref[4]) < TOL[dtype]
+    assert torch.all(wide.grad[..., :128] == 0)
+    # without a gradient the state sequence is not even written; the result is the same
+    with torch.no_grad():
+        out2 = hk.fused_linear_scan_gated(x, xg, ag, lam, y)
+    assert torch.equal(out2, out)
+
+
+def test_fused_linear_scan_gated_under_autocast():
+    (x, xg, ag), lam, gout = _leaves(1, 200, 64, "f32", seed=7)
+    y = torch.randn(1, 200, 64, device="cuda").bfloat16().requires_grad_(True)  # a linear's output under autocast
+    with torch.autocast(device_type="cuda", dtype=torch.bfloat16):
+        out = hk.fused_linear_scan_gated(x, xg, ag, lam, y)
+    assert out.dtype == torch.bfloat16
+    out.backward(gout.bfloat16())
+    assert x.grad.dtype == torch.float32 and y.grad.dtype == torch.bfloat16 and lam.grad.dtype == torch.float32
+    xr, xgr, agr, yr = (capi.to_np(t) for t in (x, xg, ag, y))
+    _, out_ref = oracle.rglru_scan_gated_fwd(xr, xgr, agr, capi.to_np(lam), yr)
+    assert max_rel(capi.to_np(out), out_ref) < TOL["bf16"]
+    with torch.autocast(device_type="cuda", dtype=torch.bfloat16):
+        h_saved = capi.to_np(hk.fused_linear_scan(x.detach(), xg.detach(), ag.detach(), lam.detach()))
+    ref = oracle.rglru_scan_gated_bwd(xr, xgr, agr, capi.to_np(lam), yr, h_saved, capi.to_np(gout.bfloat16()))
+    for t, want in zip((x, xg, ag, lam, y), ref):
+        assert max_rel(capi.to_np(t.grad), want) < TOL["bf16"]
+
+
 def test_scan_wrapper_contract_errors_and_copies():
     (x, xg, ag), lam, gout = _leaves(1, 20, 64, "f32", seed=3)
     with pytest.raises(AssertionError, match="multiple of 64"):
@@ -173,11 +217,13 @@ def test_model_prefill_then_decode_matches_full_forward():
             assert max_rel(capi.to_np(step_logits[:, 0]), capi.to_np(full_logits[:, T + k])) < 1e-3
 
 
-def test_model_gradients_match_a_pure_torch_model_of_the_same_weights():
+@pytest.mark.parametrize("fused_epilogue", [True, False])
+def test_model_gradients_match_a_pure_torch_model_of_the_same_weights(fused_epilogue):
     """End-to-end fwd+bwd of the small model in fp32 against the same model with the scan
     and conv swapped for the torch-loop oracle pieces."""
     torch.manual_seed(2)
     cfg = _small_config()
+    cfg.fused_epilogue = fused_epilogue
     model = hk.HawkModel(cfg).cuda()
     _randomise_zero_inits(model)
     ids = torch.randint(1, cfg.vocab_size, (2, 48), device="cuda")
@@ -191,18 +237,23 @@ def test_model_gradients_match_a_pure_torch_model_of_the_same_weights():
     def ref_scan(x, xg, ag, lam):
         return rglru_torch.rglru_scan_loop(x, xg, ag, lam)
 
+    def ref_scan_gated(x, xg, ag, lam, y, return_last_state=False):
+        h = rglru_torch.rglru_scan_loop(x, xg, ag, lam)
+        out = F.gelu(y) * h
+        return (out, h[:, -1:, :].detach()) if return_last_state else out
+
     def ref_conv(self, x, state=None):
         return rglru_torch.conv1d_library(x, self.w, self.b)
 
     model.zero_grad()
-    old_scan, old_conv = hm.fused_linear_scan, he.Conv1D.forward
+    old = hm.fused_linear_scan, hm.fused_linear_scan_gated, he.Conv1D.forward
     try:
-        hm.fused_linear_scan = ref_scan
+        hm.fused_linear_scan, hm.fused_linear_scan_gated = ref_scan, ref_scan_gated
         he.Conv1D.forward = ref_conv
         ref_loss = model(ids, ids)
         ref_loss.backward()
     finally:
-        hm.fused_linear_scan, he.Conv1D.forward = old_scan, old_conv
+        hm.fused_linear_scan, hm.fused_linear_scan_gated, he.Conv1D.forward = old
     assert abs(float(loss) - float(ref_loss)) < 1e-4
     for n, p in model.named_parameters():
         assert max_rel(capi.to_np(got[n]), capi.to_np(p.grad)) < 1e-3, n
@@ -224,3 +275,24 @@ def test_torch_compile_traces_the_ops_without_graph_breaks():
     x.grad = None
     fn(x, xg, ag, lam).backward(gout)
     assert torch.allclose(g_compiled, x.grad, atol=1e-6)
+
+
+def test_torch_compile_traces_the_gated_scan_without_graph_breaks():
+    (x, xg, ag), lam, gout = _leaves(1, 70, 64, "f32", seed=4)
+    lin = torch.nn.Linear(64, 128, bias=False).cuda()
+
+    def fn(x, xg, ag, lam):
+        branch, gate = lin(x).chunk(2, dim=-1)
+        out, h_last = hk.fused_linear_scan_gated(branch, xg, ag, lam, gate, return_last_state=True)
+        return out, h_last
+
+    eager, eager_last = fn(x, xg, ag, lam)
+    compiled = torch.compile(fn, backend="aot_eager", fullgraph=True)
+    out, last = compiled(x, xg, ag, lam)
+    assert torch.allclose(out, eager, atol=1e-6) and torch.allclose(last, eager_last, atol=1e-6)
+    out.backward(gout)
+    g_compiled, w_compiled = x.grad.clone(), lin.weight.grad.clone()
+    x.grad, lin.weight.grad = None, None
+    fn(x, xg, ag, lam)[0].backward(gout)
+    assert torch.allclose(g_compiled, x.grad, atol=1e-5)
+    assert torch.allclose(w_compiled, lin.weight.grad, atol=1e-4)

@@ -222,3 +222,33 @@ def test_f32_port_tracks_f64():
     g32 = oracle.rglru_scan_bwd(x, xg, ag, lam, h64, gout, precision="f32")
     for a, b in zip(g32, g64):
         assert max_rel(a, b) < 1e-3
+
+
+# ------------------------------------------------------------------------------ gated epilogue
+def test_gelu_and_its_derivative_match_the_library_routine():
+    y = np.concatenate([np.linspace(-9.0, 9.0, 2001), [0.0, -0.0, 1e-8, -1e-8, 30.0, -30.0]])
+    t = torch.from_numpy(y).requires_grad_(True)
+    g = torch.nn.functional.gelu(t)  # exact (erf) form, the default used at hawk/hawk.py:135
+    (dg,) = torch.autograd.grad(g.sum(), t)
+    # the library evaluates 0.5 y (1 + erf(y / sqrt 2)), which cancels in the far negative tail;
+    # the oracle uses the normal CDF directly, hence the absolute floor
+    np.testing.assert_allclose(oracle.gelu(y), g.detach().numpy(), rtol=1e-12, atol=2e-15)
+    np.testing.assert_allclose(oracle.gelu_grad(y), dg.numpy(), rtol=1e-10, atol=2e-15)
+    # closed-form anchors: gelu(0) = 0, gelu'(0) = 1/2, gelu(y) - gelu(-y) = y
+    assert oracle.gelu(0.0) == 0.0 and oracle.gelu_grad(0.0) == 0.5
+    np.testing.assert_allclose(oracle.gelu(y) - oracle.gelu(-y), y, rtol=1e-12, atol=1e-12)
+
+
+def test_gated_scan_matches_autograd_of_the_torch_composition():
+    x, xg, ag, lam, gout = make_scan_inputs(2, 19, 6, seed=4)
+    y = 1.5 * np.random.default_rng(8).standard_normal(x.shape)
+    t = [torch.from_numpy(v).requires_grad_(True) for v in (x, xg, ag, lam, y)]
+    h = rglru_torch.rglru_scan_loop(*t[:4])
+    out = torch.nn.functional.gelu(t[4]) * h
+    grads = torch.autograd.grad(out, t, torch.from_numpy(gout))
+    h_o, out_o = oracle.rglru_scan_gated_fwd(x, xg, ag, lam, y)
+    assert max_rel(out_o, out.detach().numpy()) < 1e-12
+    got = oracle.rglru_scan_gated_bwd(x, xg, ag, lam, y, h_o, gout)
+    order = (0, 1, 2, 3, 4)  # dx, dx_rg_lru, da_rg_lru, dLambda, dy
+    for k, a in zip(order, got):
+        assert max_rel(a, grads[k].numpy()) < 1e-10, k
