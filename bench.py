@@ -7,7 +7,9 @@ pre-allocated (nothing is allocated inside the timed region).
 
 Default workload: B=8, T=4096, D=2560, bf16 activations, fp32 state (the configuration
 the 70 %-of-HBM-peak target is quoted on).  ``--workload long`` runs B=2, T=32768,
-D=4096; ``--workload scan_conv`` adds the temporal conv1d forward and backward.
+D=4096; ``--workload scan_conv`` adds the temporal conv1d forward and backward;
+``--workload scan_gated`` runs the scan fused with the block's gate (out = gelu(y) * h,
+y being one half of a [B, T, 2D] projection), 12 + 20 bytes per element.
 
 Prints one JSON line:
   value        tokens/s = B*T / (wall time per step), whole job on one GPU
@@ -52,6 +54,7 @@ WORKLOADS = {
     "scan": (8, 4096, 2560, (0.9, 0.999), False),
     "long": (2, 32768, 4096, (0.99, 0.9999), False),
     "scan_conv": (8, 4096, 2560, (0.9, 0.999), True),
+    "scan_gated": (8, 4096, 2560, (0.9, 0.999), False),
 }
 
 
@@ -131,9 +134,20 @@ def main():
         dw = torch.empty(W, D, device=dev)
         db = torch.empty(D, device=dev)
         cws = torch.empty(lib.hawk_conv1d_bwd_workspace_bytes(B, T, D, W), dtype=torch.uint8, device=dev)
+    gated = args.workload == "scan_gated"
+    if gated:
+        xy = torch.randn(B, T, 2 * D, device=dev, generator=gen).to(bf)
+        y = xy[..., D:]               # the gate half of the block's input projection, in place
+        gated_out = torch.empty_like(x)
+        dy = torch.empty_like(x)
     stream = torch.cuda.current_stream(dev).cuda_stream
 
     def fwd():
+        if gated:
+            _lib.check("scan_gated_fwd", lib.hawk_rglru_scan_gated_fwd(
+                x.data_ptr(), xg.data_ptr(), ag.data_ptr(), lam.data_ptr(), y.data_ptr(), 2 * D, h.data_ptr(),
+                gated_out.data_ptr(), None, B, T, D, code, code, ws.data_ptr(), ws.numel(), stream))
+            return
         src = x
         if with_conv:
             _lib.check("conv_fwd", lib.hawk_conv1d_fwd(x.data_ptr(), cw.data_ptr(), cb.data_ptr(), None,
@@ -144,6 +158,12 @@ def main():
                                                        ws.data_ptr(), ws.numel(), stream))
 
     def bwd():
+        if gated:
+            _lib.check("scan_gated_bwd", lib.hawk_rglru_scan_gated_bwd(
+                x.data_ptr(), xg.data_ptr(), ag.data_ptr(), lam.data_ptr(), y.data_ptr(), 2 * D, h.data_ptr(),
+                gout.data_ptr(), dx.data_ptr(), dxg.data_ptr(), dag.data_ptr(), dy.data_ptr(), D, dlam.data_ptr(),
+                B, T, D, code, code, ws.data_ptr(), ws.numel(), stream))
+            return
         src = u if with_conv else x
         _lib.check("scan_bwd", lib.hawk_rglru_scan_bwd(src.data_ptr(), xg.data_ptr(), ag.data_ptr(),
                                                        lam.data_ptr(), h.data_ptr(), gout.data_ptr(),
@@ -191,9 +211,10 @@ def main():
     bwd_ms = float(np.mean([e[1].elapsed_time(e[2]) for e in ev]))
     ms_per_step = wall * 1e3 / args.steps
     elem = 2  # bytes per bf16 activation element
-    fwd_bytes = 4 * elem * N + (2 * elem * N if with_conv else 0)
-    bwd_bytes = 8 * elem * N
-    step_bytes = 12 * elem * N + (5 * elem * N if with_conv else 0)
+    # gated: the forward also reads y and writes out; the backward also reads y and writes dy
+    fwd_bytes = (6 if gated else 4) * elem * N + (2 * elem * N if with_conv else 0)
+    bwd_bytes = (10 if gated else 8) * elem * N
+    step_bytes = fwd_bytes + bwd_bytes + (3 * elem * N if with_conv else 0)
     bwd_gbs = bwd_bytes / (bwd_ms * 1e-3) / 1e9
 
     out = {
@@ -212,12 +233,14 @@ def main():
         "config": {
             "workload": f"{args.workload}: RG-LRU scan"
                         + (" + temporal conv1d (W=4)" if with_conv else "")
+                        + (" fused with out = gelu(y) * h" if gated else "")
                         + f" fwd+bwd, B={B}, T={T}, D={D}, bf16",
             "B": B, "T": T, "D": D,
         },
         "roofline": {
             "bound": "hbm",
-            "kernel": "rglru_scan_bwd_kernel (+ dlam_reduce_kernel, same launch call)",
+            "kernel": "rglru_scan_bwd_kernel" + (" (gated)" if gated else "")
+                      + " (+ dlam_reduce_kernel, same launch call)",
             "achieved": bwd_gbs,
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",

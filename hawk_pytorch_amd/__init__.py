@@ -7,6 +7,7 @@ from .external import (
     BlockDiagonalLinear,
     Conv1D,
     rglru_step,
+    rglru_step_gated,
     rnn_param_init,
     temporal_conv1d,
     temporal_conv1d_step,
@@ -36,6 +37,7 @@ __all__ = [
     "fused_linear_scan",
     "fused_linear_scan_gated",
     "rglru_step",
+    "rglru_step_gated",
     "rnn_param_init",
     "sequential_scan_backward",
     "sequential_scan_forward",

@@ -197,4 +197,17 @@ int hawk_rglru_step(const void* x, const void* x_rg_lru, const void* a_rg_lru, c
                             as_stream(stream));
 }
 
+int hawk_rglru_step_gated(const void* x, const void* x_rg_lru, const void* a_rg_lru, const float* bias_i,
+                          const float* bias_a, const float* a_param, const void* y, long long ldy, void* recc_state,
+                          void* h_out, void* out, int B, int D, int dtype, int state_dtype, void* stream) {
+    if (!x || !x_rg_lru || !a_rg_lru || !a_param || !recc_state || !y || !out) return HAWK_ERR_NULL_POINTER;
+    if (!dtype_ok(dtype) || !dtype_ok(state_dtype)) return HAWK_ERR_BAD_DTYPE;
+    if (B < 1 || D < 1 || B > kMaxGridY || ldy < D) return HAWK_ERR_BAD_SHAPE;
+    if (!aligned16(x) || !aligned16(x_rg_lru) || !aligned16(a_rg_lru) || !aligned16(recc_state) || !aligned16(out) ||
+        (h_out && !aligned16(h_out)) || !aligned_elem(y, dtype))
+        return HAWK_ERR_ALIGNMENT;
+    return hawk::rglru_step_gated(x, x_rg_lru, a_rg_lru, bias_i, bias_a, a_param, y, ldy, recc_state, h_out, out, B,
+                                  D, dtype, state_dtype, as_stream(stream));
+}
+
 }  // extern "C"

@@ -41,5 +41,8 @@ int conv1d_step(void* conv_state, const void* x_new, const float* w, const float
                 int W, int dtype, int y_dtype, hipStream_t st);
 int rglru_step(const void* x, const void* xg, const void* ag, const float* lam, void* state, void* h_out, int B,
                int D, int dtype, int state_dtype, hipStream_t st);
+int rglru_step_gated(const void* x, const void* xg, const void* ag, const float* bias_i, const float* bias_a,
+                     const float* lam, const void* y, long long ldy, void* state, void* h_out, void* out, int B,
+                     int D, int dtype, int state_dtype, hipStream_t st);
 
 }  // namespace hawk

@@ -6,6 +6,8 @@
 // cache buffers in place and work for any batch size.
 #include "hawk_scan.h"
 
+#include <stdint.h>
+
 #include "hawk_device.h"
 
 namespace hawk {
@@ -69,11 +71,18 @@ __global__ __launch_bounds__(256) void conv1d_step_kernel(ST* __restrict__ state
 }
 
 // h = alpha * state + sqrt(1 - alpha^2) * (sigmoid(x_rg_lru) * x); state <- h; h_out <- h.
+// Optional, each switched by a non-null pointer (uniform over the launch):
+//   bias_i, bias_a [D] fp32   added to the two gate logits first (the block-diagonal
+//                             projections' biases), so the projections can skip them
+//   y (rows ldy apart), out   out <- gelu(y) * h, the block's gate
 template <typename ET, typename ST, int V>
 __global__ __launch_bounds__(256) void rglru_step_kernel(const ET* __restrict__ x, const ET* __restrict__ xg,
-                                                        const ET* __restrict__ ag, const float* __restrict__ lam,
-                                                        ST* __restrict__ state, ET* __restrict__ h_out, int D,
-                                                        int nvec) {
+                                                        const ET* __restrict__ ag,
+                                                        const float* __restrict__ bias_i,
+                                                        const float* __restrict__ bias_a,
+                                                        const float* __restrict__ lam, const ET* __restrict__ y,
+                                                        size_t ldy, ST* __restrict__ state, ET* __restrict__ h_out,
+                                                        ET* __restrict__ out, int D, int nvec) {
     typedef typename Raw<ET, V>::type eraw_t;
     typedef typename Raw<ST, V>::type sraw_t;
     const int vc = blockIdx.x * blockDim.x + threadIdx.x;
@@ -81,26 +90,41 @@ __global__ __launch_bounds__(256) void rglru_step_kernel(const ET* __restrict__ 
     if (vc >= nvec) return;
     const int c0 = vc * V;
     const size_t o = (size_t)b * D + c0;
-    float fx[V], fxg[V], fag[V], fs[V], out[V];
+    float fx[V], fxg[V], fag[V], fs[V], hn[V];
     unpack(load_raw<ET, V>(x + o), fx);
     unpack(load_raw<ET, V>(xg + o), fxg);
     unpack(load_raw<ET, V>(ag + o), fag);
     unpack(load_raw<ST, V>(state + o), fs);
 #pragma unroll
     for (int v = 0; v < V; ++v) {
+        if (bias_i != nullptr) fxg[v] += bias_i[c0 + v];
+        if (bias_a != nullptr) fag[v] += bias_a[c0 + v];
         const float s = softplus_precise(lam[c0 + v]);
         const float i = sigmoid_fast(fxg[v]);
         const float r = sigmoid_fast(fag[v]);
         const float alpha = hw_exp2(-8.0f * kLog2e * s * r);
         const float z = one_minus_exp(-16.0f * s * r);
-        out[v] = fmaf(alpha, fs[v], hw_sqrt(z) * (i * fx[v]));
+        hn[v] = fmaf(alpha, fs[v], hw_sqrt(z) * (i * fx[v]));
     }
     eraw_t rh;
     sraw_t rs;
-    pack(out, rh);
-    pack(out, rs);
-    *reinterpret_cast<eraw_t*>(h_out + o) = rh;
+    pack(hn, rh);
+    pack(hn, rs);
+    if (h_out != nullptr) *reinterpret_cast<eraw_t*>(h_out + o) = rh;
     *reinterpret_cast<sraw_t*>(state + o) = rs;
+    if (y != nullptr) {
+        float fy[V], g[V];
+        unpack(load_raw<ET, V>(y + (size_t)b * ldy + c0), fy);
+#pragma unroll
+        for (int v = 0; v < V; ++v) {
+            float cdf, e;
+            normal_cdf<true>(fy[v], cdf, e);
+            g[v] = (fy[v] * cdf) * hn[v];
+        }
+        eraw_t ro;
+        pack(g, ro);
+        *reinterpret_cast<eraw_t*>(out + o) = ro;
+    }
 }
 
 int pick_v(int D) { return (D % 4 == 0) ? 4 : ((D % 2 == 0) ? 2 : 1); }
@@ -121,9 +145,14 @@ int conv_step_dispatch(void* state, const void* x_new, const float* w, const flo
 }
 
 template <typename ET, typename ST>
-int rglru_step_dispatch(const void* x, const void* xg, const void* ag, const float* lam, void* state, void* h_out,
+int rglru_step_dispatch(const void* x, const void* xg, const void* ag, const float* bias_i, const float* bias_a,
+                        const float* lam, const void* y, long long ldy, void* state, void* h_out, void* out,
                         int B, int D, hipStream_t st) {
-    const int V = pick_v(D);
+    int V = pick_v(D);
+    // y may be a slice of a wider row: its vectors must stay aligned in every row
+    while (V > 1 && y != nullptr &&
+           ((ldy % V) != 0 || (reinterpret_cast<uintptr_t>(y) % (V * sizeof(ET))) != 0))
+        V /= 2;
     const int nvec = D / V;
     const dim3 grid((unsigned)ceil_div(nvec, 256), (unsigned)B), block(256);
     const ET* xp = static_cast<const ET*>(x);
@@ -131,9 +160,18 @@ int rglru_step_dispatch(const void* x, const void* xg, const void* ag, const flo
     const ET* agp = static_cast<const ET*>(ag);
     ST* sp = static_cast<ST*>(state);
     ET* hp = static_cast<ET*>(h_out);
-    if (V == 4) hipLaunchKernelGGL((rglru_step_kernel<ET, ST, 4>), grid, block, 0, st, xp, xgp, agp, lam, sp, hp, D, nvec);
-    else if (V == 2) hipLaunchKernelGGL((rglru_step_kernel<ET, ST, 2>), grid, block, 0, st, xp, xgp, agp, lam, sp, hp, D, nvec);
-    else hipLaunchKernelGGL((rglru_step_kernel<ET, ST, 1>), grid, block, 0, st, xp, xgp, agp, lam, sp, hp, D, nvec);
+    const ET* yp = static_cast<const ET*>(y);
+    ET* op = static_cast<ET*>(out);
+    const size_t ld = (size_t)ldy;
+    if (V == 4)
+        hipLaunchKernelGGL((rglru_step_kernel<ET, ST, 4>), grid, block, 0, st, xp, xgp, agp, bias_i, bias_a, lam, yp, ld,
+                           sp, hp, op, D, nvec);
+    else if (V == 2)
+        hipLaunchKernelGGL((rglru_step_kernel<ET, ST, 2>), grid, block, 0, st, xp, xgp, agp, bias_i, bias_a, lam, yp, ld,
+                           sp, hp, op, D, nvec);
+    else
+        hipLaunchKernelGGL((rglru_step_kernel<ET, ST, 1>), grid, block, 0, st, xp, xgp, agp, bias_i, bias_a, lam, yp, ld,
+                           sp, hp, op, D, nvec);
     return hipGetLastError() == hipSuccess ? HAWK_OK : HAWK_ERR_LAUNCH;
 }
 
@@ -149,14 +187,23 @@ int conv1d_step(void* conv_state, const void* x_new, const float* w, const float
     return conv_step_dispatch<float, float>(conv_state, x_new, w, bias, y, B, D, W, st);
 }
 
+int rglru_step_gated(const void* x, const void* xg, const void* ag, const float* bias_i, const float* bias_a,
+                     const float* lam, const void* y, long long ldy, void* state, void* h_out, void* out, int B,
+                     int D, int dtype, int state_dtype, hipStream_t st) {
+    if (dtype == HAWK_DTYPE_BF16) {
+        if (state_dtype == HAWK_DTYPE_BF16)
+            return rglru_step_dispatch<bf16_t, bf16_t>(x, xg, ag, bias_i, bias_a, lam, y, ldy, state, h_out, out, B, D, st);
+        return rglru_step_dispatch<bf16_t, float>(x, xg, ag, bias_i, bias_a, lam, y, ldy, state, h_out, out, B, D, st);
+    }
+    if (state_dtype == HAWK_DTYPE_BF16)
+        return rglru_step_dispatch<float, bf16_t>(x, xg, ag, bias_i, bias_a, lam, y, ldy, state, h_out, out, B, D, st);
+    return rglru_step_dispatch<float, float>(x, xg, ag, bias_i, bias_a, lam, y, ldy, state, h_out, out, B, D, st);
+}
+
 int rglru_step(const void* x, const void* xg, const void* ag, const float* lam, void* state, void* h_out, int B,
                int D, int dtype, int state_dtype, hipStream_t st) {
-    if (dtype == HAWK_DTYPE_BF16) {
-        if (state_dtype == HAWK_DTYPE_BF16) return rglru_step_dispatch<bf16_t, bf16_t>(x, xg, ag, lam, state, h_out, B, D, st);
-        return rglru_step_dispatch<bf16_t, float>(x, xg, ag, lam, state, h_out, B, D, st);
-    }
-    if (state_dtype == HAWK_DTYPE_BF16) return rglru_step_dispatch<float, bf16_t>(x, xg, ag, lam, state, h_out, B, D, st);
-    return rglru_step_dispatch<float, float>(x, xg, ag, lam, state, h_out, B, D, st);
+    return rglru_step_gated(x, xg, ag, nullptr, nullptr, lam, nullptr, 0, state, h_out, nullptr, B, D, dtype,
+                            state_dtype, st);
 }
 
 }  // namespace hawk

@@ -224,6 +224,36 @@ def rglru_step(x, x_rg_lru, a_rg_lru, a_param, recc_state):
     return h.reshape(shape)
 
 
+def rglru_step_gated(x, x_rg_lru, a_rg_lru, a_param, recc_state, y, bias_i=None, bias_a=None):
+    """One-token RG-LRU update fused with what surrounds it in a Hawk block: the two gate
+    projections' biases (``bias_i``, ``bias_a``, any shape with D elements, optional) are
+    added to the logits in the kernel, the state is updated in place and
+    ``gelu(y) * h`` is returned (hawk/hawk.py:134-151, :181-182, :196-198 in one launch).
+    ``y`` may be a slice of a wider tensor (the gate half of the input projection)."""
+    D = x.shape[-1]
+    shape = x.shape
+    B = x.numel() // D
+    assert recc_state.numel() == B * D and recc_state.is_contiguous()
+    dev = _lib.require_cuda(x, x_rg_lru, a_rg_lru, a_param, recc_state, y)
+    run_dtype = x.dtype if x.dtype in (torch.bfloat16, torch.float32) else torch.float32
+    xs = [_lib.dense16(t.reshape(B, D).to(run_dtype)) for t in (x, x_rg_lru, a_rg_lru)]
+    lam = _lib.dense16(a_param.detach().float())
+    biases = [None if b is None else _lib.dense16(b.detach().float().reshape(D)) for b in (bias_i, bias_a)]
+    y2 = y.reshape(B, D) if y.dtype == run_dtype else y.reshape(B, D).to(run_dtype)
+    if y2.stride(1) != 1 or (B > 1 and y2.stride(0) < D):
+        y2 = y2.contiguous()
+    ldy = y2.stride(0) if B > 1 else D
+    out = torch.empty((B, D), dtype=run_dtype, device=dev)
+    with torch.cuda.device(dev):
+        status = _lib.load().hawk_rglru_step_gated(
+            xs[0].data_ptr(), xs[1].data_ptr(), xs[2].data_ptr(), _lib.ptr(biases[0]), _lib.ptr(biases[1]),
+            lam.data_ptr(), y2.data_ptr(), ldy, recc_state.data_ptr(), None, out.data_ptr(), B, D,
+            _lib.dtype_code(run_dtype), _lib.dtype_code(recc_state.dtype), _lib.stream_ptr(dev),
+        )
+    _lib.check("hawk_rglru_step_gated", status)
+    return out.reshape(shape)
+
+
 # ---------------------------------------------------------------------------------------
 # Pieces of the harness model that are not on the hot path (library GEMMs, initialisers).
 # ---------------------------------------------------------------------------------------
@@ -266,8 +296,12 @@ class BlockDiagonalLinear(nn.Module):
         nn.init.normal_(self.w, mean=0.0, std=math.sqrt(self.w_init_variance_scale / self.block_width))
         nn.init.zeros_(self.b)
 
-    def forward(self, x: torch.Tensor) -> torch.Tensor:
+    def forward(self, x: torch.Tensor, add_bias: bool = True) -> torch.Tensor:
+        """``add_bias=False`` leaves ``b`` out for a consumer that adds it itself (the fused
+        decode step does)."""
         lead = x.shape[:-1]
         xb = x.reshape(*lead, self.num_blocks, self.block_width)
-        yb = torch.einsum("...hi,hij->...hj", xb, self.w) + self.b
+        yb = torch.einsum("...hi,hij->...hj", xb, self.w)
+        if add_bias:
+            yb = yb + self.b
         return yb.reshape(*lead, self.width)

@@ -12,8 +12,9 @@ What differs from upstream is confined to the recurrent block:
   ``HawkConfig.fused_epilogue`` (default) the scan kernel also applies the block's gate,
   ``gelu(y) * h``, and its backward also produces the gate's gradient;
 * decode (``use_cache=True`` with a warm ``RNNCache``) issues two fused kernels per layer
-  (conv window roll + conv, RG-LRU state update) instead of about thirty eager ones, works
-  for any batch size, and evaluates the two gate projections once instead of twice.
+  (conv window roll + conv; gate biases + RG-LRU state update + output gate) instead of
+  about thirty eager ones, works for any batch size, and evaluates the two gate
+  projections once instead of twice.
 """
 
 from __future__ import annotations
@@ -27,7 +28,7 @@ import torch.nn as nn
 import torch.nn.functional as F
 
 from .cache import RNNCache
-from .external import BlockDiagonalLinear, Conv1D, rglru_step, rnn_param_init
+from .external import BlockDiagonalLinear, Conv1D, rglru_step, rglru_step_gated, rnn_param_init
 from .scan_fused import fused_linear_scan, fused_linear_scan_gated
 
 
@@ -116,10 +117,22 @@ class Hawk(nn.Module):
             assert layer_past is not None
             u = self.conv1d.step(layer_past.conv_state, branch[:, -1:, :])
             gate_branch = gate_branch[:, -1:, :]
+            layer_past.current_cache_size = 1
+            if self.config.fused_epilogue:
+                gated = rglru_step_gated(
+                    u,
+                    self.rg_lru_input_gate(u, add_bias=False),
+                    self.rg_lru_a_gate(u, add_bias=False),
+                    self.rg_lru_a_param,
+                    layer_past.recc_state,
+                    gate_branch,
+                    bias_i=self.rg_lru_input_gate.b,
+                    bias_a=self.rg_lru_a_gate.b,
+                )
+                return self.resid_proj(gated), layer_past
             h = rglru_step(
                 u, self.rg_lru_input_gate(u), self.rg_lru_a_gate(u), self.rg_lru_a_param, layer_past.recc_state
             )
-            layer_past.current_cache_size = 1
             cache = layer_past
         else:
             if self.use_cache:

@@ -174,6 +174,19 @@ int hawk_rglru_step(const void* x, const void* x_rg_lru, const void* a_rg_lru,
                     const float* a_param, void* recc_state, void* h_out, int B, int D,
                     int dtype, int state_dtype, void* stream);
 
+/* The same step with the work around it folded in (one launch instead of five):
+ *   bias_i, bias_a  [D] fp32 or NULL: added to x_rg_lru / a_rg_lru first, so the two
+ *                   block-diagonal projections (hawk/external.py:224-233, called at
+ *                   hawk/hawk.py:181-182) can leave their bias out
+ *   y, out          out [B,D] <- gelu(y) * h, the gate of Hawk.epilogue (hawk/hawk.py:134-135);
+ *                   y is [B,D] with rows ldy >= D elements apart (the gate half of the
+ *                   input projection, passed in place), aligned to its element size
+ *   h_out           may be NULL here (the state itself lands in recc_state) */
+int hawk_rglru_step_gated(const void* x, const void* x_rg_lru, const void* a_rg_lru,
+                          const float* bias_i, const float* bias_a, const float* a_param,
+                          const void* y, long long ldy, void* recc_state, void* h_out, void* out,
+                          int B, int D, int dtype, int state_dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -187,3 +187,16 @@ def scan_gated_bwd(x, xg, ag, lam, y, h, gout, dy=None, ws=None):
         B, T, D, _lib.dtype_code(x.dtype), _lib.dtype_code(h.dtype), ws.data_ptr(), ws.numel(), _stream())
     _lib.check("hawk_rglru_scan_gated_bwd", rc)
     return dx, dxg, dag, dlam, dy
+
+
+def rglru_step_gated(x, xg, ag, bias_i, bias_a, lam, y, state, want_h=True):
+    """y: [B,D] view with unit channel stride (rows may be further apart than D)."""
+    B, D = x.shape
+    h = torch.empty_like(x) if want_h else None
+    out = torch.empty_like(x)
+    rc = _lib.load().hawk_rglru_step_gated(
+        x.data_ptr(), xg.data_ptr(), ag.data_ptr(), _lib.ptr(bias_i), _lib.ptr(bias_a), lam.data_ptr(),
+        y.data_ptr(), y.stride(0) if B > 1 else D, state.data_ptr(), _lib.ptr(h), out.data_ptr(), B, D,
+        _lib.dtype_code(x.dtype), _lib.dtype_code(state.dtype), _stream())
+    _lib.check("hawk_rglru_step_gated", rc)
+    return out, h

@@ -40,6 +40,35 @@ def test_rglru_step_bf16_cache_fp32_activations():
 
 
 @pytest.mark.parametrize("dtype", ["f32", "bf16"])
+@pytest.mark.parametrize("with_bias", [True, False])
+@pytest.mark.parametrize("B,D", [(1, 64), (256, 2560), (3, 130), (5, 7)])
+def test_rglru_step_gated(B, D, with_bias, dtype):
+    """Biases of the two gate projections added in the kernel, state updated in place,
+    gelu(y) * h returned; y is the second half of a [B, 2D] projection."""
+    x, xg, ag, lam, st = make_scan_inputs(B, 1, D, seed=B + D + 1)
+    rng = np.random.default_rng(B * D)
+    d = [capi.to_dev(a[:, 0], dtype) for a in (x, xg, ag, st)]
+    xr, xgr, agr, sr = (capi.to_np(t) for t in d)
+    lam_d = capi.to_dev(lam, "f32")
+    bi = capi.to_dev(rng.standard_normal(D), "f32") if with_bias else None
+    ba = capi.to_dev(rng.standard_normal(D), "f32") if with_bias else None
+    wide = capi.to_dev(2.0 * rng.standard_normal((B, 2 * D)), dtype)
+    y = wide[:, D:]
+    state = d[3].clone()
+    out, h = capi.rglru_step_gated(d[0], d[1], d[2], bi, ba, lam_d, y, state)
+    zero = np.zeros(D)
+    h_ref = oracle.rglru_step(xr, xgr + (capi.to_np(bi) if with_bias else zero),
+                              agr + (capi.to_np(ba) if with_bias else zero), capi.to_np(lam_d), sr)
+    assert max_rel(capi.to_np(h), h_ref) < TOL[dtype]
+    assert max_rel(capi.to_np(out), oracle.gelu(capi.to_np(y)) * h_ref) < TOL[dtype]
+    assert torch.equal(state, h)
+    # h_out is optional
+    state2 = d[3].clone()
+    out2, none = capi.rglru_step_gated(d[0], d[1], d[2], bi, ba, lam_d, y, state2, want_h=False)
+    assert none is None and torch.equal(out2, out) and torch.equal(state2, state)
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
 @pytest.mark.parametrize("W", [1, 2, 4, 8])
 @pytest.mark.parametrize("B,D", [(1, 64), (256, 2560), (3, 30)])
 def test_conv_step(B, D, W, dtype):
