@@ -9,7 +9,10 @@ Default workload: B=8, T=4096, D=2560, bf16 activations, fp32 state (the configu
 the 70 %-of-HBM-peak target is quoted on).  ``--workload long`` runs B=2, T=32768,
 D=4096; ``--workload scan_conv`` adds the temporal conv1d forward and backward;
 ``--workload scan_gated`` runs the scan fused with the block's gate (out = gelu(y) * h,
-y being one half of a [B, T, 2D] projection), 12 + 20 bytes per element.
+y being one half of a [B, T, 2D] projection), 12 + 20 bytes per element;
+``--workload decode`` times one-token steps of a 26-layer Hawk (R = H = 2560, I = 7680,
+10 gate blocks, vocabulary 32000, bf16 weights) at batch 256 after a 1024-token prefill,
+eagerly and as a replayed HIP graph, plus the two hot-path kernels of a layer on their own.
 
 Prints one JSON line:
   value        tokens/s = B*T / (wall time per step), whole job on one GPU
@@ -86,12 +89,145 @@ def cpu_baseline(B, D, lo, hi, seed, budget_rows=512):
     }
 
 
+def run_decode(args, lib, dev):
+    """Decode at batch 256: tokens/s of whole model steps, and the hot path's share of a layer."""
+    import hawk_pytorch_amd as hk
+    from hawk_pytorch_amd import _lib
+
+    B, prompt_len, vocab = 256, 1024, 32000
+    cfg = hk.HawkConfig(vocab_size=vocab, hidden_size=2560, intermediate_size=7680, num_hidden_layers=26,
+                        recurrent_size=2560, num_blocks=10, conv_width=4)
+    torch.manual_seed(args.seed)
+    with torch.device(dev):
+        model = hk.HawkModel(cfg, use_cache=True)
+    model.eval().bfloat16()
+    for layer in model.layers:
+        r = layer.recc
+        # the recurrence's own parameters stay fp32 (the kernels read them as fp32)
+        for p in (r.rg_lru_a_param, r.conv1d.w, r.conv1d.b, r.rg_lru_input_gate.b, r.rg_lru_a_gate.b):
+            p.data = p.data.float()
+        r.conv1d.out_dtype = torch.bfloat16
+        torch.nn.init.normal_(r.resid_proj.weight, std=0.02)
+        torch.nn.init.normal_(layer.mlp.resid_proj.weight, std=0.02)
+    torch.nn.init.normal_(model.lm_head.weight, std=0.02)
+
+    gen = torch.Generator(device=dev).manual_seed(args.seed)
+    prompt = torch.randint(1, vocab, (B, prompt_len), device=dev, generator=gen)
+    tok = torch.randint(1, vocab, (B, 1), device=dev, generator=gen)
+    caches = model.new_cache(B)
+    # weights are bf16 already, so autocast only rounds the few fp32 activations (the gate
+    # logits pick up an fp32 bias) before the GEMMs; it casts no weight
+    with torch.no_grad(), torch.autocast(device_type="cuda", dtype=torch.bfloat16):
+        logits, caches = model(prompt, layer_past=caches)
+        del logits
+        for _ in range(args.warmup):
+            model(tok, layer_past=caches)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            model(tok, layer_past=caches)
+        torch.cuda.synchronize()
+        eager_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+
+        graph = torch.cuda.CUDAGraph()
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            model(tok, layer_past=caches)
+        torch.cuda.current_stream().wait_stream(side)
+        with torch.cuda.graph(graph):
+            static_logits, _ = model(tok, layer_past=caches)
+        for _ in range(args.warmup):
+            graph.replay()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            graph.replay()
+        torch.cuda.synchronize()
+        graph_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+        finite = bool(torch.isfinite(static_logits.float()).all())
+
+    # the two hot-path launches of one layer, through the C ABI
+    D, W = 2560, 4
+    bf, code = torch.bfloat16, _lib.HAWK_DTYPE_BF16
+    conv_state = torch.randn(B, W - 1, D, device=dev).to(bf)
+    xy = torch.randn(B, 2 * D, device=dev).to(bf)
+    xn, y = xy[:, :D].contiguous(), xy[:, D:]
+    cw, cb = torch.randn(W, D, device=dev) * 0.5, torch.zeros(D, device=dev)
+    u, xg, ag = (torch.randn(B, D, device=dev).to(bf) for _ in range(3))
+    bi, ba = torch.zeros(D, device=dev), torch.zeros(D, device=dev)
+    lam = lambda_for_a8_range(torch.Generator().manual_seed(args.seed), D, 0.9, 0.999).to(dev)
+    state = torch.zeros(B, D, device=dev).to(bf)
+    out = torch.empty(B, D, device=dev, dtype=bf)
+    def layer_hot_path():
+        stream = torch.cuda.current_stream(dev).cuda_stream
+        _lib.check("conv1d_step", lib.hawk_conv1d_step(conv_state.data_ptr(), xn.data_ptr(), cw.data_ptr(),
+                                                       cb.data_ptr(), u.data_ptr(), B, D, W, code, code, stream))
+        _lib.check("rglru_step_gated", lib.hawk_rglru_step_gated(
+            u.data_ptr(), xg.data_ptr(), ag.data_ptr(), bi.data_ptr(), ba.data_ptr(), lam.data_ptr(), y.data_ptr(),
+            2 * D, state.data_ptr(), None, out.data_ptr(), B, D, code, code, stream))
+
+    # 26 layers' worth of the two launches as one HIP graph, so that the figure is the GPU's
+    # time and not the host's launch rate
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        layer_hot_path()
+    torch.cuda.current_stream().wait_stream(side)
+    hot_graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(hot_graph):
+        for _ in range(26):
+            layer_hot_path()
+    for _ in range(5):
+        hot_graph.replay()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    n_rep = 40
+    e0.record()
+    for _ in range(n_rep):
+        hot_graph.replay()
+    e1.record()
+    torch.cuda.synchronize()
+    hot_us = e0.elapsed_time(e1) * 1e3 / (n_rep * 26)
+    # conv step: read 3 state rows + new row, write y and 3 rows; RG-LRU step: read u, two logits,
+    # state, y, write state and out  (bf16)
+    hot_bytes = (4 + 4 + 7) * 2 * B * D
+    gbs = hot_bytes / (hot_us * 1e-6) / 1e9
+
+    out_json = {
+        "metric": "decode tokens/s, batch 256, 1 GPU (whole model step; hot path reported beside it)",
+        "value": B / (graph_ms * 1e-3),
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": graph_ms,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16 weights and activations, f32 recurrence arithmetic",
+        "data": f"synthetic, seed {args.seed}: random-init weights, random {prompt_len}-token prompt, vocabulary {vocab}",
+        "config": {"workload": "decode: 26 layers, R=H=2560, I=7680, 10 gate blocks, B=256, one token per step",
+                   "B": B, "layers": 26, "D": D, "vocab": vocab, "prompt": prompt_len},
+        "eager_ms_per_step": eager_ms,
+        "graph_ms_per_step": graph_ms,
+        "logits_finite": finite,
+        "hot_path_us_per_layer_step": hot_us,
+        "roofline": {
+            "bound": "hbm",
+            "kernel": "conv1d_step_kernel + rglru_step_kernel (two launches per layer and token; launch-bound)",
+            "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS, "traffic": None,
+            "algorithmic_bytes_per_launch": hot_bytes,
+        },
+    }
+    print(json.dumps(out_json))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", choices=sorted(WORKLOADS), default="scan")
+    ap.add_argument("--workload", choices=sorted(WORKLOADS) + ["decode"], default="scan")
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calibration-copy", action="store_true",
@@ -113,6 +249,9 @@ def main():
     lib = _lib.load()
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if args.workload == "decode":
+        run_decode(args, lib, dev)
+        return
     B, T, D, (lo, hi), with_conv = WORKLOADS[args.workload]
     N = B * T * D
     code = _lib.HAWK_DTYPE_BF16
