@@ -56,6 +56,8 @@ SIGNATURES = {
     "hawk_conv1d_bwd": (_c_int, [_c_void_p] * 6 + [_c_int] * 6 + [_c_void_p, _c_size_t, _c_void_p]),
     "hawk_conv1d_step": (_c_int, [_c_void_p] * 5 + [_c_int] * 5 + [_c_void_p]),
     "hawk_rglru_step": (_c_int, [_c_void_p] * 6 + [_c_int] * 4 + [_c_void_p]),
+    "hawk_gate_proj_supported": (_c_int, [_c_int, _c_int]),
+    "hawk_gate_proj_fwd": (_c_int, [_c_void_p] * 7 + [_c_int] * 6 + [_c_void_p]),
     "hawk_rglru_step_gated": (
         _c_int, [_c_void_p] * 7 + [ctypes.c_longlong] + [_c_void_p] * 3 + [_c_int] * 4 + [_c_void_p]
     ),

@@ -210,4 +210,20 @@ int hawk_rglru_step_gated(const void* x, const void* x_rg_lru, const void* a_rg_
                                   D, dtype, state_dtype, as_stream(stream));
 }
 
+int hawk_gate_proj_supported(int D, int num_blocks) {
+    if (D < 1 || num_blocks < 1 || D % num_blocks != 0) return 0;
+    return hawk::gate_proj_block_width_supported(D / num_blocks) ? 1 : 0;
+}
+
+int hawk_gate_proj_fwd(const void* x, const void* w_i, const float* b_i, const void* w_a, const float* b_a,
+                       void* x_rg_lru, void* a_rg_lru, int M, int D, int num_blocks, int x_dtype, int w_dtype,
+                       int out_dtype, void* stream) {
+    if (!x || !w_i || !w_a || !x_rg_lru || !a_rg_lru) return HAWK_ERR_NULL_POINTER;
+    if (!dtype_ok(x_dtype) || !dtype_ok(w_dtype) || !dtype_ok(out_dtype)) return HAWK_ERR_BAD_DTYPE;
+    if (M < 1 || !hawk_gate_proj_supported(D, num_blocks)) return HAWK_ERR_BAD_SHAPE;
+    if (!aligned16(x) || !aligned16(x_rg_lru) || !aligned16(a_rg_lru)) return HAWK_ERR_ALIGNMENT;
+    return hawk::gate_proj_fwd(x, w_i, b_i, w_a, b_a, x_rg_lru, a_rg_lru, M, D, num_blocks, x_dtype, w_dtype,
+                               out_dtype, as_stream(stream));
+}
+
 }  // extern "C"

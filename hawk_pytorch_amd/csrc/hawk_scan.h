@@ -45,4 +45,9 @@ int rglru_step_gated(const void* x, const void* xg, const void* ag, const float*
                      const float* lam, const void* y, long long ldy, void* state, void* h_out, void* out, int B,
                      int D, int dtype, int state_dtype, hipStream_t st);
 
+// hawk_gates.hip
+bool gate_proj_block_width_supported(int bw);
+int gate_proj_fwd(const void* x, const void* w_i, const float* b_i, const void* w_a, const float* b_a, void* out_i,
+                  void* out_a, int M, int D, int nb, int x_dtype, int w_dtype, int out_dtype, hipStream_t st);
+
 }  // namespace hawk

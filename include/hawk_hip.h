@@ -187,6 +187,25 @@ int hawk_rglru_step_gated(const void* x, const void* x_rg_lru, const void* a_rg_
                           const void* y, long long ldy, void* recc_state, void* h_out, void* out,
                           int B, int D, int dtype, int state_dtype, void* stream);
 
+/* ---------------------------------------------------------------------------------------
+ * Block-diagonal gate projections (matrix cores, bf16 operands, fp32 accumulation).
+ * ------------------------------------------------------------------------------------- */
+
+/* 1 if the (D, num_blocks) pair is served: D divisible by num_blocks and a block width of
+ * 32, 64, 128 or 256.  Other shapes stay with the caller's library GEMM. */
+int hawk_gate_proj_supported(int D, int num_blocks);
+
+/* Both gate logits of M = B*T tokens in one pass over x:
+ *   x_rg_lru[m, h*bw+j] = b_i[h*bw+j] + sum_i x[m, h*bw+i] w_i[h, i, j]     (same for a_rg_lru)
+ * Replaces the two BlockDiagonalLinear calls of hawk/hawk.py:181-182 (einsum + bias,
+ * hawk/external.py:224-233).  x [M,D] has x_dtype; w_i, w_a [num_blocks, bw, bw] have
+ * w_dtype; b_i, b_a [D] are fp32 or NULL; the outputs [M,D] have out_dtype.  x and the
+ * weights are rounded to bf16 in registers (what bf16 autocast does to this einsum); the
+ * sums and the bias add are fp32. */
+int hawk_gate_proj_fwd(const void* x, const void* w_i, const float* b_i, const void* w_a,
+                       const float* b_a, void* x_rg_lru, void* a_rg_lru, int M, int D,
+                       int num_blocks, int x_dtype, int w_dtype, int out_dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -176,3 +176,37 @@ def rglru_scan_gated_bwd(x, x_rg_lru, a_rg_lru, a_param, y, h_saved, grad_out):
     dy = go * hs * gelu_grad(y)
     dx, dxg, dag, dlam = rglru_scan_bwd(x, x_rg_lru, a_rg_lru, a_param, hs, go * gelu(y))
     return dx, dxg, dag, dlam, dy
+
+
+# ---------------------------------------------------------------------------------------
+# Block-diagonal gate projection (restates hawk/external.py:224-233): per block h,
+# y[..., h, j] = sum_i x[..., h, i] w[h, i, j] + b[h, j].
+# ---------------------------------------------------------------------------------------
+def block_diagonal_linear(x, w, b=None):
+    """x [..., D], w [nb, bw, bw], b [nb, bw] or [D] or None -> [..., D]; fp64."""
+    x = np.asarray(x, dtype=np.float64)
+    w = np.asarray(w, dtype=np.float64)
+    nb, bw, _ = w.shape
+    assert x.shape[-1] == nb * bw and w.shape == (nb, bw, bw)
+    y = np.empty_like(x).reshape(-1, nb, bw)
+    xb = x.reshape(-1, nb, bw)
+    for h in range(nb):
+        y[:, h, :] = xb[:, h, :] @ w[h]
+    if b is not None:
+        y = y + np.asarray(b, dtype=np.float64).reshape(1, nb, bw)
+    return y.reshape(x.shape)
+
+
+def block_diagonal_linear_bwd(x, w, grad_y):
+    """(dx, dw, db) of block_diagonal_linear; fp64."""
+    x = np.asarray(x, dtype=np.float64)
+    w = np.asarray(w, dtype=np.float64)
+    gy = np.asarray(grad_y, dtype=np.float64)
+    nb, bw, _ = w.shape
+    xb, gb = x.reshape(-1, nb, bw), gy.reshape(-1, nb, bw)
+    dx = np.empty_like(xb)
+    dw = np.empty_like(w)
+    for h in range(nb):
+        dx[:, h, :] = gb[:, h, :] @ w[h].T
+        dw[h] = xb[:, h, :].T @ gb[:, h, :]
+    return dx.reshape(x.shape), dw, gb.sum(axis=0)

@@ -200,3 +200,17 @@ def rglru_step_gated(x, xg, ag, bias_i, bias_a, lam, y, state, want_h=True):
         _lib.dtype_code(x.dtype), _lib.dtype_code(state.dtype), _stream())
     _lib.check("hawk_rglru_step_gated", rc)
     return out, h
+
+
+def gate_proj_fwd(x, w_i, b_i, w_a, b_a, out_dtype=None):
+    """x [M,D] (bf16/fp32), w_* [nb,bw,bw] (bf16/fp32), b_* [D] fp32 or None."""
+    M, D = x.shape
+    nb = w_i.shape[0]
+    out_dtype = out_dtype or x.dtype
+    oi = torch.empty((M, D), dtype=out_dtype, device="cuda")
+    oa = torch.empty((M, D), dtype=out_dtype, device="cuda")
+    rc = _lib.load().hawk_gate_proj_fwd(
+        x.data_ptr(), w_i.data_ptr(), _lib.ptr(b_i), w_a.data_ptr(), _lib.ptr(b_a), oi.data_ptr(), oa.data_ptr(),
+        M, D, nb, _lib.dtype_code(x.dtype), _lib.dtype_code(w_i.dtype), _lib.dtype_code(out_dtype), _stream())
+    _lib.check("hawk_gate_proj_fwd", rc)
+    return oi, oa

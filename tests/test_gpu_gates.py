@@ -1,0 +1,98 @@
+"""GPU parity of the fused block-diagonal gate projections (matrix-core kernels) against the
+fp64 oracle, through the C ABI.  The kernels round activations and weights to bf16 and
+accumulate in fp32, so the oracle is fed the bf16-rounded operands and the tolerance is the
+bf16 one (2e-2 max-rel) for bf16 outputs and 1e-4 for fp32 outputs."""
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+import capi
+from conftest import max_rel
+
+pytestmark = pytest.mark.gpu
+
+
+def _bf16_round(a):
+    return torch.from_numpy(np.asarray(a, dtype=np.float32)).to(torch.bfloat16).double().numpy()
+
+
+def _case(M, D, nb, x_dtype, w_dtype, out_dtype, seed=0, bias=True):
+    rng = np.random.default_rng(seed)
+    bw = D // nb
+    x = rng.standard_normal((M, D))
+    wi = rng.standard_normal((nb, bw, bw)) / np.sqrt(bw)
+    wa = rng.standard_normal((nb, bw, bw)) / np.sqrt(bw)
+    bi = rng.standard_normal(D) if bias else None
+    ba = rng.standard_normal(D) if bias else None
+    xd = capi.to_dev(x, x_dtype)
+    wid, wad = capi.to_dev(wi, w_dtype), capi.to_dev(wa, w_dtype)
+    bid = capi.to_dev(bi, "f32") if bias else None
+    bad = capi.to_dev(ba, "f32") if bias else None
+    oi, oa = capi.gate_proj_fwd(xd, wid, bid, wad, bad, capi.TORCH_DTYPE[out_dtype])
+    torch.cuda.synchronize()
+    xr = _bf16_round(capi.to_np(xd))
+    ref_i = oracle.block_diagonal_linear(xr, _bf16_round(capi.to_np(wid)), capi.to_np(bid) if bias else None)
+    ref_a = oracle.block_diagonal_linear(xr, _bf16_round(capi.to_np(wad)), capi.to_np(bad) if bias else None)
+    tol = 2e-2 if out_dtype == "bf16" else 1e-4
+    assert max_rel(capi.to_np(oi), ref_i) < tol, ("x_rg_lru", M, D, nb, max_rel(capi.to_np(oi), ref_i))
+    assert max_rel(capi.to_np(oa), ref_a) < tol, ("a_rg_lru", M, D, nb, max_rel(capi.to_np(oa), ref_a))
+    return oi, oa
+
+
+@pytest.mark.parametrize("D,nb", [(256, 1), (2560, 10), (512, 16), (512, 8), (512, 4), (768, 3), (384, 3), (96, 3)])
+@pytest.mark.parametrize("M", [1, 31, 32, 33, 1000])
+def test_block_widths_and_ragged_rows(M, D, nb):
+    _case(M, D, nb, "bf16", "f32", "f32", seed=M + D)
+
+
+@pytest.mark.parametrize("x_dtype,w_dtype,out_dtype", [("bf16", "bf16", "bf16"), ("f32", "f32", "f32"),
+                                                       ("f32", "f32", "bf16"), ("bf16", "f32", "bf16")])
+def test_dtype_combinations(x_dtype, w_dtype, out_dtype):
+    _case(4096 + 17, 2560, 10, x_dtype, w_dtype, out_dtype, seed=3)
+    _case(300, 512, 16, x_dtype, w_dtype, out_dtype, seed=4, bias=False)
+
+
+def test_each_output_depends_only_on_its_own_block():
+    """Perturbing the inputs of one block must leave every other block's logits bit-identical."""
+    M, D, nb = 200, 1024, 8
+    rng = np.random.default_rng(5)
+    x = capi.to_dev(rng.standard_normal((M, D)), "bf16")
+    w = [capi.to_dev(rng.standard_normal((nb, 128, 128)) / 11.0, "f32") for _ in range(2)]
+    a0, b0 = capi.gate_proj_fwd(x, w[0], None, w[1], None)
+    x2 = x.clone()
+    x2[:, 3 * 128:4 * 128] += 1.0
+    a1, b1 = capi.gate_proj_fwd(x2, w[0], None, w[1], None)
+    keep = [c for c in range(D) if not 3 * 128 <= c < 4 * 128]
+    assert torch.equal(a0[:, keep], a1[:, keep]) and torch.equal(b0[:, keep], b1[:, keep])
+    assert not torch.equal(a0[:, 3 * 128:4 * 128], a1[:, 3 * 128:4 * 128])
+
+
+def test_unsupported_shapes_are_refused():
+    from hawk_pytorch_amd import _lib
+    lib = _lib.load()
+    assert lib.hawk_gate_proj_supported(2560, 10) == 1 and lib.hawk_gate_proj_supported(512, 16) == 1
+    assert lib.hawk_gate_proj_supported(2560, 3) == 0 and lib.hawk_gate_proj_supported(1024, 2) == 0
+    x = torch.zeros((4, 1024), device="cuda")
+    w = torch.zeros((2, 512, 512), device="cuda")
+    with pytest.raises(_lib.HawkHipError):
+        capi.gate_proj_fwd(x, w, None, w, None)
+
+
+def test_full_benchmark_shape_against_the_library_gemm():
+    """B*T = 32768 tokens, D = 2560, 10 blocks: every element against torch's batched GEMM
+    on the same bf16 operands (fp32 accumulation on both sides)."""
+    M, D, nb = 32768, 2560, 10
+    g = torch.Generator(device="cuda").manual_seed(1)
+    x = torch.randn((M, D), generator=g, device="cuda").to(torch.bfloat16)
+    wi = torch.randn((nb, 256, 256), generator=g, device="cuda") / 16.0
+    wa = torch.randn((nb, 256, 256), generator=g, device="cuda") / 16.0
+    bi = torch.randn(D, generator=g, device="cuda")
+    ba = torch.randn(D, generator=g, device="cuda")
+    oi, oa = capi.gate_proj_fwd(x, wi, bi, wa, ba, torch.float32)
+    xb = x.reshape(M, nb, 256).transpose(0, 1)
+    for got, w, b in ((oi, wi, bi), (oa, wa, ba)):
+        ref = torch.bmm(xb.float(), w.to(torch.bfloat16).float()).transpose(0, 1).reshape(M, D) + b
+        err = float((got - ref).abs().max() / ref.abs().max())
+        assert err < 1e-4, err

@@ -252,3 +252,31 @@ def test_gated_scan_matches_autograd_of_the_torch_composition():
     order = (0, 1, 2, 3, 4)  # dx, dx_rg_lru, da_rg_lru, dLambda, dy
     for k, a in zip(order, got):
         assert max_rel(a, grads[k].numpy()) < 1e-10, k
+
+
+# ------------------------------------------------------------------------------ gate projections
+def test_block_diagonal_linear_equals_a_dense_layer_with_a_block_diagonal_matrix():
+    rng = np.random.default_rng(0)
+    nb, bw, M = 3, 5, 7
+    x = rng.standard_normal((2, M, nb * bw))
+    w = rng.standard_normal((nb, bw, bw))
+    b = rng.standard_normal((nb, bw))
+    dense = np.zeros((nb * bw, nb * bw))
+    for h in range(nb):
+        dense[h * bw:(h + 1) * bw, h * bw:(h + 1) * bw] = w[h]
+    want = x @ dense + b.reshape(-1)
+    np.testing.assert_allclose(oracle.block_diagonal_linear(x, w, b), want, rtol=1e-13, atol=1e-13)
+    # and the einsum upstream writes (hawk/external.py:230)
+    t = torch.einsum("...hi,hij->...hj", torch.from_numpy(x).reshape(2, M, nb, bw), torch.from_numpy(w))
+    np.testing.assert_allclose(oracle.block_diagonal_linear(x, w), t.reshape(2, M, -1).numpy(), rtol=1e-13, atol=1e-13)
+    # backward against autograd
+    xt = torch.from_numpy(x).requires_grad_(True)
+    wt = torch.from_numpy(w).requires_grad_(True)
+    bt = torch.from_numpy(b).requires_grad_(True)
+    y = (torch.einsum("...hi,hij->...hj", xt.reshape(2, M, nb, bw), wt) + bt).reshape(2, M, -1)
+    gy = rng.standard_normal(y.shape)
+    y.backward(torch.from_numpy(gy))
+    dx, dw, db = oracle.block_diagonal_linear_bwd(x, w, gy)
+    np.testing.assert_allclose(dx, xt.grad.numpy(), rtol=1e-12, atol=1e-12)
+    np.testing.assert_allclose(dw, wt.grad.numpy(), rtol=1e-12, atol=1e-12)
+    np.testing.assert_allclose(db, bt.grad.numpy(), rtol=1e-12, atol=1e-12)
