@@ -226,4 +226,34 @@ int hawk_gate_proj_fwd(const void* x, const void* w_i, const float* b_i, const v
                                out_dtype, as_stream(stream));
 }
 
+int hawk_gate_proj_bwd_input(const void* d_x_rg_lru, const void* d_a_rg_lru, const void* w_i, const void* w_a,
+                             void* dx, int M, int D, int num_blocks, int g_dtype, int w_dtype, int dx_dtype,
+                             void* stream) {
+    if (!d_x_rg_lru || !d_a_rg_lru || !w_i || !w_a || !dx) return HAWK_ERR_NULL_POINTER;
+    if (!dtype_ok(g_dtype) || !dtype_ok(w_dtype) || !dtype_ok(dx_dtype)) return HAWK_ERR_BAD_DTYPE;
+    if (M < 1 || !hawk_gate_proj_supported(D, num_blocks)) return HAWK_ERR_BAD_SHAPE;
+    if (!aligned16(d_x_rg_lru) || !aligned16(d_a_rg_lru) || !aligned16(dx) || !aligned16(w_i) || !aligned16(w_a))
+        return HAWK_ERR_ALIGNMENT;
+    return hawk::gate_proj_bwd_input(d_x_rg_lru, d_a_rg_lru, w_i, w_a, dx, M, D, num_blocks, g_dtype, w_dtype,
+                                     dx_dtype, as_stream(stream));
+}
+
+size_t hawk_gate_proj_bwd_weights_workspace_bytes(int M, int D, int num_blocks) {
+    if (M < 1 || !hawk_gate_proj_supported(D, num_blocks)) return 0;
+    return hawk::gate_proj_bwd_weights_workspace_bytes(M, D, num_blocks);
+}
+
+int hawk_gate_proj_bwd_weights(const void* x, const void* d_x_rg_lru, const void* d_a_rg_lru, float* dw_i,
+                               float* db_i, float* dw_a, float* db_a, int M, int D, int num_blocks, int x_dtype,
+                               int g_dtype, void* workspace_device, size_t workspace_bytes, void* stream) {
+    if (!x || !d_x_rg_lru || !d_a_rg_lru || !dw_i || !dw_a) return HAWK_ERR_NULL_POINTER;
+    if (!dtype_ok(x_dtype) || !dtype_ok(g_dtype)) return HAWK_ERR_BAD_DTYPE;
+    if (M < 1 || !hawk_gate_proj_supported(D, num_blocks)) return HAWK_ERR_BAD_SHAPE;
+    if (!aligned16(x) || !aligned16(d_x_rg_lru) || !aligned16(d_a_rg_lru)) return HAWK_ERR_ALIGNMENT;
+    if (workspace_device == nullptr) return HAWK_ERR_WORKSPACE;
+    if (!aligned16(workspace_device)) return HAWK_ERR_ALIGNMENT;
+    return hawk::gate_proj_bwd_weights(x, d_x_rg_lru, d_a_rg_lru, dw_i, db_i, dw_a, db_a, M, D, num_blocks, x_dtype,
+                                       g_dtype, workspace_device, workspace_bytes, as_stream(stream));
+}
+
 }  // extern "C"

@@ -207,6 +207,338 @@ __global__ __launch_bounds__(kGateThreads, 1) void gate_proj_fwd_kernel(
     }
 }
 
+// ---------------------------------------------------------------------------------------
+// Input gradient of the two projections:
+//   dx[m, h*bw + i] = sum_j dxg[m, h*bw + j] w_i[h, i, j] + sum_j dag[m, h*bw + j] w_a[h, i, j]
+// Same decomposition as the forward: wave (g, c) keeps w_g[h, 32c.., :] (rows of the weight
+// matrix, contiguous in memory) as B operands, reads gate g's gradient tile from LDS as A
+// operands, and the two gates' partial tiles are added on the way out.
+// ---------------------------------------------------------------------------------------
+template <typename GT, typename WT, typename DT, int BW>
+__global__ __launch_bounds__(kGateThreads, 1) void gate_proj_bwd_input_kernel(
+    const GT* __restrict__ dxg, const GT* __restrict__ dag, const WT* __restrict__ w_i, const WT* __restrict__ w_a,
+    DT* __restrict__ dx, int M, int D, int nb, int ntiles) {
+    constexpr int KS = BW / 16;
+    constexpr int G = kGroup / BW;
+    constexpr int kORowBytes = kGroup * 4 + 16;             // fp32 partial sums of one gate, one row
+    constexpr int kOTileBytes = kTileRows * kORowBytes;
+    extern __shared__ __align__(16) unsigned char smem[];
+    unsigned char* sA = smem;                               // [stage][gate] gradient tiles
+    unsigned char* sO = smem + 4 * kATileBytes;             // [gate] partial result tiles
+
+    const int tid = threadIdx.x;
+    const int lane = tid & (kWave - 1);
+    const int w = __builtin_amdgcn_readfirstlane(tid / kWave);
+    const int group = blockIdx.y, worker = blockIdx.x, nworkers = gridDim.x;
+    const int g = w >> 3, c = w & 7;
+    const int blk = (32 * c) / BW;
+    const int h = group * G + blk;
+    const int col = lane & 31, khalf = 8 * (lane >> 5);
+    const int i_in = 32 * c - blk * BW + col;               // input channel within the block
+    const WT* wsel = g ? w_a : w_i;
+
+    const int lrow = tid >> 5, lc8 = tid & 31;
+    const int lcol = group * kGroup + lc8 * 8;
+    const bool col_ok = lcol < D;
+    auto load_tile = [&](int it, Row8<GT>& r0, Row8<GT>& r1) {
+        const int t = worker + it * nworkers;
+        const int row = t * kTileRows + lrow;
+        const bool ok = col_ok && t < ntiles && row < M;
+        const size_t off = ok ? (size_t)row * D + lcol : 0;
+        r0.load(dxg + off, ok);
+        r1.load(dag + off, ok);
+    };
+    auto stage_tile = [&](int buf, const Row8<GT>& r0, const Row8<GT>& r1) {
+        unsigned char* p = sA + (2 * buf) * kATileBytes + lrow * kARowBytes + lc8 * 16;
+        *reinterpret_cast<u32x4*>(p) = r0.as_bf16();
+        *reinterpret_cast<u32x4*>(p + kATileBytes) = r1.as_bf16();
+    };
+
+    Row8<GT> ra0, ra1, rb0, rb1;
+    load_tile(0, ra0, ra1);
+    load_tile(1, rb0, rb1);
+    __builtin_amdgcn_sched_barrier(0);
+
+    // weights: lane holds row i of w_g[h] and 8 consecutive j per k-step (contiguous)
+    const float live = (h < nb) ? 1.0f : 0.0f;
+    const WT* wrow = wsel + ((size_t)min(h, nb - 1) * BW + i_in) * BW + khalf;
+    bf16x8 bfrag[KS];
+    constexpr int kWBatch = KS < 4 ? KS : 4;
+#pragma unroll
+    for (int s0 = 0; s0 < KS; s0 += kWBatch) {
+        float v[kWBatch][8];
+#pragma unroll
+        for (int j = 0; j < kWBatch; ++j)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) v[j][e] = elem_to_f32(wrow[16 * (s0 + j) + e]);
+#pragma unroll
+        for (int j = 0; j < kWBatch; ++j) {
+            const u32x4 packed = {pack_bf16x2(live * v[j][0], live * v[j][1]), pack_bf16x2(live * v[j][2], live * v[j][3]),
+                                  pack_bf16x2(live * v[j][4], live * v[j][5]), pack_bf16x2(live * v[j][6], live * v[j][7])};
+            bfrag[s0 + j] = __builtin_bit_cast(bf16x8, packed);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    }
+
+    stage_tile(0, ra0, ra1);
+    load_tile(2, ra0, ra1);
+    __syncthreads();
+
+    const int a_off = g * kATileBytes + col * kARowBytes + (blk * BW + khalf) * 2;
+    unsigned char* o_base = sO + g * kOTileBytes + (4 * (lane >> 5)) * kORowBytes + (32 * c + col) * 4;
+    const unsigned char* o_src = sO + lrow * kORowBytes + lc8 * 32;
+
+    auto step = [&](int it, int cur, Row8<GT>& rn0, Row8<GT>& rn1) {
+        f32x16 acc = {};
+        const unsigned char* a_base = sA + (2 * cur) * kATileBytes + a_off;
+        constexpr int kBatch = KS < 4 ? KS : 4;
+#pragma unroll
+        for (int s0 = 0; s0 < KS; s0 += kBatch) {
+            bf16x8 a[kBatch];
+#pragma unroll
+            for (int j = 0; j < kBatch; ++j) a[j] = *reinterpret_cast<const bf16x8*>(a_base + (s0 + j) * 32);
+#pragma unroll
+            for (int j = 0; j < kBatch; ++j)
+                acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[j], bfrag[s0 + j], acc, 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int m = 8 * (r / 4) + (r % 4);
+            *reinterpret_cast<float*>(o_base + m * kORowBytes) = acc[r];
+        }
+        stage_tile(cur ^ 1, rn0, rn1);
+        load_tile(it + 3, rn0, rn1);
+        __syncthreads();
+        const int row = (worker + it * nworkers) * kTileRows + lrow;
+        if (col_ok && row < M) {
+            const f32x4 p0 = *reinterpret_cast<const f32x4*>(o_src), p1 = *reinterpret_cast<const f32x4*>(o_src + 16);
+            const f32x4 q0 = *reinterpret_cast<const f32x4*>(o_src + kOTileBytes);
+            const f32x4 q1 = *reinterpret_cast<const f32x4*>(o_src + kOTileBytes + 16);
+            const f32x4 s0 = p0 + q0, s1 = p1 + q1;
+            DT* dst = dx + (size_t)row * D + lcol;
+            if constexpr (sizeof(DT) == 4) {
+                __builtin_nontemporal_store(s0, reinterpret_cast<f32x4*>(dst));
+                __builtin_nontemporal_store(s1, reinterpret_cast<f32x4*>(dst) + 1);
+            } else {
+                const u32x4 packed = {pack_bf16x2(s0.x, s0.y), pack_bf16x2(s0.z, s0.w), pack_bf16x2(s1.x, s1.y),
+                                      pack_bf16x2(s1.z, s1.w)};
+                __builtin_nontemporal_store(packed, reinterpret_cast<u32x4*>(dst));
+            }
+        }
+        __syncthreads();
+    };
+
+    for (int it = 0; worker + it * nworkers < ntiles; it += 2) {
+        step(it, 0, rb0, rb1);
+        if (worker + (it + 1) * nworkers >= ntiles) break;
+        step(it + 1, 1, ra0, ra1);
+    }
+}
+
+// ---------------------------------------------------------------------------------------
+// Weight and bias gradients:
+//   dw_g[h, i, j] = sum_m x[m, h*bw + i] dg[m, h*bw + j],   db_g[c] = sum_m dg[m, c]
+// The contraction runs over the rows, so both operands are needed "column-wise".  A
+// workgroup (msplit, 256-channel group, gate) walks over its share of the rows 32 at a time;
+// waves 0-7 fetch the x tile and waves 8-15 the gradient tile, each lane 8 rows of two
+// adjacent channels, transpose them in registers and write them to LDS as
+// [8-row chunk][channel][8 rows], which is exactly the 16 bytes an MFMA operand lane needs
+// (bank-conflict free both ways).  Every wave accumulates up to 2 x 2 output tiles of
+// 32 x 32 in registers over the whole row range and writes them to a per-split partial
+// buffer; a second kernel adds the splits in a fixed order.
+// ---------------------------------------------------------------------------------------
+constexpr int kChunkBytes = kGroup * 16;          // one 8-row chunk of a transposed tile
+constexpr int kTTileBytes = 4 * kChunkBytes;      // 32 rows
+
+template <typename ET>
+__device__ __forceinline__ void load_pair(const ET* p, bool ok, uint32_t (&raw)[2]);
+template <>
+__device__ __forceinline__ void load_pair<bf16_t>(const bf16_t* p, bool ok, uint32_t (&raw)[2]) {
+    raw[0] = ok ? *reinterpret_cast<const uint32_t*>(p) : 0u;
+    raw[1] = 0u;
+}
+template <>
+__device__ __forceinline__ void load_pair<float>(const float* p, bool ok, uint32_t (&raw)[2]) {
+    const u32x2 v = ok ? *reinterpret_cast<const u32x2*>(p) : u32x2{0u, 0u};
+    raw[0] = v.x;
+    raw[1] = v.y;
+}
+template <typename ET>
+__device__ __forceinline__ uint32_t pair_as_bf16(const uint32_t (&raw)[2]) {
+    if constexpr (sizeof(ET) == 2) return raw[0];
+    return pack_bf16x2(__uint_as_float(raw[0]), __uint_as_float(raw[1]));
+}
+
+template <typename XT, typename GT, int BW>
+__global__ __launch_bounds__(kGateThreads, 1) void gate_proj_bwd_weights_kernel(
+    const XT* __restrict__ x, const GT* __restrict__ dg_i, const GT* __restrict__ dg_a, float* __restrict__ part_w,
+    float* __restrict__ part_b, int M, int D, int nb, int rows_per_split) {
+    constexpr int G = kGroup / BW;                 // blocks per group
+    constexpr int NT = BW / 32;                    // 32-wide tiles per block side
+    constexpr int TI = BW >= 256 ? 2 : 1;          // output tiles per wave: TI x TJ
+    constexpr int TJ = BW >= 128 ? 2 : 1;
+    constexpr int WPB = (NT * NT) / (TI * TJ);     // waves per block
+    constexpr int RAWW = (sizeof(XT) > 2 || sizeof(GT) > 2) ? 2 : 1;
+    __shared__ __align__(16) unsigned char sT[2][2][kTTileBytes];   // [stage][x | dg][chunk][channel][8 rows]
+    __shared__ float s_db[4][kGroup];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & (kWave - 1);
+    const int w = __builtin_amdgcn_readfirstlane(tid / kWave);
+    const int split = blockIdx.x, group = blockIdx.y, gate = blockIdx.z;
+    const GT* dg = gate ? dg_a : dg_i;
+    const int row_begin = split * rows_per_split;
+    const int row_end = min(row_begin + rows_per_split, M);
+    const int ntiles = (row_end - row_begin + kTileRows - 1) / kTileRows;
+
+    // ---- loader role: 8 rows x 2 channels per lane
+    const bool loads_x = w < 8;
+    const int q = (w & 7) >> 1;                                  // 8-row chunk of the tile
+    const int c2 = (w & 1) * 64 + lane;                          // channel pair within the group
+    const int lch = group * kGroup + 2 * c2;
+    const bool ch_ok = lch < D;
+    uint32_t ra[8][RAWW], rb[8][RAWW];
+    auto load_rows = [&](int t, uint32_t (&r)[8][RAWW]) {
+        const int row0 = row_begin + t * kTileRows + 8 * q;
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            const bool ok = ch_ok && t < ntiles && row0 + k < row_end;
+            const size_t off = ok ? (size_t)(row0 + k) * D + lch : 0;
+            uint32_t tmp[2];
+            if (loads_x) load_pair<XT>(x + off, ok, tmp);
+            else load_pair<GT>(dg + off, ok, tmp);
+#pragma unroll
+            for (int z = 0; z < RAWW; ++z) r[k][z] = tmp[z];
+        }
+    };
+    float colsum[2] = {0.0f, 0.0f};
+    auto stage_rows = [&](int buf, const uint32_t (&r)[8][RAWW]) {
+        uint32_t d[8];
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            uint32_t tmp[2] = {r[k][0], RAWW > 1 ? r[k][RAWW - 1] : 0u};
+            d[k] = loads_x ? pair_as_bf16<XT>(tmp) : pair_as_bf16<GT>(tmp);
+        }
+        if (!loads_x) {
+#pragma unroll
+            for (int k = 0; k < 8; ++k) {
+                colsum[0] += bf16_lo(d[k]);
+                colsum[1] += bf16_hi(d[k]);
+            }
+        }
+        // channel 2 c2 takes the low halves, channel 2 c2 + 1 the high halves; rows in order
+        u32x4 lo, hi;
+        lo.x = (d[0] & 0xffffu) | (d[1] << 16);
+        lo.y = (d[2] & 0xffffu) | (d[3] << 16);
+        lo.z = (d[4] & 0xffffu) | (d[5] << 16);
+        lo.w = (d[6] & 0xffffu) | (d[7] << 16);
+        hi.x = (d[0] >> 16) | (d[1] & 0xffff0000u);
+        hi.y = (d[2] >> 16) | (d[3] & 0xffff0000u);
+        hi.z = (d[4] >> 16) | (d[5] & 0xffff0000u);
+        hi.w = (d[6] >> 16) | (d[7] & 0xffff0000u);
+        unsigned char* p = &sT[buf][loads_x ? 0 : 1][q * kChunkBytes + (2 * c2) * 16];
+        *reinterpret_cast<u32x4*>(p) = lo;
+        *reinterpret_cast<u32x4*>(p + 16) = hi;
+    };
+
+    // ---- compute role: TI x TJ output tiles of block `blk`
+    const int blk = w / WPB;                       // block within the group (idle if >= G)
+    const int wi = w % WPB;
+    const int i0 = (wi / (NT / TJ)) * TI, j0 = (wi % (NT / TJ)) * TJ;
+    const int h = group * G + blk;
+    const bool computes = blk < G && h < nb;
+    const int col = lane & 31;
+    const int a_off = (lane >> 5) * kChunkBytes + (blk * BW + i0 * 32 + col) * 16;
+    const int b_off = (lane >> 5) * kChunkBytes + (blk * BW + j0 * 32 + col) * 16;
+    f32x16 acc[TI][TJ];
+#pragma unroll
+    for (int a = 0; a < TI; ++a)
+#pragma unroll
+        for (int b = 0; b < TJ; ++b) acc[a][b] = f32x16{};
+
+    load_rows(0, ra);
+    load_rows(1, rb);
+    stage_rows(0, ra);
+    load_rows(2, ra);
+    __syncthreads();
+
+    auto step = [&](int t, int cur, uint32_t (&rnext)[8][RAWW]) {
+        if (computes) {
+#pragma unroll
+            for (int ks = 0; ks < 2; ++ks) {
+                bf16x8 fa[TI], fb[TJ];
+#pragma unroll
+                for (int a = 0; a < TI; ++a)
+                    fa[a] = *reinterpret_cast<const bf16x8*>(&sT[cur][0][2 * ks * kChunkBytes + a_off + a * 32 * 16]);
+#pragma unroll
+                for (int b = 0; b < TJ; ++b)
+                    fb[b] = *reinterpret_cast<const bf16x8*>(&sT[cur][1][2 * ks * kChunkBytes + b_off + b * 32 * 16]);
+#pragma unroll
+                for (int a = 0; a < TI; ++a)
+#pragma unroll
+                    for (int b = 0; b < TJ; ++b)
+                        acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[a], fb[b], acc[a][b], 0, 0, 0);
+            }
+        }
+        stage_rows(cur ^ 1, rnext);
+        load_rows(t + 3, rnext);
+        __syncthreads();
+    };
+    for (int t = 0; t < ntiles; t += 2) {
+        step(t, 0, rb);
+        if (t + 1 >= ntiles) break;
+        step(t + 1, 1, ra);
+    }
+
+    // ---- partial results of this split
+    if (computes) {
+        float* dst = part_w + (((size_t)split * 2 + gate) * nb + h) * BW * BW;
+#pragma unroll
+        for (int a = 0; a < TI; ++a)
+#pragma unroll
+            for (int b = 0; b < TJ; ++b)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int i = (i0 + a) * 32 + 8 * (r / 4) + 4 * (lane >> 5) + (r % 4);
+                    const int j = (j0 + b) * 32 + col;
+                    dst[(size_t)i * BW + j] = acc[a][b][r];
+                }
+    }
+    if (!loads_x) {
+        s_db[q][2 * c2] = colsum[0];
+        s_db[q][2 * c2 + 1] = colsum[1];
+    }
+    __syncthreads();
+    if (tid < kGroup && group * kGroup + tid < D)
+        part_b[((size_t)split * 2 + gate) * D + group * kGroup + tid] =
+            (s_db[0][tid] + s_db[1][tid]) + (s_db[2][tid] + s_db[3][tid]);
+}
+
+// dw_g = sum over splits of the partial tiles, db_g likewise; fixed order.
+__global__ void gate_proj_reduce_kernel(const float* __restrict__ part_w, const float* __restrict__ part_b,
+                                        float* __restrict__ dw_i, float* __restrict__ dw_a, float* __restrict__ db_i,
+                                        float* __restrict__ db_a, int nsplit, size_t wcount, int D) {
+    const size_t total = 2 * wcount + 2 * (size_t)D;
+    for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+         idx += (size_t)gridDim.x * blockDim.x) {
+        float sum = 0.0f;
+        if (idx < 2 * wcount) {
+            for (int s = 0; s < nsplit; ++s) sum += part_w[(size_t)s * 2 * wcount + idx];
+            if (idx < wcount) dw_i[idx] = sum;
+            else dw_a[idx - wcount] = sum;
+        } else {
+            const size_t k = idx - 2 * wcount;
+            for (int s = 0; s < nsplit; ++s) sum += part_b[(size_t)s * 2 * D + k];
+            if (k < (size_t)D) {
+                if (db_i != nullptr) db_i[k] = sum;
+            } else if (db_a != nullptr) {
+                db_a[k - D] = sum;
+            }
+        }
+    }
+}
+
 inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
 
 template <typename XT, typename WT, typename OT, int BW>
@@ -248,6 +580,76 @@ int gate_fwd_out(const void* x, const void* w_i, const float* b_i, const void* w
     return gate_fwd_bw<XT, WT, float>(x, w_i, b_i, w_a, b_a, out_i, out_a, M, D, nb, bw, st);
 }
 
+template <typename GT, typename WT, typename DT, int BW>
+int launch_gate_bwd_input(const void* dxg, const void* dag, const void* w_i, const void* w_a, void* dx, int M, int D,
+                          int nb, hipStream_t st) {
+    const int ngroups = ceil_div(D, kGroup);
+    const int ntiles = ceil_div(M, kTileRows);
+    int nworkers = kNumCU / ngroups;
+    if (nworkers < 1) nworkers = 1;
+    if (nworkers > ntiles) nworkers = ntiles;
+    const size_t smem = 4 * kATileBytes + 2 * (size_t)kTileRows * (kGroup * 4 + 16);
+    auto kernel = gate_proj_bwd_input_kernel<GT, WT, DT, BW>;
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                            (int)smem) != hipSuccess)
+        return HAWK_ERR_LAUNCH;
+    hipLaunchKernelGGL(kernel, dim3((unsigned)nworkers, (unsigned)ngroups), dim3(kGateThreads), smem, st,
+                       static_cast<const GT*>(dxg), static_cast<const GT*>(dag), static_cast<const WT*>(w_i),
+                       static_cast<const WT*>(w_a), static_cast<DT*>(dx), M, D, nb, ntiles);
+    return hipGetLastError() == hipSuccess ? HAWK_OK : HAWK_ERR_LAUNCH;
+}
+
+template <typename GT, typename WT, typename DT>
+int gate_bwd_input_bw(const void* dxg, const void* dag, const void* w_i, const void* w_a, void* dx, int M, int D,
+                      int nb, int bw, hipStream_t st) {
+    switch (bw) {
+        case 32: return launch_gate_bwd_input<GT, WT, DT, 32>(dxg, dag, w_i, w_a, dx, M, D, nb, st);
+        case 64: return launch_gate_bwd_input<GT, WT, DT, 64>(dxg, dag, w_i, w_a, dx, M, D, nb, st);
+        case 128: return launch_gate_bwd_input<GT, WT, DT, 128>(dxg, dag, w_i, w_a, dx, M, D, nb, st);
+        case 256: return launch_gate_bwd_input<GT, WT, DT, 256>(dxg, dag, w_i, w_a, dx, M, D, nb, st);
+        default: return HAWK_ERR_BAD_SHAPE;
+    }
+}
+
+template <typename GT, typename WT>
+int gate_bwd_input_out(const void* dxg, const void* dag, const void* w_i, const void* w_a, void* dx, int M, int D,
+                       int nb, int bw, int dx_dtype, hipStream_t st) {
+    if (dx_dtype == HAWK_DTYPE_BF16)
+        return gate_bwd_input_bw<GT, WT, bf16_t>(dxg, dag, w_i, w_a, dx, M, D, nb, bw, st);
+    return gate_bwd_input_bw<GT, WT, float>(dxg, dag, w_i, w_a, dx, M, D, nb, bw, st);
+}
+
+int weight_splits(int M, int D) {
+    const int ngroups = ceil_div(D, kGroup);
+    int n = kNumCU / (2 * ngroups);
+    if (n < 1) n = 1;
+    const int ntiles = ceil_div(M, kTileRows);
+    return n > ntiles ? ntiles : n;
+}
+
+template <typename XT, typename GT, int BW>
+int launch_gate_bwd_weights(const void* x, const void* dg_i, const void* dg_a, float* part_w, float* part_b, int M,
+                            int D, int nb, int nsplit, hipStream_t st) {
+    const int rows_per_split = ceil_div(ceil_div(M, nsplit), kTileRows) * kTileRows;
+    hipLaunchKernelGGL((gate_proj_bwd_weights_kernel<XT, GT, BW>),
+                       dim3((unsigned)nsplit, (unsigned)ceil_div(D, kGroup), 2u), dim3(kGateThreads), 0, st,
+                       static_cast<const XT*>(x), static_cast<const GT*>(dg_i), static_cast<const GT*>(dg_a), part_w,
+                       part_b, M, D, nb, rows_per_split);
+    return hipGetLastError() == hipSuccess ? HAWK_OK : HAWK_ERR_LAUNCH;
+}
+
+template <typename XT, typename GT>
+int gate_bwd_weights_bw(const void* x, const void* dg_i, const void* dg_a, float* part_w, float* part_b, int M, int D,
+                        int nb, int bw, int nsplit, hipStream_t st) {
+    switch (bw) {
+        case 32: return launch_gate_bwd_weights<XT, GT, 32>(x, dg_i, dg_a, part_w, part_b, M, D, nb, nsplit, st);
+        case 64: return launch_gate_bwd_weights<XT, GT, 64>(x, dg_i, dg_a, part_w, part_b, M, D, nb, nsplit, st);
+        case 128: return launch_gate_bwd_weights<XT, GT, 128>(x, dg_i, dg_a, part_w, part_b, M, D, nb, nsplit, st);
+        case 256: return launch_gate_bwd_weights<XT, GT, 256>(x, dg_i, dg_a, part_w, part_b, M, D, nb, nsplit, st);
+        default: return HAWK_ERR_BAD_SHAPE;
+    }
+}
+
 }  // namespace
 
 bool gate_proj_block_width_supported(int bw) { return bw == 32 || bw == 64 || bw == 128 || bw == 256; }
@@ -263,6 +665,52 @@ int gate_proj_fwd(const void* x, const void* w_i, const float* b_i, const void* 
     if (w_dtype == HAWK_DTYPE_BF16)
         return gate_fwd_out<float, bf16_t>(x, w_i, b_i, w_a, b_a, out_i, out_a, M, D, nb, bw, out_dtype, st);
     return gate_fwd_out<float, float>(x, w_i, b_i, w_a, b_a, out_i, out_a, M, D, nb, bw, out_dtype, st);
+}
+
+int gate_proj_bwd_input(const void* dxg, const void* dag, const void* w_i, const void* w_a, void* dx, int M, int D,
+                        int nb, int g_dtype, int w_dtype, int dx_dtype, hipStream_t st) {
+    const int bw = D / nb;
+    if (g_dtype == HAWK_DTYPE_BF16) {
+        if (w_dtype == HAWK_DTYPE_BF16)
+            return gate_bwd_input_out<bf16_t, bf16_t>(dxg, dag, w_i, w_a, dx, M, D, nb, bw, dx_dtype, st);
+        return gate_bwd_input_out<bf16_t, float>(dxg, dag, w_i, w_a, dx, M, D, nb, bw, dx_dtype, st);
+    }
+    if (w_dtype == HAWK_DTYPE_BF16)
+        return gate_bwd_input_out<float, bf16_t>(dxg, dag, w_i, w_a, dx, M, D, nb, bw, dx_dtype, st);
+    return gate_bwd_input_out<float, float>(dxg, dag, w_i, w_a, dx, M, D, nb, bw, dx_dtype, st);
+}
+
+size_t gate_proj_bwd_weights_workspace_bytes(int M, int D, int nb) {
+    const size_t bw = (size_t)(D / nb);
+    return (size_t)weight_splits(M, D) * 2 * ((size_t)nb * bw * bw + (size_t)D) * sizeof(float);
+}
+
+int gate_proj_bwd_weights(const void* x, const void* dg_i, const void* dg_a, float* dw_i, float* db_i, float* dw_a,
+                          float* db_a, int M, int D, int nb, int x_dtype, int g_dtype, void* ws, size_t ws_bytes,
+                          hipStream_t st) {
+    const int bw = D / nb;
+    const int nsplit = weight_splits(M, D);
+    const size_t wcount = (size_t)nb * bw * bw;
+    if (ws == nullptr || ws_bytes < gate_proj_bwd_weights_workspace_bytes(M, D, nb)) return HAWK_ERR_WORKSPACE;
+    float* part_w = static_cast<float*>(ws);
+    float* part_b = part_w + (size_t)nsplit * 2 * wcount;
+    int rc;
+    if (x_dtype == HAWK_DTYPE_BF16) {
+        rc = g_dtype == HAWK_DTYPE_BF16
+                 ? gate_bwd_weights_bw<bf16_t, bf16_t>(x, dg_i, dg_a, part_w, part_b, M, D, nb, bw, nsplit, st)
+                 : gate_bwd_weights_bw<bf16_t, float>(x, dg_i, dg_a, part_w, part_b, M, D, nb, bw, nsplit, st);
+    } else {
+        rc = g_dtype == HAWK_DTYPE_BF16
+                 ? gate_bwd_weights_bw<float, bf16_t>(x, dg_i, dg_a, part_w, part_b, M, D, nb, bw, nsplit, st)
+                 : gate_bwd_weights_bw<float, float>(x, dg_i, dg_a, part_w, part_b, M, D, nb, bw, nsplit, st);
+    }
+    if (rc != HAWK_OK) return rc;
+    const size_t total = 2 * wcount + 2 * (size_t)D;
+    size_t blocks = (total + 255) / 256;
+    if (blocks > 4096) blocks = 4096;
+    hipLaunchKernelGGL(gate_proj_reduce_kernel, dim3((unsigned)blocks), dim3(256), 0, st, part_w, part_b, dw_i, dw_a,
+                       db_i, db_a, nsplit, wcount, D);
+    return hipGetLastError() == hipSuccess ? HAWK_OK : HAWK_ERR_LAUNCH;
 }
 
 }  // namespace hawk

@@ -206,6 +206,27 @@ int hawk_gate_proj_fwd(const void* x, const void* w_i, const float* b_i, const v
                        const float* b_a, void* x_rg_lru, void* a_rg_lru, int M, int D,
                        int num_blocks, int x_dtype, int w_dtype, int out_dtype, void* stream);
 
+/* Gradient of the two projections with respect to x, in one pass over both logit gradients:
+ *   dx[m, h*bw+i] = sum_j d_x_rg_lru[m, h*bw+j] w_i[h, i, j] + sum_j d_a_rg_lru[m, h*bw+j] w_a[h, i, j]
+ * (what autograd derives from the einsum of hawk/external.py:230, twice, plus the add of
+ * the two results).  Gradients have g_dtype, weights w_dtype, dx has dx_dtype; operands are
+ * rounded to bf16 in registers, sums are fp32. */
+int hawk_gate_proj_bwd_input(const void* d_x_rg_lru, const void* d_a_rg_lru, const void* w_i,
+                             const void* w_a, void* dx, int M, int D, int num_blocks, int g_dtype,
+                             int w_dtype, int dx_dtype, void* stream);
+
+/* Gradients of the weights and biases of the two projections:
+ *   dw_g[h, i, j] = sum_m x[m, h*bw+i] d_g[m, h*bw+j],   db_g[c] = sum_m d_g[m, c]
+ * (autograd of hawk/external.py:230 with respect to w and b).  dw_i, dw_a
+ * [num_blocks, bw, bw] and db_i, db_a [D] (may be NULL) are fp32 and are overwritten.  The
+ * row range is split over workgroups; their partial sums live in the caller's workspace
+ * (size from the query) and are added in a fixed order, so results are reproducible. */
+size_t hawk_gate_proj_bwd_weights_workspace_bytes(int M, int D, int num_blocks);
+int hawk_gate_proj_bwd_weights(const void* x, const void* d_x_rg_lru, const void* d_a_rg_lru,
+                               float* dw_i, float* db_i, float* dw_a, float* db_a, int M, int D,
+                               int num_blocks, int x_dtype, int g_dtype, void* workspace_device,
+                               size_t workspace_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

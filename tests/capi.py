@@ -214,3 +214,33 @@ def gate_proj_fwd(x, w_i, b_i, w_a, b_a, out_dtype=None):
         M, D, nb, _lib.dtype_code(x.dtype), _lib.dtype_code(w_i.dtype), _lib.dtype_code(out_dtype), _stream())
     _lib.check("hawk_gate_proj_fwd", rc)
     return oi, oa
+
+
+def gate_proj_bwd_input(dxg, dag, w_i, w_a, dx_dtype=None):
+    M, D = dxg.shape
+    nb = w_i.shape[0]
+    dx_dtype = dx_dtype or dxg.dtype
+    dx = torch.empty((M, D), dtype=dx_dtype, device="cuda")
+    rc = _lib.load().hawk_gate_proj_bwd_input(
+        dxg.data_ptr(), dag.data_ptr(), w_i.data_ptr(), w_a.data_ptr(), dx.data_ptr(), M, D, nb,
+        _lib.dtype_code(dxg.dtype), _lib.dtype_code(w_i.dtype), _lib.dtype_code(dx_dtype), _stream())
+    _lib.check("hawk_gate_proj_bwd_input", rc)
+    return dx
+
+
+def gate_proj_bwd_weights(x, dxg, dag, nb, with_bias=True):
+    M, D = x.shape
+    bw = D // nb
+    lib = _lib.load()
+    n = lib.hawk_gate_proj_bwd_weights_workspace_bytes(M, D, nb)
+    assert n > 0
+    ws = torch.full((n,), 0xAB, dtype=torch.uint8, device="cuda")  # garbage: the kernels must not rely on zeros
+    dwi = torch.empty((nb, bw, bw), dtype=torch.float32, device="cuda")
+    dwa = torch.empty_like(dwi)
+    dbi = torch.empty(D, dtype=torch.float32, device="cuda") if with_bias else None
+    dba = torch.empty(D, dtype=torch.float32, device="cuda") if with_bias else None
+    rc = lib.hawk_gate_proj_bwd_weights(
+        x.data_ptr(), dxg.data_ptr(), dag.data_ptr(), dwi.data_ptr(), _lib.ptr(dbi), dwa.data_ptr(), _lib.ptr(dba),
+        M, D, nb, _lib.dtype_code(x.dtype), _lib.dtype_code(dxg.dtype), ws.data_ptr(), n, _stream())
+    _lib.check("hawk_gate_proj_bwd_weights", rc)
+    return dwi, dbi, dwa, dba

@@ -96,3 +96,95 @@ def test_full_benchmark_shape_against_the_library_gemm():
         ref = torch.bmm(xb.float(), w.to(torch.bfloat16).float()).transpose(0, 1).reshape(M, D) + b
         err = float((got - ref).abs().max() / ref.abs().max())
         assert err < 1e-4, err
+
+
+# ---------------------------------------------------------------------------------------- input gradient
+def _bwd_input_case(M, D, nb, g_dtype, w_dtype, dx_dtype, seed=0):
+    rng = np.random.default_rng(seed)
+    bw = D // nb
+    gi, ga = rng.standard_normal((M, D)), rng.standard_normal((M, D))
+    wi = rng.standard_normal((nb, bw, bw)) / np.sqrt(bw)
+    wa = rng.standard_normal((nb, bw, bw)) / np.sqrt(bw)
+    gid, gad = capi.to_dev(gi, g_dtype), capi.to_dev(ga, g_dtype)
+    wid, wad = capi.to_dev(wi, w_dtype), capi.to_dev(wa, w_dtype)
+    dx = capi.gate_proj_bwd_input(gid, gad, wid, wad, capi.TORCH_DTYPE[dx_dtype])
+    torch.cuda.synchronize()
+    zeros = np.zeros((M, D))
+    ref = (oracle.block_diagonal_linear_bwd(zeros, _bf16_round(capi.to_np(wid)), _bf16_round(capi.to_np(gid)))[0]
+           + oracle.block_diagonal_linear_bwd(zeros, _bf16_round(capi.to_np(wad)), _bf16_round(capi.to_np(gad)))[0])
+    tol = 2e-2 if dx_dtype == "bf16" else 1e-4
+    assert max_rel(capi.to_np(dx), ref) < tol, (M, D, nb, max_rel(capi.to_np(dx), ref))
+
+
+@pytest.mark.parametrize("D,nb", [(256, 1), (2560, 10), (512, 16), (512, 8), (512, 4), (768, 3), (384, 3), (96, 3)])
+@pytest.mark.parametrize("M", [1, 33, 1000])
+def test_input_gradient_block_widths_and_ragged_rows(M, D, nb):
+    _bwd_input_case(M, D, nb, "bf16", "f32", "f32", seed=M + D)
+
+
+@pytest.mark.parametrize("g_dtype,w_dtype,dx_dtype", [("bf16", "bf16", "bf16"), ("f32", "f32", "f32"),
+                                                      ("bf16", "f32", "bf16"), ("f32", "bf16", "bf16")])
+def test_input_gradient_dtype_combinations(g_dtype, w_dtype, dx_dtype):
+    _bwd_input_case(4096 + 17, 2560, 10, g_dtype, w_dtype, dx_dtype, seed=7)
+    _bwd_input_case(300, 512, 16, g_dtype, w_dtype, dx_dtype, seed=8)
+
+
+def test_input_gradient_is_the_adjoint_of_the_forward():
+    """<forward(x), (gi, ga)> == <x, bwd_input(gi, ga)> with zero bias, on the full shape."""
+    M, D, nb = 32768, 2560, 10
+    g = torch.Generator(device="cuda").manual_seed(2)
+    mk = lambda: torch.randn((M, D), generator=g, device="cuda").to(torch.bfloat16)  # noqa: E731
+    x, gi, ga = mk(), mk(), mk()
+    wi = torch.randn((nb, 256, 256), generator=g, device="cuda") / 16.0
+    wa = torch.randn((nb, 256, 256), generator=g, device="cuda") / 16.0
+    oi, oa = capi.gate_proj_fwd(x, wi, None, wa, None, torch.float32)
+    dx = capi.gate_proj_bwd_input(gi, ga, wi, wa, torch.float32)
+    lhs = (oi.double() * gi.double()).sum() + (oa.double() * ga.double()).sum()
+    rhs = (x.double() * dx.double()).sum()
+    assert abs(float(lhs - rhs)) < 1e-5 * abs(float(lhs)), (float(lhs), float(rhs))
+
+
+# ---------------------------------------------------------------------------------------- weight gradients
+def _bwd_weights_case(M, D, nb, x_dtype, g_dtype, seed=0):
+    rng = np.random.default_rng(seed)
+    bw = D // nb
+    x, gi, ga = (rng.standard_normal((M, D)) for _ in range(3))
+    xd, gid, gad = capi.to_dev(x, x_dtype), capi.to_dev(gi, g_dtype), capi.to_dev(ga, g_dtype)
+    dwi, dbi, dwa, dba = capi.gate_proj_bwd_weights(xd, gid, gad, nb)
+    torch.cuda.synchronize()
+    xr = _bf16_round(capi.to_np(xd))
+    zeros_w = np.zeros((nb, bw, bw))
+    for name, gd, dw, db in (("i", gid, dwi, dbi), ("a", gad, dwa, dba)):
+        gr = _bf16_round(capi.to_np(gd))
+        _, ref_w, ref_b = oracle.block_diagonal_linear_bwd(xr, zeros_w, gr)
+        assert max_rel(capi.to_np(dw), ref_w) < 1e-4, (name, M, D, nb, max_rel(capi.to_np(dw), ref_w))
+        assert max_rel(capi.to_np(db), ref_b.reshape(-1)) < 1e-4, (name, "bias", M, D, nb)
+
+
+@pytest.mark.parametrize("D,nb", [(256, 1), (2560, 10), (512, 16), (512, 8), (512, 4), (768, 3), (384, 3), (96, 3)])
+@pytest.mark.parametrize("M", [1, 33, 1000])
+def test_weight_gradients_block_widths_and_ragged_rows(M, D, nb):
+    _bwd_weights_case(M, D, nb, "bf16", "bf16", seed=M + D)
+
+
+@pytest.mark.parametrize("x_dtype,g_dtype", [("f32", "f32"), ("bf16", "f32"), ("f32", "bf16")])
+def test_weight_gradients_dtype_combinations(x_dtype, g_dtype):
+    _bwd_weights_case(4096 + 17, 2560, 10, x_dtype, g_dtype, seed=9)
+    _bwd_weights_case(300, 512, 16, x_dtype, g_dtype, seed=10)
+
+
+def test_weight_gradients_full_shape_against_the_library_gemm_and_reproducible():
+    M, D, nb = 32768, 2560, 10
+    g = torch.Generator(device="cuda").manual_seed(3)
+    mk = lambda: torch.randn((M, D), generator=g, device="cuda").to(torch.bfloat16)  # noqa: E731
+    x, gi, ga = mk(), mk(), mk()
+    first = capi.gate_proj_bwd_weights(x, gi, ga, nb)
+    second = capi.gate_proj_bwd_weights(x, gi, ga, nb)
+    for a, b in zip(first, second):
+        assert torch.equal(a, b)
+    xb = x.reshape(M, nb, 256).transpose(0, 1).float()
+    for gd, dw, db in ((gi, first[0], first[1]), (ga, first[2], first[3])):
+        ref_w = torch.bmm(xb.transpose(1, 2), gd.reshape(M, nb, 256).transpose(0, 1).float())
+        assert float((dw - ref_w).abs().max() / ref_w.abs().max()) < 1e-4
+        ref_b = gd.double().sum(dim=0)
+        assert float((db.double() - ref_b).abs().max() / ref_b.abs().max()) < 1e-4
