@@ -6,6 +6,7 @@ from .cache import RNNCache
 from .external import (
     BlockDiagonalLinear,
     Conv1D,
+    gate_projections,
     rglru_step,
     rglru_step_gated,
     rnn_param_init,
@@ -35,6 +36,7 @@ __all__ = [
     "RNNCache",
     "RNNLayer",
     "fused_linear_scan",
+    "gate_projections",
     "fused_linear_scan_gated",
     "rglru_step",
     "rglru_step_gated",

@@ -305,3 +305,149 @@ class BlockDiagonalLinear(nn.Module):
         if add_bias:
             yb = yb + self.b
         return yb.reshape(*lead, self.width)
+
+
+# ---------------------------------------------------------------------------------------
+# Both gate projections in one pass (matrix-core kernels): the pair of BlockDiagonalLinear
+# calls of hawk/hawk.py:181-182 and their autograd.
+# ---------------------------------------------------------------------------------------
+_gate_ws: dict = {}
+
+
+def _gate_workspace(dev: torch.device, nbytes: int) -> torch.Tensor:
+    key = (dev.index if dev.index is not None else torch.cuda.current_device(), _lib.stream_ptr(dev))
+    ws = _gate_ws.get(key)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+        _gate_ws[key] = ws
+    return ws
+
+
+def _launch_gate_fwd(x, w_i, b_i, w_a, b_a, out_bf16: bool):
+    dev = _lib.require_cuda(x, w_i, b_i, w_a, b_a)
+    nb, bw, _ = w_i.shape
+    D = nb * bw
+    M = x.numel() // D
+    x2, w_i, w_a, b_i, b_a = (_lib.dense16(t) for t in (x.reshape(M, D), w_i, w_a, b_i, b_a))
+    out_dtype = torch.bfloat16 if out_bf16 else torch.float32
+    xg = torch.empty(x.shape, dtype=out_dtype, device=dev)
+    ag = torch.empty(x.shape, dtype=out_dtype, device=dev)
+    with torch.cuda.device(dev):
+        status = _lib.load().hawk_gate_proj_fwd(
+            x2.data_ptr(), w_i.data_ptr(), b_i.data_ptr(), w_a.data_ptr(), b_a.data_ptr(), xg.data_ptr(),
+            ag.data_ptr(), M, D, nb, _lib.dtype_code(x2.dtype), _lib.dtype_code(w_i.dtype),
+            _lib.dtype_code(out_dtype), _lib.stream_ptr(dev),
+        )
+    _lib.check("hawk_gate_proj_fwd", status)
+    return xg, ag
+
+
+def _launch_gate_bwd(x, d_xg, d_ag, w_i, w_a):
+    dev = _lib.require_cuda(x, d_xg, d_ag, w_i, w_a)
+    nb, bw, _ = w_i.shape
+    D = nb * bw
+    M = x.numel() // D
+    x2, g_i, g_a, w_i, w_a = (_lib.dense16(t) for t in (x.reshape(M, D), d_xg.reshape(M, D), d_ag.reshape(M, D), w_i, w_a))
+    lib = _lib.load()
+    dx = torch.empty(x.shape, dtype=x.dtype, device=dev)
+    dw_i = torch.empty((nb, bw, bw), dtype=torch.float32, device=dev)
+    dw_a = torch.empty_like(dw_i)
+    db_i = torch.empty(D, dtype=torch.float32, device=dev)
+    db_a = torch.empty(D, dtype=torch.float32, device=dev)
+    nbytes = lib.hawk_gate_proj_bwd_weights_workspace_bytes(M, D, nb)
+    ws = _gate_workspace(dev, nbytes)
+    with torch.cuda.device(dev):
+        st = _lib.stream_ptr(dev)
+        status = lib.hawk_gate_proj_bwd_input(
+            g_i.data_ptr(), g_a.data_ptr(), w_i.data_ptr(), w_a.data_ptr(), dx.data_ptr(), M, D, nb,
+            _lib.dtype_code(g_i.dtype), _lib.dtype_code(w_i.dtype), _lib.dtype_code(dx.dtype), st,
+        )
+        _lib.check("hawk_gate_proj_bwd_input", status)
+        status = lib.hawk_gate_proj_bwd_weights(
+            x2.data_ptr(), g_i.data_ptr(), g_a.data_ptr(), dw_i.data_ptr(), db_i.data_ptr(), dw_a.data_ptr(),
+            db_a.data_ptr(), M, D, nb, _lib.dtype_code(x2.dtype), _lib.dtype_code(g_i.dtype), ws.data_ptr(),
+            ws.numel(), st,
+        )
+        _lib.check("hawk_gate_proj_bwd_weights", status)
+    return dx, dw_i, db_i, dw_a, db_a
+
+
+@torch.library.custom_op("hawk_amd::gate_proj_fwd", mutates_args=(), device_types="cuda")
+def _gate_proj_fwd_op(
+    x: torch.Tensor, w_i: torch.Tensor, b_i: torch.Tensor, w_a: torch.Tensor, b_a: torch.Tensor, out_bf16: bool
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    return _launch_gate_fwd(x, w_i, b_i, w_a, b_a, out_bf16)
+
+
+@_gate_proj_fwd_op.register_fake
+def _(x, w_i, b_i, w_a, b_a, out_bf16):
+    dt = torch.bfloat16 if out_bf16 else torch.float32
+    return torch.empty(x.shape, dtype=dt, device=x.device), torch.empty(x.shape, dtype=dt, device=x.device)
+
+
+@torch.library.custom_op("hawk_amd::gate_proj_bwd", mutates_args=(), device_types="cuda")
+def _gate_proj_bwd_op(
+    x: torch.Tensor, d_xg: torch.Tensor, d_ag: torch.Tensor, w_i: torch.Tensor, w_a: torch.Tensor
+) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+    return _launch_gate_bwd(x, d_xg, d_ag, w_i, w_a)
+
+
+@_gate_proj_bwd_op.register_fake
+def _(x, d_xg, d_ag, w_i, w_a):
+    nb, bw, _ = w_i.shape
+    f32 = dict(dtype=torch.float32, device=x.device)
+    return (
+        torch.empty(x.shape, dtype=x.dtype, device=x.device),
+        torch.empty((nb, bw, bw), **f32), torch.empty(nb * bw, **f32),
+        torch.empty((nb, bw, bw), **f32), torch.empty(nb * bw, **f32),
+    )
+
+
+class _GateProjection(Function):
+    """(x_rg_lru, a_rg_lru) = (blockdiag(w_i) x + b_i, blockdiag(w_a) x + b_a), bf16 operands."""
+
+    @staticmethod
+    def forward(ctx, x, w_i, b_i, w_a, b_a, out_bf16: bool):
+        xc = x if x.is_contiguous() else x.contiguous()
+        ctx.save_for_backward(xc, w_i, w_a)
+        ctx.param_dtypes = (w_i.dtype, b_i.dtype, w_a.dtype, b_a.dtype)
+        return _gate_proj_fwd_op(xc, w_i, b_i.float().reshape(-1), w_a, b_a.float().reshape(-1), out_bf16)
+
+    @staticmethod
+    def backward(ctx, d_xg, d_ag):  # type: ignore[override]
+        x, w_i, w_a = ctx.saved_tensors
+        gdt = torch.bfloat16 if (d_xg.dtype == torch.bfloat16 and d_ag.dtype == torch.bfloat16) else torch.float32
+        d_xg, d_ag = (g.to(gdt).contiguous() for g in (d_xg, d_ag))
+        dx, dw_i, db_i, dw_a, db_a = _gate_proj_bwd_op(x, d_xg, d_ag, w_i, w_a)
+        nb, bw, _ = w_i.shape
+        dts = ctx.param_dtypes
+        return (dx, dw_i.to(dts[0]), db_i.reshape(nb, bw).to(dts[1]), dw_a.to(dts[2]),
+                db_a.reshape(nb, bw).to(dts[3]), None)
+
+
+def gate_projections_supported(x: torch.Tensor, gate: "BlockDiagonalLinear") -> bool:
+    """The fused kernels compute with bf16 operands, which is the arithmetic of this einsum
+    under bf16 autocast or on bf16 tensors; plain fp32 calls keep the library GEMM."""
+    if x.device.type != "cuda" or x.dtype not in (torch.bfloat16, torch.float32):
+        return False
+    if gate.w.dtype not in (torch.bfloat16, torch.float32):
+        return False
+    if not (x.dtype == torch.bfloat16 or torch.is_autocast_enabled("cuda")):
+        return False
+    return bool(_lib.load().hawk_gate_proj_supported(gate.width, gate.num_blocks))
+
+
+def gate_projections(x: torch.Tensor, input_gate: "BlockDiagonalLinear", a_gate: "BlockDiagonalLinear",
+                     out_dtype: Optional[torch.dtype] = None) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Both gate logits of hawk/hawk.py:181-182, ``(input_gate(x), a_gate(x))``.
+
+    One kernel reads x once and writes both logits (and one pair of kernels does the whole
+    backward) whenever ``gate_projections_supported``; otherwise the two modules are called
+    as upstream does.  ``out_dtype`` (bf16 or fp32) applies to the fused path and defaults to
+    x's dtype.
+    """
+    if not gate_projections_supported(x, input_gate):
+        return input_gate(x), a_gate(x)
+    assert a_gate.width == input_gate.width and a_gate.num_blocks == input_gate.num_blocks
+    out_bf16 = (out_dtype or x.dtype) == torch.bfloat16
+    return _GateProjection.apply(x, input_gate.w, input_gate.b, a_gate.w, a_gate.b, out_bf16)

@@ -28,7 +28,17 @@ import torch.nn as nn
 import torch.nn.functional as F
 
 from .cache import RNNCache
-from .external import BlockDiagonalLinear, Conv1D, rglru_step, rglru_step_gated, rnn_param_init
+from .external import (
+    BlockDiagonalLinear,
+    Conv1D,
+    gate_projections,
+    gate_projections_supported,
+    rglru_step,
+    rglru_step_gated,
+    rnn_param_init,
+    temporal_conv1d,
+    temporal_conv1d_step,
+)
 from .scan_fused import fused_linear_scan, fused_linear_scan_gated
 
 
@@ -45,6 +55,9 @@ class HawkConfig:
     post_norm: bool = False
     # not an upstream field: apply gelu(y) * h inside the scan kernels (hawk/hawk.py:134-135)
     fused_epilogue: bool = True
+    # not an upstream field: both gate projections in one matrix-core kernel when the arithmetic
+    # is bf16 anyway (bf16 tensors or bf16 autocast); hawk/hawk.py:181-182
+    fused_gates: bool = True
 
     def __post_init__(self):
         if self.post_norm:
@@ -115,31 +128,40 @@ class Hawk(nn.Module):
         if warm:
             # one new token per batch row; only the last position is used, as upstream
             assert layer_past is not None
-            u = self.conv1d.step(layer_past.conv_state, branch[:, -1:, :])
+            fused_gates = self.config.fused_gates and gate_projections_supported(branch, self.rg_lru_input_gate)
             gate_branch = gate_branch[:, -1:, :]
             layer_past.current_cache_size = 1
+            if fused_gates:
+                u = temporal_conv1d_step(layer_past.conv_state, branch[:, -1:, :], self.conv1d.w, self.conv1d.b,
+                                         torch.bfloat16)
+                xg, ag = gate_projections(u, self.rg_lru_input_gate, self.rg_lru_a_gate, torch.bfloat16)
+                bias_i = bias_a = None  # already added by the projection kernel
+            else:
+                u = self.conv1d.step(layer_past.conv_state, branch[:, -1:, :])
+                xg = self.rg_lru_input_gate(u, add_bias=False)
+                ag = self.rg_lru_a_gate(u, add_bias=False)
+                bias_i, bias_a = self.rg_lru_input_gate.b, self.rg_lru_a_gate.b
             if self.config.fused_epilogue:
-                gated = rglru_step_gated(
-                    u,
-                    self.rg_lru_input_gate(u, add_bias=False),
-                    self.rg_lru_a_gate(u, add_bias=False),
-                    self.rg_lru_a_param,
-                    layer_past.recc_state,
-                    gate_branch,
-                    bias_i=self.rg_lru_input_gate.b,
-                    bias_a=self.rg_lru_a_gate.b,
-                )
+                gated = rglru_step_gated(u, xg, ag, self.rg_lru_a_param, layer_past.recc_state, gate_branch,
+                                         bias_i=bias_i, bias_a=bias_a)
                 return self.resid_proj(gated), layer_past
-            h = rglru_step(
-                u, self.rg_lru_input_gate(u), self.rg_lru_a_gate(u), self.rg_lru_a_param, layer_past.recc_state
-            )
+            if bias_i is not None:
+                xg, ag = xg + bias_i.reshape(-1), ag + bias_a.reshape(-1)
+            h = rglru_step(u, xg, ag, self.rg_lru_a_param, layer_past.recc_state)
             cache = layer_past
         else:
             if self.use_cache:
                 assert layer_past is not None, "use_cache=True needs one RNNCache per layer in layer_past"
                 layer_past.seed_conv_state(branch)
-            u = self.conv1d(branch)
-            gates = (self.rg_lru_input_gate(u), self.rg_lru_a_gate(u), self.rg_lru_a_param.float())
+            if self.config.fused_gates and gate_projections_supported(branch, self.rg_lru_input_gate):
+                # bf16 end to end: upstream's gate einsums (under autocast) and its scan
+                # (cast_inputs, hawk/scan_fused.py:428) round the conv output to bf16 anyway
+                u = temporal_conv1d(branch, self.conv1d.w, self.conv1d.b, torch.bfloat16)
+                xg, ag = gate_projections(u, self.rg_lru_input_gate, self.rg_lru_a_gate, torch.bfloat16)
+            else:
+                u = self.conv1d(branch)
+                xg, ag = self.rg_lru_input_gate(u), self.rg_lru_a_gate(u)
+            gates = (xg, ag, self.rg_lru_a_param.float())
             cache = layer_past if self.use_cache else None
             if self.config.fused_epilogue:
                 gated, h_last = fused_linear_scan_gated(u, *gates, gate_branch, return_last_state=True)

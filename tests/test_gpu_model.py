@@ -338,3 +338,54 @@ def test_torch_compile_traces_the_gated_scan_without_graph_breaks():
     fn(x, xg, ag, lam)[0].backward(gout)
     assert torch.allclose(g_compiled, x.grad, atol=1e-5)
     assert torch.allclose(w_compiled, lin.weight.grad, atol=1e-4)
+
+
+@pytest.mark.parametrize("mode", ["bf16", "autocast"])
+def test_gate_projections_autograd_matches_the_two_modules(mode):
+    """Fused projection pair (forward and both backward kernels) against the two
+    BlockDiagonalLinear modules run through the library GEMM on the same operands."""
+    torch.manual_seed(11)
+    D, nb = 512, 4
+    gi = hk.BlockDiagonalLinear(D, nb).cuda()
+    ga = hk.BlockDiagonalLinear(D, nb).cuda()
+    with torch.no_grad():
+        gi.b.normal_()
+        ga.b.normal_()
+    xdt = torch.bfloat16 if mode == "bf16" else torch.float32
+    x = torch.randn(2, 150, D, device="cuda").to(xdt).requires_grad_(True)
+    go_i = torch.randn(2, 150, D, device="cuda").to(torch.bfloat16)
+    go_a = torch.randn(2, 150, D, device="cuda").to(torch.bfloat16)
+
+    def run(fn):
+        for p in (x, gi.w, gi.b, ga.w, ga.b):
+            p.grad = None
+        with torch.autocast(device_type="cuda", dtype=torch.bfloat16, enabled=(mode == "autocast")):
+            a, b = fn()
+        (a.float() * go_i.float()).sum().backward(retain_graph=True)
+        (b.float() * go_a.float()).sum().backward()
+        return (a.detach().float(), b.detach().float(),
+                *(p.grad.detach().float().clone() for p in (x, gi.w, gi.b, ga.w, ga.b)))
+
+    from hawk_pytorch_amd.external import gate_projections_supported
+    with torch.autocast(device_type="cuda", dtype=torch.bfloat16, enabled=(mode == "autocast")):
+        assert gate_projections_supported(x, gi)
+    got = run(lambda: hk.gate_projections(x, gi, ga, torch.bfloat16))
+    if mode == "bf16":
+        gi_ref, ga_ref = gi.bfloat16(), ga.bfloat16()  # library path needs matching dtypes
+        want = run(lambda: (gi_ref(x), ga_ref(x)))
+    else:
+        want = run(lambda: (gi(x), ga(x)))
+    names = ("x_rg_lru", "a_rg_lru", "dx", "dw_i", "db_i", "dw_a", "db_a")
+    for name, a, b in zip(names, got, want):
+        assert a.shape == b.shape, name
+        assert max_rel(capi.to_np(a), capi.to_np(b)) < TOL["bf16"], (name, max_rel(capi.to_np(a), capi.to_np(b)))
+
+
+def test_gate_projections_keep_the_library_gemm_for_plain_fp32():
+    from hawk_pytorch_amd.external import gate_projections_supported
+    gi = hk.BlockDiagonalLinear(256, 2).cuda()
+    ga = hk.BlockDiagonalLinear(256, 2).cuda()
+    x = torch.randn(3, 5, 256, device="cuda")
+    assert not gate_projections_supported(x, gi)
+    a, b = hk.gate_projections(x, gi, ga)
+    assert torch.equal(a, gi(x)) and torch.equal(b, ga(x))
