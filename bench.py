@@ -10,6 +10,8 @@ the 70 %-of-HBM-peak target is quoted on).  ``--workload long`` runs B=2, T=3276
 D=4096; ``--workload scan_conv`` adds the temporal conv1d forward and backward;
 ``--workload scan_gated`` runs the scan fused with the block's gate (out = gelu(y) * h,
 y being one half of a [B, T, 2D] projection), 12 + 20 bytes per element;
+``--workload gates`` runs the fused block-diagonal gate projections (matrix-core kernels:
+forward, input gradient, weight gradients) on 32768 tokens, D = 2560, 10 blocks, bf16;
 ``--workload decode`` times one-token steps of a 26-layer Hawk (R = H = 2560, I = 7680,
 10 gate blocks, vocabulary 32000, bf16 weights) at batch 256 after a 1024-token prefill,
 eagerly and as a replayed HIP graph, plus the two hot-path kernels of a layer on their own.
@@ -87,6 +89,88 @@ def cpu_baseline(B, D, lo, hi, seed, budget_rows=512):
         "sample": f"first {T} of the time rows at B={B}, D={D}, fp32, forward + autograd backward, "
                   f"{dt:.2f} s, host has {os.cpu_count()} logical cpus",
     }
+
+
+def run_gates(args, lib, dev):
+    """Both gate projections of a layer on B*T = 32768 tokens: forward, dx, dw/db."""
+    from hawk_pytorch_amd import _lib
+
+    M, D, nb = 8 * 4096, 2560, 10
+    bw = D // nb
+    bf, code, f32 = torch.bfloat16, _lib.HAWK_DTYPE_BF16, _lib.HAWK_DTYPE_F32
+    gen = torch.Generator(device=dev).manual_seed(args.seed)
+    x, gi, ga = (torch.randn(M, D, device=dev, generator=gen).to(bf) for _ in range(3))
+    wi, wa = (torch.randn(nb, bw, bw, device=dev, generator=gen) / bw ** 0.5 for _ in range(2))
+    bi, ba = (torch.randn(D, device=dev, generator=gen) for _ in range(2))
+    oi, oa, dx = torch.empty_like(x), torch.empty_like(x), torch.empty_like(x)
+    dwi, dwa = torch.empty_like(wi), torch.empty_like(wa)
+    dbi, dba = torch.empty_like(bi), torch.empty_like(ba)
+    nws = lib.hawk_gate_proj_bwd_weights_workspace_bytes(M, D, nb)
+    ws = torch.empty(nws, dtype=torch.uint8, device=dev)
+    stream = torch.cuda.current_stream(dev).cuda_stream
+
+    def fwd():
+        _lib.check("gate_proj_fwd", lib.hawk_gate_proj_fwd(
+            x.data_ptr(), wi.data_ptr(), bi.data_ptr(), wa.data_ptr(), ba.data_ptr(), oi.data_ptr(), oa.data_ptr(),
+            M, D, nb, code, f32, code, stream))
+
+    def bwd_input():
+        _lib.check("gate_proj_bwd_input", lib.hawk_gate_proj_bwd_input(
+            gi.data_ptr(), ga.data_ptr(), wi.data_ptr(), wa.data_ptr(), dx.data_ptr(), M, D, nb, code, f32, code,
+            stream))
+
+    def bwd_weights():
+        _lib.check("gate_proj_bwd_weights", lib.hawk_gate_proj_bwd_weights(
+            x.data_ptr(), gi.data_ptr(), ga.data_ptr(), dwi.data_ptr(), dbi.data_ptr(), dwa.data_ptr(),
+            dba.data_ptr(), M, D, nb, code, code, ws.data_ptr(), nws, stream))
+
+    if args.calibration_copy:
+        for _ in range(3):
+            oi.copy_(x)
+        torch.cuda.synchronize()
+    for _ in range(args.warmup):
+        fwd(), bwd_input(), bwd_weights()
+    torch.cuda.synchronize()
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(args.steps)]
+    t0 = time.perf_counter()
+    for k in range(args.steps):
+        ev[k][0].record()
+        fwd()
+        ev[k][1].record()
+        bwd_input()
+        ev[k][2].record()
+        bwd_weights()
+        ev[k][3].record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms = [float(np.mean([e[i].elapsed_time(e[i + 1]) for e in ev])) for i in range(3)]
+    ms_per_step = wall * 1e3 / args.steps
+    N = M * D
+    # forward: read x, write two logits; dx: read two gradients, write dx; dw: read x and two gradients
+    alg = [3 * 2 * N, 3 * 2 * N, 3 * 2 * N]
+    flops = [4.0 * N * bw] * 3
+    gbs = [alg[i] / (ms[i] * 1e-3) / 1e9 for i in range(3)]
+    out = {
+        "metric": "fused gate projections fwd+bwd tokens/s, 1 GPU",
+        "value": M / (ms_per_step * 1e-3),
+        "unit": "tokens/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16 operands, f32 accumulation",
+        "data": f"synthetic, seed {args.seed}: activations and gradients ~ N(0,1), weights ~ N(0, 1/bw)",
+        "config": {"workload": f"gates: both block-diagonal gate projections fwd + input grad + weight grads, "
+                               f"M={M}, D={D}, {nb} blocks of {bw}, bf16", "M": M, "D": D, "num_blocks": nb},
+        "roofline": {
+            "bound": "hbm",
+            "kernel": "gate_proj_bwd_weights_kernel (+ gate_proj_reduce_kernel, same launch call)",
+            "achieved": gbs[2], "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs[2] / HBM_PEAK_GBS,
+            "traffic": None, "algorithmic_bytes_per_launch": alg[2], "launch_ms": ms[2],
+        },
+        "kernels": {name: {"ms": ms[i], "GBs": gbs[i], "frac": gbs[i] / HBM_PEAK_GBS,
+                           "TFLOPs": flops[i] / (ms[i] * 1e-3) / 1e12}
+                    for i, name in enumerate(("fwd", "bwd_input", "bwd_weights"))},
+    }
+    print(json.dumps(out))
 
 
 def run_decode(args, lib, dev):
@@ -227,7 +311,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", choices=sorted(WORKLOADS) + ["decode"], default="scan")
+    ap.add_argument("--workload", choices=sorted(WORKLOADS) + ["decode", "gates"], default="scan")
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calibration-copy", action="store_true",
@@ -251,6 +335,9 @@ def main():
     torch.cuda.set_device(dev)
     if args.workload == "decode":
         run_decode(args, lib, dev)
+        return
+    if args.workload == "gates":
+        run_gates(args, lib, dev)
         return
     B, T, D, (lo, hi), with_conv = WORKLOADS[args.workload]
     N = B * T * D

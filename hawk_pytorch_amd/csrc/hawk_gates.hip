@@ -32,6 +32,7 @@ namespace hawk {
 namespace {
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef bf16x8 bf16x8_t;
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 constexpr int kGroup = 256;                    // channels per workgroup
@@ -43,6 +44,33 @@ constexpr int kNumCU = 256;
 
 __device__ __forceinline__ float elem_to_f32(float v) { return v; }
 __device__ __forceinline__ float elem_to_f32(bf16_t v) { return __uint_as_float((uint32_t)v.bits << 16); }
+
+// Weight fetches go through a buffer resource (scalar base, one per-lane offset, scalar
+// per-access offset), with the default cache policy: every workgroup re-reads them.
+__device__ __forceinline__ float load_weight(rsrc_t r, uint32_t lane_bytes, uint32_t off_bytes, const float*) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, lane_bytes, off_bytes, kAuxDefault));
+}
+__device__ __forceinline__ float load_weight(rsrc_t r, uint32_t lane_bytes, uint32_t off_bytes, const bf16_t*) {
+    const uint16_t b = __builtin_bit_cast(uint16_t, __builtin_amdgcn_raw_buffer_load_b16(r, lane_bytes, off_bytes, kAuxDefault));
+    return __uint_as_float((uint32_t)b << 16);
+}
+// eight consecutive weights as a bf16 MFMA operand (scaled by `live`, 0 or 1)
+__device__ __forceinline__ bf16x8_t load_weight8(rsrc_t r, uint32_t lane_bytes, uint32_t off_bytes, float live,
+                                                 const float*) {
+    const u32x4 a = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(r, lane_bytes, off_bytes, kAuxDefault));
+    const u32x4 b = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(r, lane_bytes, off_bytes + 16, kAuxDefault));
+    const u32x4 packed = {pack_bf16x2(live * __uint_as_float(a.x), live * __uint_as_float(a.y)),
+                          pack_bf16x2(live * __uint_as_float(a.z), live * __uint_as_float(a.w)),
+                          pack_bf16x2(live * __uint_as_float(b.x), live * __uint_as_float(b.y)),
+                          pack_bf16x2(live * __uint_as_float(b.z), live * __uint_as_float(b.w))};
+    return __builtin_bit_cast(bf16x8_t, packed);
+}
+__device__ __forceinline__ bf16x8_t load_weight8(rsrc_t r, uint32_t lane_bytes, uint32_t off_bytes, float live,
+                                                 const bf16_t*) {
+    u32x4 a = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(r, lane_bytes, off_bytes, kAuxDefault));
+    if (live == 0.0f) a = u32x4{0u, 0u, 0u, 0u};
+    return __builtin_bit_cast(bf16x8_t, a);
+}
 
 // Eight consecutive activations as they sit in registers between the global load and the LDS store.
 template <typename XT>
@@ -131,7 +159,8 @@ __global__ __launch_bounds__(kGateThreads, 1) void gate_proj_fwd_kernel(
     //      destination; a group past the last block (D not a multiple of 256) reads block
     //      nb-1 and zeroes it
     const float live = (h < nb) ? 1.0f : 0.0f;
-    const WT* wblk = wsel + ((size_t)min(h, nb - 1) * BW + khalf) * BW + n;
+    const rsrc_t wres = make_rsrc(wsel, (uint32_t)((size_t)nb * BW * BW * sizeof(WT)));
+    const uint32_t wlane = (uint32_t)((((size_t)min(h, nb - 1) * BW + khalf) * BW + n) * sizeof(WT));
     bf16x8 bfrag[KS];
     constexpr int kWBatch = KS < 4 ? KS : 4;
 #pragma unroll
@@ -140,7 +169,9 @@ __global__ __launch_bounds__(kGateThreads, 1) void gate_proj_fwd_kernel(
 #pragma unroll
         for (int j = 0; j < kWBatch; ++j)
 #pragma unroll
-            for (int e = 0; e < 8; ++e) v[j][e] = elem_to_f32(wblk[(size_t)(16 * (s0 + j) + e) * BW]);
+            for (int e = 0; e < 8; ++e)
+                v[j][e] = load_weight(wres, wlane, (uint32_t)((16 * (s0 + j) + e) * BW * sizeof(WT)),
+                                      static_cast<const WT*>(nullptr));
 #pragma unroll
         for (int j = 0; j < kWBatch; ++j) {
             const u32x4 packed = {pack_bf16x2(live * v[j][0], live * v[j][1]), pack_bf16x2(live * v[j][2], live * v[j][3]),
@@ -261,23 +292,13 @@ __global__ __launch_bounds__(kGateThreads, 1) void gate_proj_bwd_input_kernel(
 
     // weights: lane holds row i of w_g[h] and 8 consecutive j per k-step (contiguous)
     const float live = (h < nb) ? 1.0f : 0.0f;
-    const WT* wrow = wsel + ((size_t)min(h, nb - 1) * BW + i_in) * BW + khalf;
+    const rsrc_t wres = make_rsrc(wsel, (uint32_t)((size_t)nb * BW * BW * sizeof(WT)));
+    const uint32_t wlane = (uint32_t)((((size_t)min(h, nb - 1) * BW + i_in) * BW + khalf) * sizeof(WT));
     bf16x8 bfrag[KS];
-    constexpr int kWBatch = KS < 4 ? KS : 4;
 #pragma unroll
-    for (int s0 = 0; s0 < KS; s0 += kWBatch) {
-        float v[kWBatch][8];
-#pragma unroll
-        for (int j = 0; j < kWBatch; ++j)
-#pragma unroll
-            for (int e = 0; e < 8; ++e) v[j][e] = elem_to_f32(wrow[16 * (s0 + j) + e]);
-#pragma unroll
-        for (int j = 0; j < kWBatch; ++j) {
-            const u32x4 packed = {pack_bf16x2(live * v[j][0], live * v[j][1]), pack_bf16x2(live * v[j][2], live * v[j][3]),
-                                  pack_bf16x2(live * v[j][4], live * v[j][5]), pack_bf16x2(live * v[j][6], live * v[j][7])};
-            bfrag[s0 + j] = __builtin_bit_cast(bf16x8, packed);
-        }
-        __builtin_amdgcn_sched_barrier(0);
+    for (int s = 0; s < KS; ++s) {
+        bfrag[s] = load_weight8(wres, wlane, (uint32_t)(16 * s * sizeof(WT)), live, static_cast<const WT*>(nullptr));
+        if (s % 4 == 3) __builtin_amdgcn_sched_barrier(0);
     }
 
     stage_tile(0, ra0, ra1);
