@@ -312,6 +312,7 @@ class BlockDiagonalLinear(nn.Module):
 # calls of hawk/hawk.py:181-182 and their autograd.
 # ---------------------------------------------------------------------------------------
 _gate_ws: dict = {}
+_GATE_BLOCK_WIDTHS = (32, 64, 128, 256)
 
 
 def _gate_workspace(dev: torch.device, nbytes: int) -> torch.Tensor:
@@ -434,7 +435,8 @@ def gate_projections_supported(x: torch.Tensor, gate: "BlockDiagonalLinear") -> 
         return False
     if not (x.dtype == torch.bfloat16 or torch.is_autocast_enabled("cuda")):
         return False
-    return bool(_lib.load().hawk_gate_proj_supported(gate.width, gate.num_blocks))
+    # same rule as hawk_gate_proj_supported(), restated so that a tracing compiler sees plain Python
+    return gate.width % gate.num_blocks == 0 and gate.block_width in _GATE_BLOCK_WIDTHS
 
 
 def gate_projections(x: torch.Tensor, input_gate: "BlockDiagonalLinear", a_gate: "BlockDiagonalLinear",

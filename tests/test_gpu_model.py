@@ -389,3 +389,27 @@ def test_gate_projections_keep_the_library_gemm_for_plain_fp32():
     assert not gate_projections_supported(x, gi)
     a, b = hk.gate_projections(x, gi, ga)
     assert torch.equal(a, gi(x)) and torch.equal(b, ga(x))
+
+
+def test_torch_compile_traces_the_whole_model_under_autocast():
+    """Forward and backward of a small HawkModel (fused gates, fused epilogue) as one graph."""
+    torch.manual_seed(4)
+    cfg = _small_config()
+    model = hk.HawkModel(cfg).cuda()
+    _randomise_zero_inits(model)
+    ids = torch.randint(1, cfg.vocab_size, (2, 64), device="cuda")
+
+    def loss_fn(ids):
+        with torch.autocast(device_type="cuda", dtype=torch.bfloat16):
+            return model(ids, ids)
+
+    eager = loss_fn(ids)
+    eager.backward()
+    want = {n: p.grad.detach().clone() for n, p in model.named_parameters()}
+    model.zero_grad()
+    compiled = torch.compile(loss_fn, backend="aot_eager", fullgraph=True)
+    got = compiled(ids)
+    got.backward()
+    assert abs(got.item() - eager.item()) < 1e-3
+    for n, p in model.named_parameters():
+        assert max_rel(capi.to_np(p.grad), capi.to_np(want[n])) < 1e-2, n

@@ -183,3 +183,13 @@ def test_custom_ops_have_shape_rules_for_tracing():
         assert y.dtype == torch.float32 and y.shape == x.shape
         gx, gw, gb = torch.ops.hawk_amd.conv1d_bwd(y, x, w)
         assert gx.dtype == torch.bfloat16 and gw.shape == (4, 64) and gb.shape == (64,)
+
+
+def test_python_rule_for_fused_gate_projections_matches_the_library():
+    from hawk_pytorch_amd import _lib
+    from hawk_pytorch_amd.external import _GATE_BLOCK_WIDTHS
+
+    lib = _lib.load()
+    for D, nb in [(2560, 10), (512, 16), (512, 8), (512, 4), (512, 2), (512, 1), (96, 3), (100, 3), (4096, 16), (48, 3)]:
+        python_rule = D % nb == 0 and (D // nb) in _GATE_BLOCK_WIDTHS
+        assert bool(lib.hawk_gate_proj_supported(D, nb)) == python_rule, (D, nb)
