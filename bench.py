@@ -12,6 +12,9 @@ D=4096; ``--workload scan_conv`` adds the temporal conv1d forward and backward;
 y being one half of a [B, T, 2D] projection), 12 + 20 bytes per element;
 ``--workload gates`` runs the fused block-diagonal gate projections (matrix-core kernels:
 forward, input gradient, weight gradients) on 32768 tokens, D = 2560, 10 blocks, bf16;
+``--workload model`` runs full training steps (forward, backward, AdamW) of the upstream
+README model (vocabulary 32000, hidden = recurrent = 512, MLP 1024, 8 layers, 16 gate blocks)
+on a 1 x 2048 batch under bf16 autocast, with and without the fused gate / epilogue kernels;
 ``--workload decode`` times one-token steps of a 26-layer Hawk (R = H = 2560, I = 7680,
 10 gate blocks, vocabulary 32000, bf16 weights) at batch 256 after a 1024-token prefill,
 eagerly and as a replayed HIP graph, plus the two hot-path kernels of a layer on their own.
@@ -173,6 +176,55 @@ def run_gates(args, lib, dev):
     print(json.dumps(out))
 
 
+def run_model(args, lib, dev):
+    """Training steps of the README model at batch 1 x 2048, bf16 autocast."""
+    import hawk_pytorch_amd as hk
+
+    B, T, vocab = 1, 2048, 32000
+    gen = torch.Generator(device=dev).manual_seed(args.seed)
+    ids = torch.randint(1, vocab, (B, T), device=dev, generator=gen)
+
+    def time_steps(**flags):
+        torch.manual_seed(args.seed)
+        cfg = hk.HawkConfig(vocab_size=vocab, hidden_size=512, intermediate_size=1024, num_hidden_layers=8,
+                            recurrent_size=512, num_blocks=16, conv_width=4, **flags)
+        with torch.device(dev):
+            model = hk.HawkModel(cfg)
+        opt = torch.optim.AdamW(model.parameters(), lr=1e-4)
+
+        def step():
+            with torch.autocast(device_type="cuda", dtype=torch.bfloat16):
+                loss = model(ids, ids)
+            loss.backward()
+            opt.step()
+            opt.zero_grad(set_to_none=True)
+            return loss
+
+        for _ in range(args.warmup):
+            step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            loss = step()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) * 1e3 / args.steps, float(loss.detach())
+
+    fused_ms, fused_loss = time_steps()
+    plain_ms, plain_loss = time_steps(fused_gates=False, fused_epilogue=False)
+    print(json.dumps({
+        "metric": "Hawk training step tokens/s (README model, batch 1 x 2048, bf16 autocast), 1 GPU",
+        "value": B * T / (fused_ms * 1e-3), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": fused_ms, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16 autocast, f32 parameters and recurrence arithmetic",
+        "data": f"synthetic, seed {args.seed}: random-init weights, token ids uniform in [1, {vocab})",
+        "config": {"workload": "model: README Hawk (V=32000, H=R=512, I=1024, L=8, 16 blocks, conv 4), "
+                               "forward + backward + AdamW, eager launches", "B": B, "T": T},
+        "ms_per_step_without_fused_gates_and_epilogue": plain_ms,
+        "loss_after_last_step": {"fused": fused_loss, "unfused": plain_loss},
+        "roofline": None,
+    }))
+
+
 def run_decode(args, lib, dev):
     """Decode at batch 256: tokens/s of whole model steps, and the hot path's share of a layer."""
     import hawk_pytorch_amd as hk
@@ -311,7 +363,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", choices=sorted(WORKLOADS) + ["decode", "gates"], default="scan")
+    ap.add_argument("--workload", choices=sorted(WORKLOADS) + ["decode", "gates", "model"], default="scan")
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calibration-copy", action="store_true",
@@ -338,6 +390,9 @@ def main():
         return
     if args.workload == "gates":
         run_gates(args, lib, dev)
+        return
+    if args.workload == "model":
+        run_model(args, lib, dev)
         return
     B, T, D, (lo, hi), with_conv = WORKLOADS[args.workload]
     N = B * T * D
