@@ -119,7 +119,7 @@ def run_gates(args, lib, dev):
 
     def bwd_input():
         _lib.check("gate_proj_bwd_input", lib.hawk_gate_proj_bwd_input(
-            gi.data_ptr(), ga.data_ptr(), wi.data_ptr(), wa.data_ptr(), dx.data_ptr(), M, D, nb, code, f32, code,
+            gi.data_ptr(), ga.data_ptr(), wi.data_ptr(), wa.data_ptr(), None, dx.data_ptr(), M, D, nb, code, f32, code,
             stream))
 
     def bwd_weights():

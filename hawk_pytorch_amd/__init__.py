@@ -19,6 +19,7 @@ from .scan_fused import (
     GatedDiagonalRecurrence,
     fused_linear_scan,
     fused_linear_scan_gated,
+    recurrent_core,
     sequential_scan_backward,
     sequential_scan_forward,
 )
@@ -37,6 +38,7 @@ __all__ = [
     "RNNLayer",
     "fused_linear_scan",
     "gate_projections",
+    "recurrent_core",
     "fused_linear_scan_gated",
     "rglru_step",
     "rglru_step_gated",

@@ -58,7 +58,7 @@ SIGNATURES = {
     "hawk_rglru_step": (_c_int, [_c_void_p] * 6 + [_c_int] * 4 + [_c_void_p]),
     "hawk_gate_proj_supported": (_c_int, [_c_int, _c_int]),
     "hawk_gate_proj_fwd": (_c_int, [_c_void_p] * 7 + [_c_int] * 6 + [_c_void_p]),
-    "hawk_gate_proj_bwd_input": (_c_int, [_c_void_p] * 5 + [_c_int] * 6 + [_c_void_p]),
+    "hawk_gate_proj_bwd_input": (_c_int, [_c_void_p] * 6 + [_c_int] * 6 + [_c_void_p]),
     "hawk_gate_proj_bwd_weights_workspace_bytes": (_c_size_t, [_c_int] * 3),
     "hawk_gate_proj_bwd_weights": (_c_int, [_c_void_p] * 7 + [_c_int] * 5 + [_c_void_p, _c_size_t, _c_void_p]),
     "hawk_rglru_step_gated": (

@@ -227,14 +227,15 @@ int hawk_gate_proj_fwd(const void* x, const void* w_i, const float* b_i, const v
 }
 
 int hawk_gate_proj_bwd_input(const void* d_x_rg_lru, const void* d_a_rg_lru, const void* w_i, const void* w_a,
-                             void* dx, int M, int D, int num_blocks, int g_dtype, int w_dtype, int dx_dtype,
-                             void* stream) {
+                             const void* addend, void* dx, int M, int D, int num_blocks, int g_dtype, int w_dtype,
+                             int dx_dtype, void* stream) {
     if (!d_x_rg_lru || !d_a_rg_lru || !w_i || !w_a || !dx) return HAWK_ERR_NULL_POINTER;
     if (!dtype_ok(g_dtype) || !dtype_ok(w_dtype) || !dtype_ok(dx_dtype)) return HAWK_ERR_BAD_DTYPE;
     if (M < 1 || !hawk_gate_proj_supported(D, num_blocks)) return HAWK_ERR_BAD_SHAPE;
-    if (!aligned16(d_x_rg_lru) || !aligned16(d_a_rg_lru) || !aligned16(dx) || !aligned16(w_i) || !aligned16(w_a))
+    if (!aligned16(d_x_rg_lru) || !aligned16(d_a_rg_lru) || !aligned16(dx) || !aligned16(w_i) || !aligned16(w_a) ||
+        (addend && !aligned16(addend)))
         return HAWK_ERR_ALIGNMENT;
-    return hawk::gate_proj_bwd_input(d_x_rg_lru, d_a_rg_lru, w_i, w_a, dx, M, D, num_blocks, g_dtype, w_dtype,
+    return hawk::gate_proj_bwd_input(d_x_rg_lru, d_a_rg_lru, w_i, w_a, addend, dx, M, D, num_blocks, g_dtype, w_dtype,
                                      dx_dtype, as_stream(stream));
 }
 

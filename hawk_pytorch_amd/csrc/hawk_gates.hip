@@ -82,6 +82,10 @@ struct Row8<bf16_t> {
         v = ok ? *reinterpret_cast<const u32x4*>(p) : u32x4{0u, 0u, 0u, 0u};
     }
     __device__ __forceinline__ u32x4 as_bf16() const { return v; }
+    __device__ __forceinline__ void as_f32(f32x4& a, f32x4& b) const {
+        a = f32x4{bf16_lo(v.x), bf16_hi(v.x), bf16_lo(v.y), bf16_hi(v.y)};
+        b = f32x4{bf16_lo(v.z), bf16_hi(v.z), bf16_lo(v.w), bf16_hi(v.w)};
+    }
 };
 template <>
 struct Row8<float> {
@@ -94,6 +98,10 @@ struct Row8<float> {
     __device__ __forceinline__ u32x4 as_bf16() const {
         return u32x4{pack_bf16x2(lo.x, lo.y), pack_bf16x2(lo.z, lo.w), pack_bf16x2(hi.x, hi.y),
                      pack_bf16x2(hi.z, hi.w)};
+    }
+    __device__ __forceinline__ void as_f32(f32x4& a, f32x4& b) const {
+        a = lo;
+        b = hi;
     }
 };
 
@@ -241,6 +249,7 @@ __global__ __launch_bounds__(kGateThreads, 1) void gate_proj_fwd_kernel(
 // ---------------------------------------------------------------------------------------
 // Input gradient of the two projections:
 //   dx[m, h*bw + i] = sum_j dxg[m, h*bw + j] w_i[h, i, j] + sum_j dag[m, h*bw + j] w_a[h, i, j]
+//                     (+ addend[m, h*bw + i], the gradient x receives from its other consumers)
 // Same decomposition as the forward: wave (g, c) keeps w_g[h, 32c.., :] (rows of the weight
 // matrix, contiguous in memory) as B operands, reads gate g's gradient tile from LDS as A
 // operands, and the two gates' partial tiles are added on the way out.
@@ -248,7 +257,7 @@ __global__ __launch_bounds__(kGateThreads, 1) void gate_proj_fwd_kernel(
 template <typename GT, typename WT, typename DT, int BW>
 __global__ __launch_bounds__(kGateThreads, 1) void gate_proj_bwd_input_kernel(
     const GT* __restrict__ dxg, const GT* __restrict__ dag, const WT* __restrict__ w_i, const WT* __restrict__ w_a,
-    DT* __restrict__ dx, int M, int D, int nb, int ntiles) {
+    const DT* __restrict__ addend, DT* __restrict__ dx, int M, int D, int nb, int ntiles) {
     constexpr int KS = BW / 16;
     constexpr int G = kGroup / BW;
     constexpr int kORowBytes = kGroup * 4 + 16;             // fp32 partial sums of one gate, one row
@@ -310,6 +319,11 @@ __global__ __launch_bounds__(kGateThreads, 1) void gate_proj_bwd_input_kernel(
     const unsigned char* o_src = sO + lrow * kORowBytes + lc8 * 32;
 
     auto step = [&](int it, int cur, Row8<GT>& rn0, Row8<GT>& rn1) {
+        // the addend's piece of this tile is asked for now and used after the tile's arithmetic
+        const int row = (worker + it * nworkers) * kTileRows + lrow;
+        const bool out_ok = col_ok && row < M;
+        Row8<DT> radd;
+        radd.load(addend + (out_ok && addend != nullptr ? (size_t)row * D + lcol : 0), out_ok && addend != nullptr);
         f32x16 acc = {};
         const unsigned char* a_base = sA + (2 * cur) * kATileBytes + a_off;
         constexpr int kBatch = KS < 4 ? KS : 4;
@@ -331,12 +345,13 @@ __global__ __launch_bounds__(kGateThreads, 1) void gate_proj_bwd_input_kernel(
         stage_tile(cur ^ 1, rn0, rn1);
         load_tile(it + 3, rn0, rn1);
         __syncthreads();
-        const int row = (worker + it * nworkers) * kTileRows + lrow;
-        if (col_ok && row < M) {
+        if (out_ok) {
             const f32x4 p0 = *reinterpret_cast<const f32x4*>(o_src), p1 = *reinterpret_cast<const f32x4*>(o_src + 16);
             const f32x4 q0 = *reinterpret_cast<const f32x4*>(o_src + kOTileBytes);
             const f32x4 q1 = *reinterpret_cast<const f32x4*>(o_src + kOTileBytes + 16);
-            const f32x4 s0 = p0 + q0, s1 = p1 + q1;
+            f32x4 e0, e1;
+            radd.as_f32(e0, e1);
+            const f32x4 s0 = (p0 + q0) + e0, s1 = (p1 + q1) + e1;
             DT* dst = dx + (size_t)row * D + lcol;
             if constexpr (sizeof(DT) == 4) {
                 __builtin_nontemporal_store(s0, reinterpret_cast<f32x4*>(dst));
@@ -602,8 +617,8 @@ int gate_fwd_out(const void* x, const void* w_i, const float* b_i, const void* w
 }
 
 template <typename GT, typename WT, typename DT, int BW>
-int launch_gate_bwd_input(const void* dxg, const void* dag, const void* w_i, const void* w_a, void* dx, int M, int D,
-                          int nb, hipStream_t st) {
+int launch_gate_bwd_input(const void* dxg, const void* dag, const void* w_i, const void* w_a, const void* addend,
+                          void* dx, int M, int D, int nb, hipStream_t st) {
     const int ngroups = ceil_div(D, kGroup);
     const int ntiles = ceil_div(M, kTileRows);
     int nworkers = kNumCU / ngroups;
@@ -616,28 +631,29 @@ int launch_gate_bwd_input(const void* dxg, const void* dag, const void* w_i, con
         return HAWK_ERR_LAUNCH;
     hipLaunchKernelGGL(kernel, dim3((unsigned)nworkers, (unsigned)ngroups), dim3(kGateThreads), smem, st,
                        static_cast<const GT*>(dxg), static_cast<const GT*>(dag), static_cast<const WT*>(w_i),
-                       static_cast<const WT*>(w_a), static_cast<DT*>(dx), M, D, nb, ntiles);
+                       static_cast<const WT*>(w_a), static_cast<const DT*>(addend), static_cast<DT*>(dx), M, D, nb,
+                       ntiles);
     return hipGetLastError() == hipSuccess ? HAWK_OK : HAWK_ERR_LAUNCH;
 }
 
 template <typename GT, typename WT, typename DT>
-int gate_bwd_input_bw(const void* dxg, const void* dag, const void* w_i, const void* w_a, void* dx, int M, int D,
-                      int nb, int bw, hipStream_t st) {
+int gate_bwd_input_bw(const void* dxg, const void* dag, const void* w_i, const void* w_a, const void* addend,
+                      void* dx, int M, int D, int nb, int bw, hipStream_t st) {
     switch (bw) {
-        case 32: return launch_gate_bwd_input<GT, WT, DT, 32>(dxg, dag, w_i, w_a, dx, M, D, nb, st);
-        case 64: return launch_gate_bwd_input<GT, WT, DT, 64>(dxg, dag, w_i, w_a, dx, M, D, nb, st);
-        case 128: return launch_gate_bwd_input<GT, WT, DT, 128>(dxg, dag, w_i, w_a, dx, M, D, nb, st);
-        case 256: return launch_gate_bwd_input<GT, WT, DT, 256>(dxg, dag, w_i, w_a, dx, M, D, nb, st);
+        case 32: return launch_gate_bwd_input<GT, WT, DT, 32>(dxg, dag, w_i, w_a, addend, dx, M, D, nb, st);
+        case 64: return launch_gate_bwd_input<GT, WT, DT, 64>(dxg, dag, w_i, w_a, addend, dx, M, D, nb, st);
+        case 128: return launch_gate_bwd_input<GT, WT, DT, 128>(dxg, dag, w_i, w_a, addend, dx, M, D, nb, st);
+        case 256: return launch_gate_bwd_input<GT, WT, DT, 256>(dxg, dag, w_i, w_a, addend, dx, M, D, nb, st);
         default: return HAWK_ERR_BAD_SHAPE;
     }
 }
 
 template <typename GT, typename WT>
-int gate_bwd_input_out(const void* dxg, const void* dag, const void* w_i, const void* w_a, void* dx, int M, int D,
-                       int nb, int bw, int dx_dtype, hipStream_t st) {
+int gate_bwd_input_out(const void* dxg, const void* dag, const void* w_i, const void* w_a, const void* addend,
+                       void* dx, int M, int D, int nb, int bw, int dx_dtype, hipStream_t st) {
     if (dx_dtype == HAWK_DTYPE_BF16)
-        return gate_bwd_input_bw<GT, WT, bf16_t>(dxg, dag, w_i, w_a, dx, M, D, nb, bw, st);
-    return gate_bwd_input_bw<GT, WT, float>(dxg, dag, w_i, w_a, dx, M, D, nb, bw, st);
+        return gate_bwd_input_bw<GT, WT, bf16_t>(dxg, dag, w_i, w_a, addend, dx, M, D, nb, bw, st);
+    return gate_bwd_input_bw<GT, WT, float>(dxg, dag, w_i, w_a, addend, dx, M, D, nb, bw, st);
 }
 
 int weight_splits(int M, int D) {
@@ -688,17 +704,17 @@ int gate_proj_fwd(const void* x, const void* w_i, const float* b_i, const void* 
     return gate_fwd_out<float, float>(x, w_i, b_i, w_a, b_a, out_i, out_a, M, D, nb, bw, out_dtype, st);
 }
 
-int gate_proj_bwd_input(const void* dxg, const void* dag, const void* w_i, const void* w_a, void* dx, int M, int D,
-                        int nb, int g_dtype, int w_dtype, int dx_dtype, hipStream_t st) {
+int gate_proj_bwd_input(const void* dxg, const void* dag, const void* w_i, const void* w_a, const void* addend,
+                        void* dx, int M, int D, int nb, int g_dtype, int w_dtype, int dx_dtype, hipStream_t st) {
     const int bw = D / nb;
     if (g_dtype == HAWK_DTYPE_BF16) {
         if (w_dtype == HAWK_DTYPE_BF16)
-            return gate_bwd_input_out<bf16_t, bf16_t>(dxg, dag, w_i, w_a, dx, M, D, nb, bw, dx_dtype, st);
-        return gate_bwd_input_out<bf16_t, float>(dxg, dag, w_i, w_a, dx, M, D, nb, bw, dx_dtype, st);
+            return gate_bwd_input_out<bf16_t, bf16_t>(dxg, dag, w_i, w_a, addend, dx, M, D, nb, bw, dx_dtype, st);
+        return gate_bwd_input_out<bf16_t, float>(dxg, dag, w_i, w_a, addend, dx, M, D, nb, bw, dx_dtype, st);
     }
     if (w_dtype == HAWK_DTYPE_BF16)
-        return gate_bwd_input_out<float, bf16_t>(dxg, dag, w_i, w_a, dx, M, D, nb, bw, dx_dtype, st);
-    return gate_bwd_input_out<float, float>(dxg, dag, w_i, w_a, dx, M, D, nb, bw, dx_dtype, st);
+        return gate_bwd_input_out<float, bf16_t>(dxg, dag, w_i, w_a, addend, dx, M, D, nb, bw, dx_dtype, st);
+    return gate_bwd_input_out<float, float>(dxg, dag, w_i, w_a, addend, dx, M, D, nb, bw, dx_dtype, st);
 }
 
 size_t gate_proj_bwd_weights_workspace_bytes(int M, int D, int nb) {

@@ -49,8 +49,8 @@ int rglru_step_gated(const void* x, const void* xg, const void* ag, const float*
 bool gate_proj_block_width_supported(int bw);
 int gate_proj_fwd(const void* x, const void* w_i, const float* b_i, const void* w_a, const float* b_a, void* out_i,
                   void* out_a, int M, int D, int nb, int x_dtype, int w_dtype, int out_dtype, hipStream_t st);
-int gate_proj_bwd_input(const void* dxg, const void* dag, const void* w_i, const void* w_a, void* dx, int M, int D,
-                        int nb, int g_dtype, int w_dtype, int dx_dtype, hipStream_t st);
+int gate_proj_bwd_input(const void* dxg, const void* dag, const void* w_i, const void* w_a, const void* addend,
+                        void* dx, int M, int D, int nb, int g_dtype, int w_dtype, int dx_dtype, hipStream_t st);
 size_t gate_proj_bwd_weights_workspace_bytes(int M, int D, int nb);
 int gate_proj_bwd_weights(const void* x, const void* dg_i, const void* dg_a, float* dw_i, float* db_i, float* dw_a,
                           float* db_a, int M, int D, int nb, int x_dtype, int g_dtype, void* ws, size_t ws_bytes,

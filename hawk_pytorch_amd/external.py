@@ -343,7 +343,7 @@ def _launch_gate_fwd(x, w_i, b_i, w_a, b_a, out_bf16: bool):
     return xg, ag
 
 
-def _launch_gate_bwd(x, d_xg, d_ag, w_i, w_a):
+def _launch_gate_bwd(x, d_xg, d_ag, w_i, w_a, addend=None):
     dev = _lib.require_cuda(x, d_xg, d_ag, w_i, w_a)
     nb, bw, _ = w_i.shape
     D = nb * bw
@@ -351,6 +351,8 @@ def _launch_gate_bwd(x, d_xg, d_ag, w_i, w_a):
     x2, g_i, g_a, w_i, w_a = (_lib.dense16(t) for t in (x.reshape(M, D), d_xg.reshape(M, D), d_ag.reshape(M, D), w_i, w_a))
     lib = _lib.load()
     dx = torch.empty(x.shape, dtype=x.dtype, device=dev)
+    if addend is not None:
+        addend = _lib.dense16(addend.reshape(M, D).to(x.dtype))
     dw_i = torch.empty((nb, bw, bw), dtype=torch.float32, device=dev)
     dw_a = torch.empty_like(dw_i)
     db_i = torch.empty(D, dtype=torch.float32, device=dev)
@@ -360,7 +362,7 @@ def _launch_gate_bwd(x, d_xg, d_ag, w_i, w_a):
     with torch.cuda.device(dev):
         st = _lib.stream_ptr(dev)
         status = lib.hawk_gate_proj_bwd_input(
-            g_i.data_ptr(), g_a.data_ptr(), w_i.data_ptr(), w_a.data_ptr(), dx.data_ptr(), M, D, nb,
+            g_i.data_ptr(), g_a.data_ptr(), w_i.data_ptr(), w_a.data_ptr(), _lib.ptr(addend), dx.data_ptr(), M, D, nb,
             _lib.dtype_code(g_i.dtype), _lib.dtype_code(w_i.dtype), _lib.dtype_code(dx.dtype), st,
         )
         _lib.check("hawk_gate_proj_bwd_input", status)
@@ -388,13 +390,14 @@ def _(x, w_i, b_i, w_a, b_a, out_bf16):
 
 @torch.library.custom_op("hawk_amd::gate_proj_bwd", mutates_args=(), device_types="cuda")
 def _gate_proj_bwd_op(
-    x: torch.Tensor, d_xg: torch.Tensor, d_ag: torch.Tensor, w_i: torch.Tensor, w_a: torch.Tensor
+    x: torch.Tensor, d_xg: torch.Tensor, d_ag: torch.Tensor, w_i: torch.Tensor, w_a: torch.Tensor,
+    addend: Optional[torch.Tensor] = None,
 ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
-    return _launch_gate_bwd(x, d_xg, d_ag, w_i, w_a)
+    return _launch_gate_bwd(x, d_xg, d_ag, w_i, w_a, addend)
 
 
 @_gate_proj_bwd_op.register_fake
-def _(x, d_xg, d_ag, w_i, w_a):
+def _(x, d_xg, d_ag, w_i, w_a, addend=None):
     nb, bw, _ = w_i.shape
     f32 = dict(dtype=torch.float32, device=x.device)
     return (

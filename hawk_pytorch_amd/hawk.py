@@ -39,7 +39,7 @@ from .external import (
     temporal_conv1d,
     temporal_conv1d_step,
 )
-from .scan_fused import fused_linear_scan, fused_linear_scan_gated
+from .scan_fused import fused_linear_scan, fused_linear_scan_gated, recurrent_core
 
 
 @dataclass
@@ -153,16 +153,23 @@ class Hawk(nn.Module):
             if self.use_cache:
                 assert layer_past is not None, "use_cache=True needs one RNNCache per layer in layer_past"
                 layer_past.seed_conv_state(branch)
+            cache = layer_past if self.use_cache else None
             if self.config.fused_gates and gate_projections_supported(branch, self.rg_lru_input_gate):
                 # bf16 end to end: upstream's gate einsums (under autocast) and its scan
                 # (cast_inputs, hawk/scan_fused.py:428) round the conv output to bf16 anyway
                 u = temporal_conv1d(branch, self.conv1d.w, self.conv1d.b, torch.bfloat16)
+                if self.config.fused_epilogue:
+                    # projections, scan and output gate as one autograd node
+                    gated, h_last = recurrent_core(u, self.rg_lru_input_gate, self.rg_lru_a_gate,
+                                                   self.rg_lru_a_param, gate_branch, return_last_state=True)
+                    if self.use_cache:
+                        layer_past.update_cache(h_last)
+                    return self.resid_proj(gated), cache
                 xg, ag = gate_projections(u, self.rg_lru_input_gate, self.rg_lru_a_gate, torch.bfloat16)
             else:
                 u = self.conv1d(branch)
                 xg, ag = self.rg_lru_input_gate(u), self.rg_lru_a_gate(u)
             gates = (xg, ag, self.rg_lru_a_param.float())
-            cache = layer_past if self.use_cache else None
             if self.config.fused_epilogue:
                 gated, h_last = fused_linear_scan_gated(u, *gates, gate_branch, return_last_state=True)
                 if self.use_cache:

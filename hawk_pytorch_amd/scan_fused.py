@@ -419,3 +419,51 @@ def fused_linear_scan_gated(x, x_rg_lru, a_rg_lru, a_param, y, return_last_state
     """
     out, h_last = GatedDiagonalRecurrence.apply(x, x_rg_lru, a_rg_lru, a_param, y, return_last_state)
     return (out, h_last) if return_last_state else out
+
+
+# ---------------------------------------------------------------------------------------
+# The recurrent core of a Hawk block as one autograd node: both gate projections, the scan
+# and the output gate (hawk/hawk.py:181-186 and :134-135).  Besides saving launches, one
+# node lets the backward hand the scan's gradient of u to the projection kernel, which adds
+# it to its own on the way out; as separate nodes autograd would sum the two in an extra
+# pass over the tensor.
+# ---------------------------------------------------------------------------------------
+class RecurrentCore(Function):
+    @staticmethod
+    def forward(ctx, u, w_i, b_i, w_a, b_a, a_param, y, want_last):
+        from .external import _gate_proj_fwd_op  # deferred: external imports nothing from here
+
+        assert u.dtype == torch.bfloat16, "the fused core runs on bf16 activations"
+        uc = u if u.is_contiguous() else u.contiguous()
+        lam = a_param.float().contiguous()
+        xg, ag = _gate_proj_fwd_op(uc, w_i, b_i.float().reshape(-1), w_a, b_a.float().reshape(-1), True)
+        _check_shapes(uc, xg, ag, a_param)
+        want_h = any(ctx.needs_input_grad[:7])
+        out, h, h_last = _rglru_scan_gated_fwd_op(uc, xg, ag, lam, y, True, want_h, bool(want_last))
+        if want_h:
+            ctx.save_for_backward(uc, xg, ag, h, y, w_i, w_a, a_param)
+        ctx.dtypes = (w_i.dtype, b_i.dtype, w_a.dtype, b_a.dtype, a_param.dtype, y.dtype)
+        ctx.mark_non_differentiable(h_last)
+        return out, h_last
+
+    @staticmethod
+    def backward(ctx, grad_out, _grad_last):  # type: ignore[override]
+        from .external import _gate_proj_bwd_op
+
+        u, xg, ag, h, y, w_i, w_a, a_param = ctx.saved_tensors
+        go = grad_out if grad_out.dtype == h.dtype else grad_out.to(h.dtype)
+        go = go if go.is_contiguous() else go.contiguous()
+        du_scan, d_xg, d_ag, dlam, dy = _rglru_scan_gated_bwd_op(u, xg, ag, a_param.float().contiguous(), y, h, go)
+        du, dw_i, db_i, dw_a, db_a = _gate_proj_bwd_op(u, d_xg, d_ag, w_i, w_a, du_scan)
+        nb, bw, _ = w_i.shape
+        t = ctx.dtypes
+        return (du, dw_i.to(t[0]), db_i.reshape(nb, bw).to(t[1]), dw_a.to(t[2]), db_a.reshape(nb, bw).to(t[3]),
+                dlam.to(t[4]), dy.to(t[5]), None)
+
+
+def recurrent_core(u, input_gate, a_gate, a_param, y, return_last_state: bool = False):
+    """``gelu(y) * scan(u, input_gate(u), a_gate(u), a_param)`` for bf16 ``u`` and gate modules
+    the fused projection kernels serve (see ``external.gate_projections_supported``)."""
+    out, h_last = RecurrentCore.apply(u, input_gate.w, input_gate.b, a_gate.w, a_gate.b, a_param, y,
+                                      return_last_state)
+    return (out, h_last) if return_last_state else out

@@ -208,12 +208,15 @@ int hawk_gate_proj_fwd(const void* x, const void* w_i, const float* b_i, const v
 
 /* Gradient of the two projections with respect to x, in one pass over both logit gradients:
  *   dx[m, h*bw+i] = sum_j d_x_rg_lru[m, h*bw+j] w_i[h, i, j] + sum_j d_a_rg_lru[m, h*bw+j] w_a[h, i, j]
+ *                   (+ addend[m, h*bw+i])
  * (what autograd derives from the einsum of hawk/external.py:230, twice, plus the add of
- * the two results).  Gradients have g_dtype, weights w_dtype, dx has dx_dtype; operands are
- * rounded to bf16 in registers, sums are fp32. */
+ * the two results).  addend [M,D] (dx_dtype) may be NULL; it is the gradient x receives from
+ * its other consumer, the scan (hawk/hawk.py:186), whose accumulation autograd would
+ * otherwise do in a separate pass; it may alias dx.  Gradients have g_dtype, weights
+ * w_dtype, dx has dx_dtype; operands are rounded to bf16 in registers, sums are fp32. */
 int hawk_gate_proj_bwd_input(const void* d_x_rg_lru, const void* d_a_rg_lru, const void* w_i,
-                             const void* w_a, void* dx, int M, int D, int num_blocks, int g_dtype,
-                             int w_dtype, int dx_dtype, void* stream);
+                             const void* w_a, const void* addend, void* dx, int M, int D,
+                             int num_blocks, int g_dtype, int w_dtype, int dx_dtype, void* stream);
 
 /* Gradients of the weights and biases of the two projections:
  *   dw_g[h, i, j] = sum_m x[m, h*bw+i] d_g[m, h*bw+j],   db_g[c] = sum_m d_g[m, c]

@@ -216,13 +216,14 @@ def gate_proj_fwd(x, w_i, b_i, w_a, b_a, out_dtype=None):
     return oi, oa
 
 
-def gate_proj_bwd_input(dxg, dag, w_i, w_a, dx_dtype=None):
+def gate_proj_bwd_input(dxg, dag, w_i, w_a, dx_dtype=None, addend=None, in_place=False):
+    """addend: optional [M,D] tensor of dx's dtype added to the result; in_place writes over it."""
     M, D = dxg.shape
     nb = w_i.shape[0]
     dx_dtype = dx_dtype or dxg.dtype
-    dx = torch.empty((M, D), dtype=dx_dtype, device="cuda")
+    dx = addend if in_place else torch.empty((M, D), dtype=dx_dtype, device="cuda")
     rc = _lib.load().hawk_gate_proj_bwd_input(
-        dxg.data_ptr(), dag.data_ptr(), w_i.data_ptr(), w_a.data_ptr(), dx.data_ptr(), M, D, nb,
+        dxg.data_ptr(), dag.data_ptr(), w_i.data_ptr(), w_a.data_ptr(), _lib.ptr(addend), dx.data_ptr(), M, D, nb,
         _lib.dtype_code(dxg.dtype), _lib.dtype_code(w_i.dtype), _lib.dtype_code(dx_dtype), _stream())
     _lib.check("hawk_gate_proj_bwd_input", rc)
     return dx

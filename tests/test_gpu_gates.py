@@ -188,3 +188,21 @@ def test_weight_gradients_full_shape_against_the_library_gemm_and_reproducible()
         assert float((dw - ref_w).abs().max() / ref_w.abs().max()) < 1e-4
         ref_b = gd.double().sum(dim=0)
         assert float((db.double() - ref_b).abs().max() / ref_b.abs().max()) < 1e-4
+
+
+def test_input_gradient_adds_the_addend_also_in_place():
+    M, D, nb = 1000, 2560, 10
+    g = torch.Generator(device="cuda").manual_seed(4)
+    mk = lambda: torch.randn((M, D), generator=g, device="cuda").to(torch.bfloat16)  # noqa: E731
+    gi, ga, add = mk(), mk(), mk()
+    wi = torch.randn((nb, 256, 256), generator=g, device="cuda") / 16.0
+    wa = torch.randn((nb, 256, 256), generator=g, device="cuda") / 16.0
+    plain = capi.gate_proj_bwd_input(gi, ga, wi, wa, torch.float32)
+    want = plain + add.float()
+    got = capi.gate_proj_bwd_input(gi, ga, wi, wa, torch.bfloat16, addend=add)
+    assert max_rel(capi.to_np(got), capi.to_np(want)) < 2e-2
+    got32 = capi.gate_proj_bwd_input(gi, ga, wi, wa, torch.float32, addend=add.float())
+    assert max_rel(capi.to_np(got32), capi.to_np(want)) < 1e-6
+    buf = add.clone()
+    same = capi.gate_proj_bwd_input(gi, ga, wi, wa, torch.bfloat16, addend=buf, in_place=True)
+    assert same.data_ptr() == buf.data_ptr() and torch.equal(buf, got)

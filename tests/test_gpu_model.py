@@ -413,3 +413,40 @@ def test_torch_compile_traces_the_whole_model_under_autocast():
     assert abs(got.item() - eager.item()) < 1e-3
     for n, p in model.named_parameters():
         assert max_rel(capi.to_np(p.grad), capi.to_np(want[n])) < 1e-2, n
+
+
+def test_recurrent_core_matches_its_parts():
+    """One autograd node (projections + scan + gate, gradient of u accumulated in the
+    projection kernel) against the same kernels as separate nodes."""
+    torch.manual_seed(12)
+    D, nb, B, T = 512, 4, 2, 300
+    gi = hk.BlockDiagonalLinear(D, nb).cuda()
+    ga = hk.BlockDiagonalLinear(D, nb).cuda()
+    with torch.no_grad():
+        gi.b.normal_()
+        ga.b.normal_()
+    lam = torch.nn.Parameter(torch.tensor(make_scan_inputs(1, 1, D, seed=1)[3], device="cuda", dtype=torch.float32))
+    u = torch.randn(B, T, D, device="cuda").to(torch.bfloat16).requires_grad_(True)
+    wide = torch.randn(B, T, 2 * D, device="cuda").to(torch.bfloat16).requires_grad_(True)
+    go = torch.randn(B, T, D, device="cuda").to(torch.bfloat16)
+    params = (u, wide, lam, gi.w, gi.b, ga.w, ga.b)
+
+    def run(fn):
+        for p in params:
+            p.grad = None
+        with torch.autocast(device_type="cuda", dtype=torch.bfloat16):
+            out, last = fn(wide.chunk(2, dim=-1)[1])
+        out.backward(go)
+        return (out.detach().float(), last.detach().float(), *(p.grad.detach().float().clone() for p in params))
+
+    def parts(y):
+        xg, ag = hk.gate_projections(u, gi, ga, torch.bfloat16)
+        return hk.fused_linear_scan_gated(u, xg, ag, lam, y, return_last_state=True)
+
+    got = run(lambda y: hk.recurrent_core(u, gi, ga, lam, y, return_last_state=True))
+    want = run(parts)
+    names = ("out", "h_last", "du", "d_xy", "dLambda", "dw_i", "db_i", "dw_a", "db_a")
+    for name, a, b in zip(names, got, want):
+        assert a.shape == b.shape, name
+        assert max_rel(capi.to_np(a), capi.to_np(b)) < 1e-2, (name, max_rel(capi.to_np(a), capi.to_np(b)))
+    assert torch.equal(got[0], want[0])  # the forward is the very same pair of kernels
