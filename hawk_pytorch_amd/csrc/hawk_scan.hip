@@ -615,20 +615,21 @@ __device__ __forceinline__ void bwd_tile(const IT* __restrict__ x, const IT* __r
             const float g = fgo[v] + c_true[v];
             c_true[v] = alpha * g;
             const float i = sigmoid_fast(fxg[v]);
-            const float a2 = alpha * alpha;
-            const float z = PRECISE ? one_minus_exp(2.0f * cs[v] * r) : clamp01(1.0f - a2);
-            const float rs = hw_rsq(fmaxf(z, 1e-30f));
-            const float m = z * rs;
-            // 2 * clipped sqrt derivative: 1/sqrt(max(4z,1e-6)) = 0.5/sqrt(max(z,2.5e-7))
-            const float csg2 = (z >= 2.5e-7f) ? rs : 2000.0f;
+            const float z = PRECISE ? one_minus_exp(2.0f * cs[v] * r) : clamp01(fmaf(-alpha, alpha, 1.0f));
+            const float m = hw_sqrt(z);
+            // 2 * clipped sqrt derivative: 1/sqrt(max(4z,1e-6)) = 0.5/sqrt(max(z,2.5e-7)), at most 2000
+            const float csg2 = hw_rsq(fmaxf(z, 2.5e-7f));
             const float ix = i * fx[v];
             const float gm = g * m;
-            float k4 = fmaf(fhp[v], alpha, -(ix * a2) * csg2) * r;  // dlog_a / g * r
+            const float ixa2 = PRECISE ? ix * (alpha * alpha) : fmaf(-ix, z, ix);  // i x alpha^2
+            float k4 = fmaf(fhp[v], alpha, -ixa2 * csg2) * r;  // dlog_a / g * r
             if (!ok) k4 = 0.0f;
             const float gk4 = g * k4;
             o1[v] = gm * i;
-            o2[v] = (gm * ix) * (1.0f - i);
-            o3[v] = (gk4 * (1.0f - r)) * cs[v];
+            const float t2 = o1[v] * fx[v];   // g m i x
+            o2[v] = fmaf(-t2, i, t2);         // ... (1 - i)
+            const float t3 = gk4 * cs[v];
+            o3[v] = fmaf(-t3, r, t3);         // g k4 (-8 s) (1 - r)
             acc[v] += gk4;
         }
         raw_t r1, r2, r3;
