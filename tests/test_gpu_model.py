@@ -262,43 +262,47 @@ def test_model_gradients_match_a_pure_torch_model_of_the_same_weights(fused_epil
 def test_readme_model_config_bf16_autocast_training_step():
     """The upstream README's model (vocab 32000, hidden = recurrent = 512, MLP 1024, 8 layers,
     16 gate blocks, conv 4) on a 1 x 2048 batch under bf16 autocast, forward and backward,
-    against the same weights run in fp32 with the torch-loop scan and the library conv."""
+    for every combination of the fused-kernel switches, against the same weights run in fp32
+    with the torch-loop scan, the library conv and the library gate GEMMs."""
     torch.manual_seed(3)
     cfg = hk.HawkConfig(vocab_size=32000, hidden_size=512, intermediate_size=1024, num_hidden_layers=8,
                         recurrent_size=512, num_blocks=16, conv_width=4)
     model = hk.HawkModel(cfg).cuda()
     _randomise_zero_inits(model)
     ids = torch.randint(1, cfg.vocab_size, (1, 2048), device="cuda")
-    with torch.autocast(device_type="cuda", dtype=torch.bfloat16):
-        loss = model(ids, ids)
-    loss.backward()
-    got = {n: p.grad.detach().float().clone() for n, p in model.named_parameters()}
-    assert all(torch.isfinite(g).all() for g in got.values())
 
     import hawk_pytorch_amd.hawk as hm
     import hawk_pytorch_amd.external as he
 
-    def ref_scan_gated(x, xg, ag, lam, y, return_last_state=False):
-        h = rglru_torch.rglru_scan_loop(x, xg, ag, lam)
-        out = F.gelu(y) * h
-        return (out, h[:, -1:, :].detach()) if return_last_state else out
+    def ref_scan(x, xg, ag, lam):
+        return rglru_torch.rglru_scan_loop(x, xg, ag, lam)
 
     def ref_conv(self, x, state=None):
         return rglru_torch.conv1d_library(x, self.w, self.b)
 
-    model.zero_grad()
-    old = hm.fused_linear_scan_gated, he.Conv1D.forward
+    cfg.fused_gates, cfg.fused_epilogue = False, False
+    old = hm.fused_linear_scan, he.Conv1D.forward
     try:
-        hm.fused_linear_scan_gated, he.Conv1D.forward = ref_scan_gated, ref_conv
+        hm.fused_linear_scan, he.Conv1D.forward = ref_scan, ref_conv
         ref_loss = model(ids, ids)
         ref_loss.backward()
     finally:
-        hm.fused_linear_scan_gated, he.Conv1D.forward = old
-    assert abs(loss.item() - ref_loss.item()) < 2e-2 * abs(ref_loss.item())
-    for n, p in model.named_parameters():
-        a, b = got[n].flatten(), p.grad.float().flatten()
-        cos = float(torch.dot(a, b) / (a.norm() * b.norm() + 1e-30))
-        assert cos > 0.99, (n, cos)
+        hm.fused_linear_scan, he.Conv1D.forward = old
+    want = {n: p.grad.detach().float().clone() for n, p in model.named_parameters()}
+
+    for fused_gates, fused_epilogue in [(True, True), (True, False), (False, True), (False, False)]:
+        cfg.fused_gates, cfg.fused_epilogue = fused_gates, fused_epilogue
+        model.zero_grad()
+        with torch.autocast(device_type="cuda", dtype=torch.bfloat16):
+            loss = model(ids, ids)
+        loss.backward()
+        case = (fused_gates, fused_epilogue)
+        assert abs(loss.item() - ref_loss.item()) < 2e-2 * abs(ref_loss.item()), case
+        for n, p in model.named_parameters():
+            a, b = p.grad.float().flatten(), want[n].flatten()
+            assert torch.isfinite(a).all(), (case, n)
+            cos = float(torch.dot(a, b) / (a.norm() * b.norm() + 1e-30))
+            assert cos > 0.99, (case, n, cos)
 
 
 def test_torch_compile_traces_the_ops_without_graph_breaks():
