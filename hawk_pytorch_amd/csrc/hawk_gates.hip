@@ -254,7 +254,7 @@ __global__ __launch_bounds__(kGateThreads, 1) void gate_proj_fwd_kernel(
 // matrix, contiguous in memory) as B operands, reads gate g's gradient tile from LDS as A
 // operands, and the two gates' partial tiles are added on the way out.
 // ---------------------------------------------------------------------------------------
-template <typename GT, typename WT, typename DT, int BW>
+template <typename GT, typename WT, typename DT, int BW, bool ADD>
 __global__ __launch_bounds__(kGateThreads, 1) void gate_proj_bwd_input_kernel(
     const GT* __restrict__ dxg, const GT* __restrict__ dag, const WT* __restrict__ w_i, const WT* __restrict__ w_a,
     const DT* __restrict__ addend, DT* __restrict__ dx, int M, int D, int nb, int ntiles) {
@@ -323,7 +323,7 @@ __global__ __launch_bounds__(kGateThreads, 1) void gate_proj_bwd_input_kernel(
         const int row = (worker + it * nworkers) * kTileRows + lrow;
         const bool out_ok = col_ok && row < M;
         Row8<DT> radd;
-        radd.load(addend + (out_ok && addend != nullptr ? (size_t)row * D + lcol : 0), out_ok && addend != nullptr);
+        if constexpr (ADD) radd.load(addend + (out_ok ? (size_t)row * D + lcol : 0), out_ok);
         f32x16 acc = {};
         const unsigned char* a_base = sA + (2 * cur) * kATileBytes + a_off;
         constexpr int kBatch = KS < 4 ? KS : 4;
@@ -349,9 +349,13 @@ __global__ __launch_bounds__(kGateThreads, 1) void gate_proj_bwd_input_kernel(
             const f32x4 p0 = *reinterpret_cast<const f32x4*>(o_src), p1 = *reinterpret_cast<const f32x4*>(o_src + 16);
             const f32x4 q0 = *reinterpret_cast<const f32x4*>(o_src + kOTileBytes);
             const f32x4 q1 = *reinterpret_cast<const f32x4*>(o_src + kOTileBytes + 16);
-            f32x4 e0, e1;
-            radd.as_f32(e0, e1);
-            const f32x4 s0 = (p0 + q0) + e0, s1 = (p1 + q1) + e1;
+            f32x4 s0 = p0 + q0, s1 = p1 + q1;
+            if constexpr (ADD) {
+                f32x4 e0, e1;
+                radd.as_f32(e0, e1);
+                s0 += e0;
+                s1 += e1;
+            }
             DT* dst = dx + (size_t)row * D + lcol;
             if constexpr (sizeof(DT) == 4) {
                 __builtin_nontemporal_store(s0, reinterpret_cast<f32x4*>(dst));
@@ -625,7 +629,8 @@ int launch_gate_bwd_input(const void* dxg, const void* dag, const void* w_i, con
     if (nworkers < 1) nworkers = 1;
     if (nworkers > ntiles) nworkers = ntiles;
     const size_t smem = 4 * kATileBytes + 2 * (size_t)kTileRows * (kGroup * 4 + 16);
-    auto kernel = gate_proj_bwd_input_kernel<GT, WT, DT, BW>;
+    auto kernel = addend != nullptr ? gate_proj_bwd_input_kernel<GT, WT, DT, BW, true>
+                                    : gate_proj_bwd_input_kernel<GT, WT, DT, BW, false>;
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                             (int)smem) != hipSuccess)
         return HAWK_ERR_LAUNCH;
