@@ -12,6 +12,9 @@ D=4096; ``--workload scan_conv`` adds the temporal conv1d forward and backward;
 y being one half of a [B, T, 2D] projection), 12 + 20 bytes per element;
 ``--workload gates`` runs the fused block-diagonal gate projections (matrix-core kernels:
 forward, input gradient, weight gradients) on 32768 tokens, D = 2560, 10 blocks, bf16;
+``--workload block`` chains the whole recurrent core of one layer at B=8, T=4096, D=2560 (conv,
+both gate projections, scan fused with the output gate, and the backward of all of them)
+through the C ABI, seven launches that move 31 activation-sized tensors;
 ``--workload model`` runs full training steps (forward, backward, AdamW) of the upstream
 README model (vocabulary 32000, hidden = recurrent = 512, MLP 1024, 8 layers, 16 gate blocks)
 on a 1 x 2048 batch under bf16 autocast, with and without the fused gate / epilogue kernels;
@@ -174,6 +177,92 @@ def run_gates(args, lib, dev):
                     for i, name in enumerate(("fwd", "bwd_input", "bwd_weights"))},
     }
     print(json.dumps(out))
+
+
+def run_block(args, lib, dev):
+    """conv -> gate projections -> gated scan, forward and backward, bf16 end to end."""
+    from hawk_pytorch_amd import _lib
+
+    B, T, D, nb, W = 8, 4096, 2560, 10, 4
+    M, bw, N = B * T, D // nb, B * T * D
+    bf, code, f32 = torch.bfloat16, _lib.HAWK_DTYPE_BF16, _lib.HAWK_DTYPE_F32
+    gen = torch.Generator(device=dev).manual_seed(args.seed)
+    xy = torch.randn(B, T, 2 * D, device=dev, generator=gen).to(bf)
+    xin = xy[..., :D].contiguous()          # conv input; the gate half stays in place
+    y = xy[..., D:]
+    gout = torch.randn(B, T, D, device=dev, generator=gen).to(bf)
+    cw = (torch.randn(W, D, device=dev, generator=gen) * 0.5).float()
+    cb = torch.zeros(D, device=dev)
+    wi, wa = (torch.randn(nb, bw, bw, device=dev, generator=gen) / bw ** 0.5 for _ in range(2))
+    bi, ba = (torch.randn(D, device=dev, generator=gen) * 0.1 for _ in range(2))
+    lam = lambda_for_a8_range(torch.Generator().manual_seed(args.seed), D, 0.9, 0.999).to(dev)
+    e = lambda: torch.empty(B, T, D, device=dev, dtype=bf)  # noqa: E731
+    u, xg, ag, h, out = e(), e(), e(), e(), e()
+    du, dxg, dag, dy, dxin = e(), e(), e(), e(), e()
+    dlam = torch.empty(D, device=dev)
+    dwi, dwa, dbi, dba = torch.empty_like(wi), torch.empty_like(wa), torch.empty_like(bi), torch.empty_like(ba)
+    dcw, dcb = torch.empty_like(cw), torch.empty_like(cb)
+    ws = torch.zeros(lib.hawk_scan_workspace_bytes(B, T, D, code), dtype=torch.uint8, device=dev)
+    gws = torch.empty(lib.hawk_gate_proj_bwd_weights_workspace_bytes(M, D, nb), dtype=torch.uint8, device=dev)
+    cws = torch.empty(lib.hawk_conv1d_bwd_workspace_bytes(B, T, D, W), dtype=torch.uint8, device=dev)
+    st = torch.cuda.current_stream(dev).cuda_stream
+    p = lambda t: t.data_ptr()  # noqa: E731
+
+    def fwd():
+        _lib.check("conv_fwd", lib.hawk_conv1d_fwd(p(xin), p(cw), p(cb), None, p(u), B, T, D, W, code, code, st))
+        _lib.check("gate_fwd", lib.hawk_gate_proj_fwd(p(u), p(wi), p(bi), p(wa), p(ba), p(xg), p(ag), M, D, nb,
+                                                      code, f32, code, st))
+        _lib.check("scan_gated_fwd", lib.hawk_rglru_scan_gated_fwd(
+            p(u), p(xg), p(ag), p(lam), p(y), 2 * D, p(h), p(out), None, B, T, D, code, code, p(ws), ws.numel(), st))
+
+    def bwd():
+        _lib.check("scan_gated_bwd", lib.hawk_rglru_scan_gated_bwd(
+            p(u), p(xg), p(ag), p(lam), p(y), 2 * D, p(h), p(gout), p(du), p(dxg), p(dag), p(dy), D, p(dlam),
+            B, T, D, code, code, p(ws), ws.numel(), st))
+        # the projections' input gradient accumulates onto the scan's, in place
+        _lib.check("gate_bwd_input", lib.hawk_gate_proj_bwd_input(p(dxg), p(dag), p(wi), p(wa), p(du), p(du), M, D,
+                                                                  nb, code, f32, code, st))
+        _lib.check("gate_bwd_weights", lib.hawk_gate_proj_bwd_weights(
+            p(u), p(dxg), p(dag), p(dwi), p(dbi), p(dwa), p(dba), M, D, nb, code, code, p(gws), gws.numel(), st))
+        _lib.check("conv_bwd", lib.hawk_conv1d_bwd(p(du), p(xin), p(cw), p(dxin), p(dcw), p(dcb), B, T, D, W, code,
+                                                   code, p(cws), cws.numel(), st))
+
+    for _ in range(args.warmup):
+        fwd(), bwd()
+    torch.cuda.synchronize()
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
+    t0 = time.perf_counter()
+    for k in range(args.steps):
+        ev[k][0].record()
+        fwd()
+        ev[k][1].record()
+        bwd()
+        ev[k][2].record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    flag = ctypes.c_int(0)
+    _lib.check("status", lib.hawk_scan_workspace_status(ws.data_ptr(), st, ctypes.byref(flag)))
+    assert flag.value == 0 and bool(torch.isfinite(dxin.float()).all())
+    fwd_ms = float(np.mean([e_[0].elapsed_time(e_[1]) for e_ in ev]))
+    bwd_ms = float(np.mean([e_[1].elapsed_time(e_[2]) for e_ in ev]))
+    ms_per_step = wall * 1e3 / args.steps
+    # tensors moved: conv 2, gates 3, gated scan 6 | gated scan 10, gate dx 4, gate dw 3, conv 3
+    fwd_bytes, bwd_bytes = 11 * 2 * N, 20 * 2 * N
+    step_gbs = (fwd_bytes + bwd_bytes) / (ms_per_step * 1e-3) / 1e9
+    print(json.dumps({
+        "metric": "Hawk recurrent core (conv, gate projections, gated scan) fwd+bwd tokens/s, 1 GPU",
+        "value": B * T / (ms_per_step * 1e-3), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16 activations, f32 parameters, state and accumulation",
+        "data": f"synthetic, seed {args.seed}",
+        "config": {"workload": f"block: conv1d(4) + gate projections ({nb} blocks) + scan fused with gelu(y)*h, "
+                               f"fwd+bwd, B={B}, T={T}, D={D}, bf16", "B": B, "T": T, "D": D},
+        "roofline": {"bound": "hbm", "kernel": "all seven launches of the step", "achieved": step_gbs,
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": step_gbs / HBM_PEAK_GBS, "traffic": None,
+                     "algorithmic_bytes_per_launch": fwd_bytes + bwd_bytes},
+        "fwd": {"ms": fwd_ms, "GBs": fwd_bytes / (fwd_ms * 1e-3) / 1e9},
+        "bwd": {"ms": bwd_ms, "GBs": bwd_bytes / (bwd_ms * 1e-3) / 1e9},
+    }))
 
 
 def run_model(args, lib, dev):
@@ -363,7 +452,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", choices=sorted(WORKLOADS) + ["decode", "gates", "model"], default="scan")
+    ap.add_argument("--workload", choices=sorted(WORKLOADS) + ["block", "decode", "gates", "model"], default="scan")
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calibration-copy", action="store_true",
@@ -393,6 +482,9 @@ def main():
         return
     if args.workload == "model":
         run_model(args, lib, dev)
+        return
+    if args.workload == "block":
+        run_block(args, lib, dev)
         return
     B, T, D, (lo, hi), with_conv = WORKLOADS[args.workload]
     N = B * T * D
