@@ -14,13 +14,15 @@
 //     and keeps that slice of the weights, bw x 32, in registers as MFMA B operands for the
 //     whole kernel (64 VGPRs at bw = 256): the weights are read once per workgroup;
 //   * the 32 x 256 activation tile goes global -> registers -> LDS with 16-byte accesses
-//     along rows (fp32 activations are rounded to bf16 on the way), is prefetched three
-//     tiles ahead, and is read back as MFMA A operands by all 16 waves;
+//     along rows (fp32 activations are rounded to bf16 on the way); two register sets and
+//     two LDS buffers keep the next two tiles in flight; all 16 waves read the tile back as
+//     MFMA A operands;
 //   * results pass through LDS once more so that each row leaves in 512-byte (bf16) or
 //     1-KiB (fp32) pieces.
 // Per 32-row tile a CU moves 16 KiB in and 32 KiB out (bf16) against 16 waves x bw/16 MFMAs
-// of 32x32x16; at bw = 256 that is about 2 k cycles of matrix-core time against about 5 k
-// cycles of HBM time at 5 TB/s, so the kernel is bound by HBM.
+// of 32x32x16.  At bw = 256 that is about 2 k cycles of matrix-core time and, because every
+// MFMA takes a fresh 1 KiB A operand from LDS, as many cycles of LDS time, against about 5 k
+// cycles of HBM time at 5 TB/s; with the result pass and the barriers a tile takes about 6 k.
 #include "hawk_scan.h"
 
 #include <stdint.h>
