@@ -193,3 +193,49 @@ def test_python_rule_for_fused_gate_projections_matches_the_library():
     for D, nb in [(2560, 10), (512, 16), (512, 8), (512, 4), (512, 2), (512, 1), (96, 3), (100, 3), (4096, 16), (48, 3)]:
         python_rule = D % nb == 0 and (D // nb) in _GATE_BLOCK_WIDTHS
         assert bool(lib.hawk_gate_proj_supported(D, nb)) == python_rule, (D, nb)
+
+
+def test_argument_validation_of_the_gated_and_projection_entry_points():
+    lib = _lib.load()
+    buf = (ctypes.c_char * 4096)()
+    p = (ctypes.addressof(buf) + 15) & ~15
+    E = _lib
+    # gated scan forward: (x, xg, ag, lam, y, ldy, h, out, h_last, B, T, D, in, out, ws, bytes, stream)
+    ok = [p, p, p, p, p, 64, p, p, None, 1, 8, 64, 0, 0, None, 0, None]
+
+    def gf(**kw):
+        a = list(ok)
+        for k, v in kw.items():
+            a[int(k[1:])] = v
+        return lib.hawk_rglru_scan_gated_fwd(*a)
+
+    assert gf(a4=None) == E.HAWK_ERR_NULL_POINTER            # y
+    assert gf(a7=None) == E.HAWK_ERR_NULL_POINTER            # out
+    assert gf(a5=63) == E.HAWK_ERR_BAD_SHAPE                 # row stride below D
+    assert gf(a5=1 << 25) == E.HAWK_ERR_BAD_SHAPE            # row stride beyond the addressing limit
+    assert gf(a12=1, a13=0, a10=4096) == E.HAWK_ERR_WORKSPACE  # (f32, bf16) is an offered pair: next check fails
+    assert gf(a12=0, a13=1) == E.HAWK_ERR_BAD_DTYPE
+    assert gf(a4=p + 1) == E.HAWK_ERR_ALIGNMENT              # y must be element aligned
+    assert gf(a10=4096) == E.HAWK_ERR_WORKSPACE              # several tiles, no workspace
+    # gated scan backward needs dy and a workspace
+    gb = [p, p, p, p, p, 64, p, p, p, p, p, p, 64, p, 1, 8, 64, 0, 0, None, 0, None]
+    assert lib.hawk_rglru_scan_gated_bwd(*gb) == E.HAWK_ERR_WORKSPACE
+    gb[11] = None
+    assert lib.hawk_rglru_scan_gated_bwd(*gb) == E.HAWK_ERR_NULL_POINTER
+    # decode step with gate
+    assert lib.hawk_rglru_step_gated(p, p, p, None, None, p, None, 64, p, None, p, 1, 64, 0, 0, None) \
+        == E.HAWK_ERR_NULL_POINTER
+    assert lib.hawk_rglru_step_gated(p, p, p, None, None, p, p, 32, p, None, p, 1, 64, 0, 0, None) \
+        == E.HAWK_ERR_BAD_SHAPE
+    # gate projections
+    assert lib.hawk_gate_proj_fwd(p, p, None, p, None, p, p, 4, 1024, 2, 0, 1, 0, None) == E.HAWK_ERR_BAD_SHAPE
+    assert lib.hawk_gate_proj_fwd(p, None, None, p, None, p, p, 4, 512, 4, 0, 1, 0, None) == E.HAWK_ERR_NULL_POINTER
+    assert lib.hawk_gate_proj_fwd(p, p, None, p, None, p, p, 0, 512, 4, 0, 1, 0, None) == E.HAWK_ERR_BAD_SHAPE
+    assert lib.hawk_gate_proj_fwd(p, p, None, p, None, p, p, 4, 512, 4, 0, 9, 0, None) == E.HAWK_ERR_BAD_DTYPE
+    assert lib.hawk_gate_proj_bwd_input(p, p, p, p, None, p + 4, 4, 512, 4, 0, 1, 0, None) == E.HAWK_ERR_ALIGNMENT
+    assert lib.hawk_gate_proj_bwd_weights(p, p, p, p, None, p, None, 4, 512, 4, 0, 0, None, 0, None) \
+        == E.HAWK_ERR_WORKSPACE
+    assert lib.hawk_gate_proj_bwd_weights(p, p, p, p, None, p, None, 4, 512, 4, 0, 0, p, 16, None) \
+        == E.HAWK_ERR_WORKSPACE
+    assert lib.hawk_gate_proj_bwd_weights_workspace_bytes(32768, 2560, 10) > 0
+    assert lib.hawk_gate_proj_bwd_weights_workspace_bytes(32768, 2560, 7) == 0
