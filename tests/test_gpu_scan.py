@@ -241,3 +241,46 @@ def test_full_benchmark_shapes_bf16(B, T, D, lo, hi):
     # linearity over ALL channels: h(2x) == 2 h(x) exactly in bf16 (power-of-two scaling)
     h2 = capi.scan_fwd((x.float() * 2).to(torch.bfloat16), xg, ag, lam_d, ws)
     assert torch.equal(h2.float(), h.float() * 2)
+
+
+def test_scan_launches_replay_correctly_from_a_hip_graph():
+    """Forward, backward and the gated pair captured once and replayed several times, with
+    eager launches on the same workspace in between; every replay must reproduce the eager
+    result bit for bit (the launch epoch lives in the workspace, not in the captured arguments)."""
+    B, T, D = 2, 1500, 256
+    x, xg, ag, lam, gout = make_scan_inputs(B, T, D, seed=21)
+    dev = [capi.to_dev(a, "bf16") for a in (x, xg, ag, gout)]
+    lam_d = capi.to_dev(lam, "f32")
+    wide = torch.randn(B, T, 2 * D, device="cuda").to(torch.bfloat16)
+    y = wide[..., D:]
+    ws = capi.new_workspace(B, T, D, "bf16")
+
+    def run():
+        h = capi.scan_fwd(dev[0], dev[1], dev[2], lam_d, ws)
+        g = capi.scan_bwd(dev[0], dev[1], dev[2], lam_d, h, dev[3], ws)
+        out, hg, hl = capi.scan_gated_fwd(dev[0], dev[1], dev[2], lam_d, y, ws=ws)
+        gg = capi.scan_gated_bwd(dev[0], dev[1], dev[2], lam_d, y, hg, dev[3], ws=ws)
+        return (h, *g, out, hg, hl, *gg)
+
+    eager = [t.clone() for t in run()]
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        run()
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        captured = run()
+    for rep in range(4):
+        for t in captured:
+            t.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        for a, b in zip(captured, eager):
+            assert torch.equal(a, b), rep
+        again = run()  # eager launches between replays move the workspace's epoch along
+        torch.cuda.synchronize()
+        for a, b in zip(again, eager):
+            assert torch.equal(a, b), rep
+    assert capi.workspace_flag(ws) == 0
