@@ -59,6 +59,7 @@ struct ScanWsPtrs {
     unsigned long long* agg_p; // [nseg][B][D] tile aggregate: product of alpha
     unsigned long long* agg_h; // [nseg][B][D] tile aggregate: state from zero
     float* dlam_part;          // [nseg][B][D] per-tile partial sums for dLambda
+    int lookback;              // distance between checkpoints of the carry chain (power of two)
 };
 
 __device__ __forceinline__ void publish(unsigned long long* p, uint32_t tag, float v) {
@@ -71,20 +72,22 @@ __device__ __forceinline__ bool try_read(const unsigned long long* p, uint32_t t
     return (uint32_t)(w >> 32) == tag;
 }
 
-// Every kLookback-th chain position is a checkpoint: it publishes the inclusive state at
+// Every lookback-th chain position is a checkpoint: it publishes the inclusive state at
 // its end; every other position publishes only its own aggregate.  A tile reads the
 // aggregates of its predecessors back to the nearest checkpoint, plus that checkpoint's
 // inclusive state, all in parallel (one predecessor per wave), and folds them oldest
-// first.  The order of the floating-point operations is fixed by the position alone,
-// never by timing, so results are bitwise reproducible, and the serial dependency runs
-// over checkpoints only (nseg / kLookback hops of one memory round trip each).
-#ifndef HAWK_LOOKBACK
-#define HAWK_LOOKBACK 4
-#endif
-constexpr int kLookback = HAWK_LOOKBACK;
+// first.  The order of the floating-point operations is fixed by the position and the
+// launch's shape alone, never by timing, so results are bitwise reproducible, and the serial
+// dependency runs over checkpoints only (nseg / lookback hops of one memory round trip each).
+// The distance is chosen per launch: 4 when there are enough independent chains (B x channel
+// tiles) to keep the memory system busy while each chain waits on its hops, 8 when there are
+// few and the hops themselves set the pace (one long sequence of a narrow model: 8 chains run
+// 22 % faster, 16 chains 4 %); with 60 or more chains the wider window costs 2-3 % instead.
+constexpr int kMaxLookback = 8;
+constexpr int kFewChains = 24;
 
-__device__ __forceinline__ bool is_checkpoint(int pos) { return (pos % kLookback) == 0; }
-__device__ __forceinline__ int checkpoint_before(int pos) { return ((pos - 1) / kLookback) * kLookback; }
+__device__ __forceinline__ bool is_checkpoint(int pos, int lookback) { return (pos & (lookback - 1)) == 0; }
+__device__ __forceinline__ int checkpoint_before(int pos, int lookback) { return (pos - 1) & ~(lookback - 1); }
 
 // One 64-bit atomic hands out the tile's position in the chain (ticket) together with the
 // launch tag, so a tile only ever waits for tiles that have already started.  The tile
@@ -110,7 +113,7 @@ __device__ __forceinline__ void take_ticket(unsigned long long* ctrl, uint32_t t
 
 // Carry into chain position `pos` for the V channels of this lane.
 //   tot_p/tot_h  aggregate of this whole tile (every wave holds it)
-//   s_prev       LDS [kLookback][CT] staging of the predecessors' words
+//   s_prev       LDS [kMaxLookback][CT] staging of the predecessors' words
 // Wave 0 publishes the tile's own word; wave k (k < number of predecessors) fetches
 // predecessor pos-1-k; after one barrier every wave folds the staged words.
 template <int V, int NW>
@@ -118,10 +121,10 @@ __device__ __forceinline__ void exchange_carry(const ScanWsPtrs& ws, int pos, in
                                                size_t stride, uint32_t tag, int w, int lane,
                                                const float (&tot_p)[V], const float (&tot_h)[V],
                                                float2 (*s_prev)[kWave * V], float (&cin)[V]) {
-    static_assert(kLookback % NW == 0 || NW % kLookback == 0, "waves must tile the look-back window");
+    const int lookback = ws.lookback;
     const bool publishes = pos + 1 < nseg;
     const size_t idx_self = idx_pos0 + (size_t)pos * stride;
-    if (w == 0 && publishes && !is_checkpoint(pos)) {
+    if (w == 0 && publishes && !is_checkpoint(pos, lookback)) {
 #pragma unroll
         for (int v = 0; v < V; ++v) {
             publish(ws.agg_p + idx_self + v, tag, tot_p[v]);
@@ -129,8 +132,9 @@ __device__ __forceinline__ void exchange_carry(const ScanWsPtrs& ws, int pos, in
         }
         asm volatile("" ::: "memory");
     }
-    const int npred = (pos > 0) ? pos - checkpoint_before(pos) : 0;
-    for (int k = w; k < npred; k += NW) {
+    const int npred = (pos > 0) ? pos - checkpoint_before(pos, lookback) : 0;
+    static_assert(NW >= kMaxLookback, "one wave per predecessor");
+    if (const int k = w; k < npred) {
         const int j = pos - 1 - k;
         const size_t idx = idx_pos0 + (size_t)j * stride;
         const bool cp = (k == npred - 1);
@@ -173,7 +177,7 @@ __device__ __forceinline__ void exchange_carry(const ScanWsPtrs& ws, int pos, in
             cin[v] = fmaf(a.x, cin[v], a.y);
         }
     }
-    if (w == 0 && publishes && is_checkpoint(pos)) {
+    if (w == 0 && publishes && is_checkpoint(pos, lookback)) {
 #pragma unroll
         for (int v = 0; v < V; ++v) publish(ws.incl + idx_self + v, tag, fmaf(tot_p[v], cin[v], tot_h[v]));
     }
@@ -394,7 +398,7 @@ __global__ __launch_bounds__(NW * kWave, HAWK_FWD_WAVES_PER_SIMD) void rglru_sca
     constexpr int CT = kWave * V;
     constexpr int TS = NW * TC;
     __shared__ float2 s_agg[NW][CT];
-    __shared__ float2 s_prev[kLookback][CT];
+    __shared__ float2 s_prev[kMaxLookback][CT];
     __shared__ uint32_t s_ticket[2];
 
     uint32_t ticket = blockIdx.x, tag = 0;
@@ -669,7 +673,7 @@ __global__ __launch_bounds__(NW * kWave, HAWK_BWD_WAVES_PER_SIMD) void rglru_sca
     constexpr int CT = kWave * V;
     constexpr int TS = NW * TC;
     __shared__ float2 s_agg[NW][CT];
-    __shared__ float2 s_prev[kLookback][CT];
+    __shared__ float2 s_prev[kMaxLookback][CT];
     __shared__ float s_dl[NW][CT];
     __shared__ uint32_t s_ticket[2];
 
@@ -798,9 +802,17 @@ WsLayout layout_for(int B, int D, int nseg_chain, int nseg_dlam) {
     l.total = align_up(l.off_dlam + (size_t)nseg_dlam * B * D * sizeof(float), 256);
     return l;
 }
-ScanWsPtrs carve(void* ws, const WsLayout& l) {
+int lookback_for(int B, int nct) {
+#ifdef HAWK_LOOKBACK
+    return HAWK_LOOKBACK;
+#else
+    return (long long)B * nct <= kFewChains ? kMaxLookback : 4;
+#endif
+}
+ScanWsPtrs carve(void* ws, const WsLayout& l, int lookback) {
     char* p = static_cast<char*>(ws);
     ScanWsPtrs r;
+    r.lookback = lookback;
     r.ctrl = reinterpret_cast<unsigned long long*>(p);
     r.incl = reinterpret_cast<unsigned long long*>(p + l.off_incl);
     r.agg_p = reinterpret_cast<unsigned long long*>(p + l.off_aggp);
@@ -867,10 +879,11 @@ int scan_fwd_impl(const void* x, const void* xg, const void* ag, const float* la
     const int nseg = ceil_div(T, s.rows());
     const int nct = ceil_div(D, s.chans());
     ScanWsPtrs p = {};
+    p.lookback = 4;
     if (nseg > 1) {
         const WsLayout l = layout_for(B, D, nseg, 0);
         if (ws == nullptr || ws_bytes < l.total) return HAWK_ERR_WORKSPACE;
-        p = carve(ws, l);
+        p = carve(ws, l, lookback_for(B, nct));
     }
     if (in_dtype == HAWK_DTYPE_BF16) {
         if (s.V == 2)
@@ -900,7 +913,7 @@ int scan_bwd_impl(const void* x, const void* xg, const void* ag, const float* la
     const int nct = ceil_div(D, s.chans());
     const WsLayout l = layout_for(B, D, nseg, nseg);
     if (ws == nullptr || ws_bytes < l.total) return HAWK_ERR_WORKSPACE;
-    const ScanWsPtrs p = carve(ws, l);
+    const ScanWsPtrs p = carve(ws, l, lookback_for(B, nct));
     int rc;
     if (in_dtype == HAWK_DTYPE_BF16) {
         if (s.V == 2)

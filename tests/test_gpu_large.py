@@ -2,9 +2,11 @@
 
 Each case replicates one slab of random data along the batch (or row) axis until a single
 operand passes 2^32 bytes, runs the entry point on the whole thing, and compares every replica
-bit for bit with the same entry point run on the one slab alone (well below 2^31 bytes).  The
-kernels treat batch rows independently and deterministically, so any difference is an address
-that wrapped.
+bit for bit with replica 0 and with the same entry point run on the one slab alone (well below
+2^31 bytes).  The kernels treat batch rows independently and deterministically, so any
+difference is an address that wrapped.  (The scans fold the carries of a launch with few
+independent chains in wider groups, so against the single slab they are allowed the last bit
+of a bf16 value; replicas of one launch must still agree exactly.)
 """
 
 import numpy as np
@@ -25,9 +27,14 @@ def _replicated(slab):
     return big
 
 
-def _assert_all_replicas_equal(big, one, name):
-    for b in range(B):
-        assert torch.equal(big[b], one[0]), (name, b)
+def _assert_all_replicas_equal(big, one, name, exact=True):
+    if exact:
+        assert torch.equal(big[0], one[0]), name
+    else:
+        a, b = big[0].float(), one[0].float()
+        assert float(((a - b).abs() / (b.abs() + 1e-3)).max()) <= 2.0**-7, name
+    for b in range(1, B):
+        assert torch.equal(big[b], big[0]), (name, b)
 
 
 @pytest.fixture(scope="module")
@@ -47,12 +54,12 @@ def test_scan_forward_and_backward_past_4gib(slab):
     ws = capi.new_workspace(B, T, D, "bf16")
     H = capi.scan_fwd(X, XG, AG, lam, ws)
     torch.cuda.synchronize()
-    _assert_all_replicas_equal(H, h1, "h")
+    _assert_all_replicas_equal(H, h1, "h", exact=False)
     G = capi.scan_bwd(X, XG, AG, lam, H, GO, ws)
     torch.cuda.synchronize()
     assert capi.workspace_flag(ws) == 0
     for name, big, one in zip(("dx", "dx_rg_lru", "da_rg_lru"), G, g1):
-        _assert_all_replicas_equal(big, one, name)
+        _assert_all_replicas_equal(big, one, name, exact=False)
     # dLambda sums over the batch: B equal contributions (fp32 sums in a different order)
     assert float((G[3] - g1[3] * B).abs().max()) < 1e-4 * float(g1[3].abs().max()) * B
 
@@ -65,16 +72,16 @@ def test_gated_scan_past_4gib(slab):
     ws = capi.new_workspace(B, T, D, "bf16")
     OUT, H, LAST = capi.scan_gated_fwd(X, XG, AG, lam, Y, ws=ws)
     torch.cuda.synchronize()
-    _assert_all_replicas_equal(OUT, out1, "out")
-    _assert_all_replicas_equal(H, h1, "h")
-    _assert_all_replicas_equal(LAST, last1, "h_last")
+    _assert_all_replicas_equal(OUT, out1, "out", exact=False)
+    _assert_all_replicas_equal(H, h1, "h", exact=False)
+    _assert_all_replicas_equal(LAST, last1, "h_last", exact=False)
     del OUT
     G = capi.scan_gated_bwd(X, XG, AG, lam, Y, H, GO, ws=ws)
     torch.cuda.synchronize()
     assert capi.workspace_flag(ws) == 0
     for name, big, one in zip(("dx", "dx_rg_lru", "da_rg_lru"), G[:3], g1[:3]):
-        _assert_all_replicas_equal(big, one, name)
-    _assert_all_replicas_equal(G[4], g1[4], "dy")
+        _assert_all_replicas_equal(big, one, name, exact=False)
+    _assert_all_replicas_equal(G[4], g1[4], "dy", exact=False)
 
 
 def test_conv1d_past_4gib(slab):
