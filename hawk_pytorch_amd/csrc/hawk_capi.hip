@@ -221,7 +221,8 @@ int hawk_gate_proj_fwd(const void* x, const void* w_i, const float* b_i, const v
     if (!x || !w_i || !w_a || !x_rg_lru || !a_rg_lru) return HAWK_ERR_NULL_POINTER;
     if (!dtype_ok(x_dtype) || !dtype_ok(w_dtype) || !dtype_ok(out_dtype)) return HAWK_ERR_BAD_DTYPE;
     if (M < 1 || !hawk_gate_proj_supported(D, num_blocks)) return HAWK_ERR_BAD_SHAPE;
-    if (!aligned16(x) || !aligned16(x_rg_lru) || !aligned16(a_rg_lru)) return HAWK_ERR_ALIGNMENT;
+    if (!aligned16(x) || !aligned16(x_rg_lru) || !aligned16(a_rg_lru) || !aligned16(w_i) || !aligned16(w_a))
+        return HAWK_ERR_ALIGNMENT;
     return hawk::gate_proj_fwd(x, w_i, b_i, w_a, b_a, x_rg_lru, a_rg_lru, M, D, num_blocks, x_dtype, w_dtype,
                                out_dtype, as_stream(stream));
 }

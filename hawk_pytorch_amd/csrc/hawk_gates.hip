@@ -43,6 +43,10 @@ constexpr int kGateThreads = 1024;             // 16 waves
 constexpr int kARowBytes = kGroup * 2 + 16;    // bf16 row + pad: 8 lanes' 16-byte reads cover all banks
 constexpr int kATileBytes = kTileRows * kARowBytes;
 constexpr int kNumCU = 256;
+// Row counts up to this one take the forward kernel that is cut by output columns.
+#ifndef HAWK_GATE_SMALL_M
+#define HAWK_GATE_SMALL_M 512
+#endif
 
 __device__ __forceinline__ float elem_to_f32(float v) { return v; }
 __device__ __forceinline__ float elem_to_f32(bf16_t v) { return __uint_as_float((uint32_t)v.bits << 16); }
@@ -107,10 +111,62 @@ struct Row8<float> {
     }
 };
 
+// Eight consecutive output columns of four consecutive input channels of a weight matrix, as
+// they arrive from memory, and the same 32 values as bf16 regrouped by output column
+// (column e: input channels 0..3 in two dwords), which is what the LDS transposition writes.
+template <typename WT>
+struct WeightQuad;
+template <>
+struct WeightQuad<bf16_t> {
+    static constexpr int kDwords = 16;
+    u32x4 q[4];
+    __device__ __forceinline__ void clear() {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) q[r] = u32x4{0u, 0u, 0u, 0u};
+    }
+    __device__ __forceinline__ void load(const bf16_t* p, size_t row_stride) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) q[r] = *reinterpret_cast<const u32x4*>(p + r * row_stride);
+    }
+    __device__ __forceinline__ u32x2 column(int e) const {
+        const uint32_t a = q[0][e / 2], b = q[1][e / 2], c = q[2][e / 2], d = q[3][e / 2];
+        if (e % 2 == 0) return u32x2{(a & 0xffffu) | (b << 16), (c & 0xffffu) | (d << 16)};
+        return u32x2{(a >> 16) | (b & 0xffff0000u), (c >> 16) | (d & 0xffff0000u)};
+    }
+};
+template <>
+struct WeightQuad<float> {
+    static constexpr int kDwords = 32;
+    f32x4 q[4][2];
+    __device__ __forceinline__ void clear() {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) q[r][0] = q[r][1] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    }
+    __device__ __forceinline__ void load(const float* p, size_t row_stride) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            q[r][0] = *reinterpret_cast<const f32x4*>(p + r * row_stride);
+            q[r][1] = *reinterpret_cast<const f32x4*>(p + r * row_stride + 4);
+        }
+    }
+    __device__ __forceinline__ u32x2 column(int e) const {
+        return u32x2{pack_bf16x2(q[0][e / 4][e % 4], q[1][e / 4][e % 4]),
+                     pack_bf16x2(q[2][e / 4][e % 4], q[3][e / 4][e % 4])};
+    }
+};
+
 __device__ __forceinline__ void store_out(unsigned char* p, float v, bf16_t*) {
     *reinterpret_cast<uint16_t*>(p) = to_bf16_bits(v);
 }
 __device__ __forceinline__ void store_out(unsigned char* p, float v, float*) { *reinterpret_cast<float*>(p) = v; }
+
+// LDS scratch of the forward kernel's weight transposition: [2 gates][256 columns][kPassK + 8] bf16.
+template <int BW>
+struct WeightStage {
+    static constexpr int kPassK = BW < 64 ? BW : 64;
+    static constexpr int kRowBytes = kPassK * 2 + 16;
+    static constexpr int kBytes = 2 * kGroup * kRowBytes;
+};
 
 template <typename XT, typename WT, typename OT, int BW>
 __global__ __launch_bounds__(kGateThreads, 1) void gate_proj_fwd_kernel(
@@ -164,31 +220,53 @@ __global__ __launch_bounds__(kGateThreads, 1) void gate_proj_fwd_kernel(
     load_tile(1, rb);
     __builtin_amdgcn_sched_barrier(0);  // the first tiles travel while the weights are fetched
 
-    // ---- the weights: 8 strided loads per k-step and lane (coalesced across lanes), issued
-    //      four k-steps at a time so that they fit the registers left beside their own
-    //      destination; a group past the last block (D not a multiple of 256) reads block
-    //      nb-1 and zeroes it
-    const float live = (h < nb) ? 1.0f : 0.0f;
-    const rsrc_t wres = make_rsrc(wsel, (uint32_t)((size_t)nb * BW * BW * sizeof(WT)));
-    const uint32_t wlane = (uint32_t)((((size_t)min(h, nb - 1) * BW + khalf) * BW + n) * sizeof(WT));
+    // ---- the weights.  A lane's B operand is 8 consecutive input channels of one output
+    //      column, which lie bw elements apart in memory, so they are fetched the way memory
+    //      wants it (a thread reads 8 consecutive output columns of 4 consecutive input
+    //      channels, 16 or 32 bytes each) and transposed through LDS with 8-byte writes, up to
+    //      64 input channels of both gates per pass.  A group past the last block (D not a
+    //      multiple of 256) gets zeros.
+    constexpr int kPassK = WeightStage<BW>::kPassK, kTRowBytes = WeightStage<BW>::kRowBytes;
+    constexpr int kQuads = kPassK / 4, kTasks = 2 * kQuads * (kGroup / 8);
     bf16x8 bfrag[KS];
-    constexpr int kWBatch = KS < 4 ? KS : 4;
+    {
+        const int tgate = tid / (kQuads * (kGroup / 8)), trem = tid % (kQuads * (kGroup / 8));
+        const int tkq = trem % kQuads, tn8 = (trem / kQuads) * 8;  // thread -> (4 input channels, 8 output columns)
+        const int tblk = tn8 / BW;
+        const bool twrites = tid < kTasks;
+        const bool tloads = twrites && group * G + tblk < nb;
+        const WT* tsrc_w = (tgate ? w_a : w_i) + ((size_t)(group * G + tblk) * BW + 4 * tkq) * BW + (tn8 - tblk * BW);
+        unsigned char* tdst = smem + (tgate * kGroup + tn8) * kTRowBytes + tkq * 8;
+        const unsigned char* tsrc = smem + ((g * kGroup + 32 * c + col) * kTRowBytes + khalf * 2);
+        // as many passes are kept in flight as fit in 64 registers; the registers of the
+        // matrix operands fill up as those of the raw rows drain
+        constexpr int NP = BW / kPassK;
+        constexpr int kAhead = 64 / WeightQuad<WT>::kDwords < NP ? 64 / WeightQuad<WT>::kDwords : NP;
+        WeightQuad<WT> raw[NP];
 #pragma unroll
-    for (int s0 = 0; s0 < KS; s0 += kWBatch) {
-        float v[kWBatch][8];
+        for (int pass = 0; pass < NP; ++pass) raw[pass].clear();
+        if (tloads) {
 #pragma unroll
-        for (int j = 0; j < kWBatch; ++j)
-#pragma unroll
-            for (int e = 0; e < 8; ++e)
-                v[j][e] = load_weight(wres, wlane, (uint32_t)((16 * (s0 + j) + e) * BW * sizeof(WT)),
-                                      static_cast<const WT*>(nullptr));
-#pragma unroll
-        for (int j = 0; j < kWBatch; ++j) {
-            const u32x4 packed = {pack_bf16x2(live * v[j][0], live * v[j][1]), pack_bf16x2(live * v[j][2], live * v[j][3]),
-                                  pack_bf16x2(live * v[j][4], live * v[j][5]), pack_bf16x2(live * v[j][6], live * v[j][7])};
-            bfrag[s0 + j] = __builtin_bit_cast(bf16x8, packed);
+            for (int pass = 0; pass < kAhead; ++pass) raw[pass].load(tsrc_w + (size_t)pass * kPassK * BW, BW);
         }
-        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int pass = 0; pass < NP; ++pass) {
+            u32x2 cols[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) cols[e] = raw[pass].column(e);
+            if (pass + kAhead < NP && tloads)
+                raw[pass + kAhead].load(tsrc_w + (size_t)(pass + kAhead) * kPassK * BW, BW);
+            if (pass > 0) __syncthreads();  // the previous pass has been read
+            if (twrites) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) *reinterpret_cast<u32x2*>(tdst + e * kTRowBytes) = cols[e];
+            }
+            __syncthreads();
+#pragma unroll
+            for (int s2 = 0; s2 < kPassK / 16; ++s2)
+                bfrag[pass * (kPassK / 16) + s2] = *reinterpret_cast<const bf16x8*>(tsrc + 32 * s2);
+        }
+        __syncthreads();
     }
 
     stage_tile(0, ra);
@@ -245,6 +323,104 @@ __global__ __launch_bounds__(kGateThreads, 1) void gate_proj_fwd_kernel(
         step(it, 0, rb);
         if (worker + (it + 1) * nworkers >= ntiles) break;
         step(it + 1, 1, ra);
+    }
+}
+
+// ---------------------------------------------------------------------------------------
+// The same projections for few rows (decode: one row per sequence).  With M/32 row tiles the
+// kernel above keeps at most (M/32) x (D/256) compute units busy and each of them spends most
+// of its time fetching a 256-column slice of the weights for a single tile.  Here the work is
+// cut the other way: a workgroup of 8 waves owns 32 output columns of one gate.  It reads
+// that bw x 32 slice of the weights once with 16-byte accesses along the rows of the weight
+// matrix (64 contiguous bytes each), transposes it through LDS so that a lane finds its 8
+// consecutive input channels of one output column in 16 contiguous bytes, and every wave takes
+// its B operands from there.  Wave w then walks over row tiles w, w + 8 x gridDim.y, ...: A
+// operands come straight from memory (a lane's 8 consecutive input channels are 16 contiguous
+// bytes), results leave from the accumulator registers (64 contiguous bytes per row and half
+// wave, which is acceptable while M is small).
+// ---------------------------------------------------------------------------------------
+constexpr int kSmallWaves = 8;
+
+template <typename XT, typename WT, typename OT, int BW>
+__global__ __launch_bounds__(kSmallWaves* kWave, sizeof(XT) == 2 ? 4 : 2) void gate_proj_fwd_small_kernel(
+    const XT* __restrict__ x, const WT* __restrict__ w_i, const float* __restrict__ b_i,
+    const WT* __restrict__ w_a, const float* __restrict__ b_a, OT* __restrict__ out_i, OT* __restrict__ out_a,
+    int M, int D, int nb, int ntiles) {
+    constexpr int KS = BW / 16;
+    constexpr int kWRowBytes = BW * 2 + 16;        // one output column's bw weights + pad
+    __shared__ __align__(16) unsigned char sW[32 * kWRowBytes];
+    const int tid = threadIdx.x;
+    const int lane = tid & (kWave - 1);
+    const int w = __builtin_amdgcn_readfirstlane(tid / kWave);
+    const int ncol = D / 32;                       // D is a multiple of bw, bw a multiple of 32
+    const int g = (int)blockIdx.x / ncol;          // gate
+    const int c0 = ((int)blockIdx.x - g * ncol) * 32;
+    const int h = c0 / BW;                         // a 32-column tile never straddles two blocks
+    const int col = lane & 31, khalf = 8 * (lane >> 5);
+    const WT* wsel = g ? w_a : w_i;
+    const float* bsel = g ? b_a : b_i;
+    OT* out = g ? out_a : out_i;
+    int rt = (int)blockIdx.y * kSmallWaves + w;
+    const int rstep = (int)gridDim.y * kSmallWaves;
+
+    // A operands of the first row tile travel while the weights are staged
+    const XT* xcol = x + (size_t)h * BW + khalf;
+    u32x4 abf[KS];
+    auto load_rows = [&](int t) {
+        const int row = t * kTileRows + col;
+        const bool ok = t < ntiles && row < M;
+        const XT* p = xcol + (ok ? (size_t)row * D : 0);
+#pragma unroll
+        for (int s = 0; s < KS; ++s) {
+            Row8<XT> r;
+            r.load(p + 16 * s, ok);
+            abf[s] = r.as_bf16();
+        }
+    };
+    load_rows(rt);
+    __builtin_amdgcn_sched_barrier(0);
+
+    // weights: thread -> (4 input channels, 8 consecutive output columns), written transposed
+    if (tid < BW) {
+        const int tkq = tid % (BW / 4), tn8 = (tid / (BW / 4)) * 8;
+        WeightQuad<WT> raw;
+        raw.load(wsel + ((size_t)h * BW + 4 * tkq) * BW + (c0 - h * BW) + tn8, BW);
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+            *reinterpret_cast<u32x2*>(sW + (tn8 + e) * kWRowBytes + tkq * 8) = raw.column(e);
+    }
+    const float bias = bsel != nullptr ? bsel[c0 + col] : 0.0f;
+    __syncthreads();
+    // B operands stay in LDS and are read per use: the registers go to the A operands, and
+    // two workgroups fit a compute unit (one with fp32 activations, whose rows take twice the
+    // registers while they travel)
+    const unsigned char* bsrc = sW + col * kWRowBytes + khalf * 2;
+
+    for (; rt < ntiles; rt += rstep) {
+        f32x16 acc = {};
+        constexpr int kBatch = KS < 4 ? KS : 4;
+#pragma unroll
+        for (int s0 = 0; s0 < KS; s0 += kBatch) {
+            bf16x8 b[kBatch];
+#pragma unroll
+            for (int j = 0; j < kBatch; ++j) b[j] = *reinterpret_cast<const bf16x8*>(bsrc + 32 * (s0 + j));
+#pragma unroll
+            for (int j = 0; j < kBatch; ++j)
+                acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, abf[s0 + j]), b[j], acc, 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        if (rt + rstep < ntiles) load_rows(rt + rstep);
+        __builtin_amdgcn_sched_barrier(0);
+        // accumulator register r of a lane is row 8 (r / 4) + 4 (lane / 32) + r % 4, column lane % 32
+        const int row0 = rt * kTileRows + 4 * (lane >> 5);
+        OT* obase = out + (size_t)row0 * D + c0 + col;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int m = 8 * (r / 4) + (r % 4);
+            if (row0 + m < M)
+                store_out(reinterpret_cast<unsigned char*>(obase + (size_t)m * D), acc[r] + bias,
+                          static_cast<OT*>(nullptr));
+        }
     }
 }
 
@@ -588,10 +764,24 @@ int launch_gate_fwd(const void* x, const void* w_i, const float* b_i, const void
                     void* out_a, int M, int D, int nb, hipStream_t st) {
     const int ngroups = ceil_div(D, kGroup);
     const int ntiles = ceil_div(M, kTileRows);
+    if (M <= HAWK_GATE_SMALL_M) {
+        // enough workgroups to give every compute unit a few waves; each wave keeps its weights
+        // for all the row tiles it walks over
+        const int ncolblocks = 2 * (D / 32);
+        int rsplit = ceil_div(8 * kNumCU, ncolblocks * kSmallWaves);
+        const int max_split = ceil_div(ntiles, kSmallWaves);
+        if (rsplit > max_split) rsplit = max_split;
+        hipLaunchKernelGGL((gate_proj_fwd_small_kernel<XT, WT, OT, BW>), dim3((unsigned)ncolblocks, (unsigned)rsplit),
+                           dim3(kSmallWaves * kWave), 0, st, static_cast<const XT*>(x), static_cast<const WT*>(w_i),
+                           b_i, static_cast<const WT*>(w_a), b_a, static_cast<OT*>(out_i), static_cast<OT*>(out_a), M,
+                           D, nb, ntiles);
+        return hipGetLastError() == hipSuccess ? HAWK_OK : HAWK_ERR_LAUNCH;
+    }
     int nworkers = kNumCU / ngroups;
     if (nworkers < 1) nworkers = 1;
     if (nworkers > ntiles) nworkers = ntiles;
-    const size_t smem = 2 * kATileBytes + (size_t)kTileRows * (2 * kGroup * sizeof(OT) + 16);
+    size_t smem = 2 * kATileBytes + (size_t)kTileRows * (2 * kGroup * sizeof(OT) + 16);
+    if (smem < (size_t)WeightStage<BW>::kBytes) smem = WeightStage<BW>::kBytes;
     auto kernel = gate_proj_fwd_kernel<XT, WT, OT, BW>;
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                             (int)smem) != hipSuccess)

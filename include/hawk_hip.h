@@ -201,7 +201,9 @@ int hawk_gate_proj_supported(int D, int num_blocks);
  * hawk/external.py:224-233).  x [M,D] has x_dtype; w_i, w_a [num_blocks, bw, bw] have
  * w_dtype; b_i, b_a [D] are fp32 or NULL; the outputs [M,D] have out_dtype.  x and the
  * weights are rounded to bf16 in registers (what bf16 autocast does to this einsum); the
- * sums and the bias add are fp32. */
+ * sums and the bias add are fp32.  x, the weights and the outputs must be 16-byte aligned
+ * (HAWK_ERR_ALIGNMENT otherwise).  Row counts up to 512 (decode) run a variant that is cut
+ * by output columns instead of rows; results are the same sums in the same order. */
 int hawk_gate_proj_fwd(const void* x, const void* w_i, const float* b_i, const void* w_a,
                        const float* b_a, void* x_rg_lru, void* a_rg_lru, int M, int D,
                        int num_blocks, int x_dtype, int w_dtype, int out_dtype, void* stream);

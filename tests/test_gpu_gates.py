@@ -69,6 +69,25 @@ def test_each_output_depends_only_on_its_own_block():
     assert not torch.equal(a0[:, 3 * 128:4 * 128], a1[:, 3 * 128:4 * 128])
 
 
+@pytest.mark.parametrize("D,nb", [(2560, 10), (512, 16), (768, 6)])
+@pytest.mark.parametrize("x_dtype,w_dtype,out_dtype", [("bf16", "bf16", "bf16"), ("f32", "f32", "f32"),
+                                                       ("bf16", "f32", "bf16")])
+def test_few_rows_and_many_rows_give_the_same_bits(D, nb, x_dtype, w_dtype, out_dtype):
+    """Up to 512 rows the forward runs a kernel cut by output columns (decode), above that the
+    one cut by rows; both add the same products in the same order, so the first rows of a
+    600-row call must equal a call on those rows alone, bit for bit, for every small M."""
+    rng = np.random.default_rng(17)
+    bw = D // nb
+    x = capi.to_dev(rng.standard_normal((600, D)), x_dtype)
+    wi = capi.to_dev(rng.standard_normal((nb, bw, bw)) / np.sqrt(bw), w_dtype)
+    wa = capi.to_dev(rng.standard_normal((nb, bw, bw)) / np.sqrt(bw), w_dtype)
+    bi, ba = capi.to_dev(rng.standard_normal(D), "f32"), capi.to_dev(rng.standard_normal(D), "f32")
+    big_i, big_a = capi.gate_proj_fwd(x, wi, bi, wa, ba, capi.TORCH_DTYPE[out_dtype])
+    for M in (1, 7, 32, 33, 256, 300, 512):
+        oi, oa = capi.gate_proj_fwd(x[:M].contiguous(), wi, bi, wa, ba, capi.TORCH_DTYPE[out_dtype])
+        assert torch.equal(oi, big_i[:M]) and torch.equal(oa, big_a[:M]), M
+
+
 def test_unsupported_shapes_are_refused():
     from hawk_pytorch_amd import _lib
     lib = _lib.load()

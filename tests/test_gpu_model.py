@@ -254,7 +254,7 @@ def test_model_gradients_match_a_pure_torch_model_of_the_same_weights(fused_epil
         ref_loss.backward()
     finally:
         hm.fused_linear_scan, hm.fused_linear_scan_gated, he.Conv1D.forward = old
-    assert abs(float(loss) - float(ref_loss)) < 1e-4
+    assert abs(float(loss.detach()) - float(ref_loss.detach())) < 1e-4
     for n, p in model.named_parameters():
         assert max_rel(capi.to_np(got[n]), capi.to_np(p.grad)) < 1e-3, n
 
