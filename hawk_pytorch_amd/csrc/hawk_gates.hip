@@ -27,6 +27,8 @@
 
 #include <stdint.h>
 
+#include <atomic>
+
 #include "hawk_device.h"
 
 namespace hawk {
@@ -759,6 +761,21 @@ __global__ void gate_proj_reduce_kernel(const float* __restrict__ part_w, const 
 
 inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
 
+// Raises a kernel's dynamic LDS limit once per device instead of on every launch.
+template <auto Kernel>
+bool allow_dynamic_lds(size_t bytes) {
+    static std::atomic<unsigned long long> done{0};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return false;
+    const unsigned long long bit = 1ull << (dev & 63);
+    if (done.load(std::memory_order_acquire) & bit) return true;
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(Kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                            (int)bytes) != hipSuccess)
+        return false;
+    done.fetch_or(bit, std::memory_order_release);
+    return true;
+}
+
 template <typename XT, typename WT, typename OT, int BW>
 int launch_gate_fwd(const void* x, const void* w_i, const float* b_i, const void* w_a, const float* b_a, void* out_i,
                     void* out_a, int M, int D, int nb, hipStream_t st) {
@@ -782,10 +799,8 @@ int launch_gate_fwd(const void* x, const void* w_i, const float* b_i, const void
     if (nworkers > ntiles) nworkers = ntiles;
     size_t smem = 2 * kATileBytes + (size_t)kTileRows * (2 * kGroup * sizeof(OT) + 16);
     if (smem < (size_t)WeightStage<BW>::kBytes) smem = WeightStage<BW>::kBytes;
-    auto kernel = gate_proj_fwd_kernel<XT, WT, OT, BW>;
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                            (int)smem) != hipSuccess)
-        return HAWK_ERR_LAUNCH;
+    constexpr auto kernel = gate_proj_fwd_kernel<XT, WT, OT, BW>;
+    if (!allow_dynamic_lds<kernel>(smem)) return HAWK_ERR_LAUNCH;
     hipLaunchKernelGGL(kernel, dim3((unsigned)nworkers, (unsigned)ngroups), dim3(kGateThreads), smem, st,
                        static_cast<const XT*>(x), static_cast<const WT*>(w_i), b_i, static_cast<const WT*>(w_a), b_a,
                        static_cast<OT*>(out_i), static_cast<OT*>(out_a), M, D, nb, ntiles);
@@ -821,12 +836,12 @@ int launch_gate_bwd_input(const void* dxg, const void* dag, const void* w_i, con
     if (nworkers < 1) nworkers = 1;
     if (nworkers > ntiles) nworkers = ntiles;
     const size_t smem = 4 * kATileBytes + 2 * (size_t)kTileRows * (kGroup * 4 + 16);
-    auto kernel = addend != nullptr ? gate_proj_bwd_input_kernel<GT, WT, DT, BW, true>
-                                    : gate_proj_bwd_input_kernel<GT, WT, DT, BW, false>;
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                            (int)smem) != hipSuccess)
+    constexpr auto with_addend = gate_proj_bwd_input_kernel<GT, WT, DT, BW, true>;
+    constexpr auto without = gate_proj_bwd_input_kernel<GT, WT, DT, BW, false>;
+    if (!(addend != nullptr ? allow_dynamic_lds<with_addend>(smem) : allow_dynamic_lds<without>(smem)))
         return HAWK_ERR_LAUNCH;
-    hipLaunchKernelGGL(kernel, dim3((unsigned)nworkers, (unsigned)ngroups), dim3(kGateThreads), smem, st,
+    hipLaunchKernelGGL(addend != nullptr ? with_addend : without, dim3((unsigned)nworkers, (unsigned)ngroups),
+                       dim3(kGateThreads), smem, st,
                        static_cast<const GT*>(dxg), static_cast<const GT*>(dag), static_cast<const WT*>(w_i),
                        static_cast<const WT*>(w_a), static_cast<const DT*>(addend), static_cast<DT*>(dx), M, D, nb,
                        ntiles);

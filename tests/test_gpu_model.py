@@ -305,6 +305,61 @@ def test_readme_model_config_bf16_autocast_training_step():
             assert cos > 0.99, (case, n, cos)
 
 
+def test_training_step_replays_from_a_hip_graph():
+    """Forward, backward (all fused kernels, their workspaces and reductions) and AdamW captured
+    once and replayed: losses and parameters must follow the eager run of the same steps.
+    Embedding and weight-gradient sums inside torch are not bit-reproducible, hence tolerances."""
+    cfg = hk.HawkConfig(vocab_size=1024, hidden_size=256, intermediate_size=512, num_hidden_layers=2,
+                        recurrent_size=256, num_blocks=4, conv_width=4)
+    ids = torch.randint(1, cfg.vocab_size, (2, 700), device="cuda", generator=torch.Generator("cuda").manual_seed(8))
+
+    def make():
+        torch.manual_seed(8)
+        model = hk.HawkModel(cfg).cuda()
+        _randomise_zero_inits(model)
+        return model, torch.optim.AdamW(model.parameters(), lr=1e-3, capturable=True)
+
+    def step(model, opt):
+        with torch.autocast(device_type="cuda", dtype=torch.bfloat16):
+            loss = model(ids, ids)
+        loss.backward()
+        opt.step()
+        return loss
+
+    warm, replays = 3, 4
+    eager_model, eager_opt = make()
+    eager_losses = []
+    for _ in range(warm + replays):
+        eager_losses.append(float(step(eager_model, eager_opt).detach()))
+        eager_opt.zero_grad(set_to_none=True)
+
+    model, opt = make()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(warm):
+            step(model, opt)
+            opt.zero_grad(set_to_none=True)
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        static_loss = step(model, opt)
+    graph_losses = []
+    for _ in range(replays):
+        graph.replay()
+        torch.cuda.synchronize()
+        graph_losses.append(float(static_loss.detach()))
+    assert graph_losses[-1] < graph_losses[0]  # it trains
+    for a, b in zip(graph_losses, eager_losses[warm:]):
+        assert abs(a - b) < 2e-3 * abs(b), (graph_losses, eager_losses)
+    for (n, p), (_, q) in zip(model.named_parameters(), eager_model.named_parameters()):
+        assert torch.isfinite(p).all(), n
+        # AdamW moves every weight by about lr per step whatever the gradient's size, so a sign
+        # flip of a near-zero gradient is worth 2 lr; seven steps bound the drift
+        assert float((p - q).abs().max()) < 2 * 1e-3 * (warm + replays), n
+        assert float((p - q).abs().mean()) < 1e-4, n
+
+
 def test_torch_compile_traces_the_ops_without_graph_breaks():
     (x, xg, ag), lam, gout = _leaves(1, 70, 64, "f32", seed=4)
     conv = hk.Conv1D(64, 4).cuda()
