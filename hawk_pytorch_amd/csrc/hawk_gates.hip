@@ -46,6 +46,9 @@ constexpr int kARowBytes = kGroup * 2 + 16;    // bf16 row + pad: 8 lanes' 16-by
 constexpr int kATileBytes = kTileRows * kARowBytes;
 constexpr int kNumCU = 256;
 // Row counts up to this one take the forward kernel that is cut by output columns.
+#ifndef HAWK_GATE_MIN_SPLIT_TILES
+#define HAWK_GATE_MIN_SPLIT_TILES 4
+#endif
 #ifndef HAWK_GATE_SMALL_M
 #define HAWK_GATE_SMALL_M 512
 #endif
@@ -872,8 +875,10 @@ int weight_splits(int M, int D) {
     const int ngroups = ceil_div(D, kGroup);
     int n = kNumCU / (2 * ngroups);
     if (n < 1) n = 1;
-    const int ntiles = ceil_div(M, kTileRows);
-    return n > ntiles ? ntiles : n;
+    // at least HAWK_GATE_MIN_SPLIT_TILES row tiles per split: every split costs a pass over its
+    // partial sums in the reduction
+    const int cap = (ceil_div(M, kTileRows) + HAWK_GATE_MIN_SPLIT_TILES - 1) / HAWK_GATE_MIN_SPLIT_TILES;
+    return n > cap ? cap : n;
 }
 
 template <typename XT, typename GT, int BW>
