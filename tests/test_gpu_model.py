@@ -353,6 +353,7 @@ def test_training_step_replays_from_a_hip_graph():
     for a, b in zip(graph_losses, eager_losses[warm:]):
         assert abs(a - b) < 2e-3 * abs(b), (graph_losses, eager_losses)
     for (n, p), (_, q) in zip(model.named_parameters(), eager_model.named_parameters()):
+        p, q = p.detach(), q.detach()
         assert torch.isfinite(p).all(), n
         # AdamW moves every weight by about lr per step whatever the gradient's size, so a sign
         # flip of a near-zero gradient is worth 2 lr; seven steps bound the drift
