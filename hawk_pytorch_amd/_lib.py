@@ -154,6 +154,13 @@ _workspaces: dict = {}
 
 
 def scan_workspace(dev: torch.device, nbytes: int) -> torch.Tensor:
+    if torch.cuda.is_current_stream_capturing():
+        # A captured launch gets a workspace of its own from the graph's memory pool, zeroed by a
+        # fill kernel that is part of the graph: the graph then depends on no buffer that eager
+        # code or another graph also uses, whatever stream it is replayed on and in whatever
+        # order graphs are replayed.  (A cached buffer created during a capture would hold
+        # nothing until that one graph had been replayed.)
+        return torch.zeros(max(nbytes, 256), dtype=torch.uint8, device=dev)
     key = (dev.index if dev.index is not None else torch.cuda.current_device(), stream_ptr(dev))
     ws = _workspaces.get(key)
     if ws is None or ws.numel() < nbytes:

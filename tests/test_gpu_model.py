@@ -361,6 +361,34 @@ def test_training_step_replays_from_a_hip_graph():
         assert float((p - q).abs().mean()) < 1e-4, n
 
 
+def test_captured_scans_own_their_workspace():
+    """Two graphs captured one after the other, the second replayed first: each captured scan
+    must carry its own zeroed carry workspace (a buffer first created while capturing graph A
+    would still be uninitialised when graph B runs)."""
+    g = torch.Generator(device="cuda").manual_seed(4)
+    B, T, D = 2, 1000, 256
+    x, xg, ag, x2 = (torch.randn(B, T, D, device="cuda", generator=g).to(torch.bfloat16) for _ in range(4))
+    lam = torch.randn(D, device="cuda", generator=g)
+    want_a = hk.fused_linear_scan(x, xg, ag, lam).clone()
+    want_b = hk.fused_linear_scan(x2, xg, ag, lam).clone()
+    torch.cuda.synchronize()
+    graph_a, graph_b = torch.cuda.CUDAGraph(), torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph_a):
+        got_a = hk.fused_linear_scan(x, xg, ag, lam)
+    with torch.cuda.graph(graph_b):
+        got_b = hk.fused_linear_scan(x2, xg, ag, lam)
+    for _ in range(2):
+        got_a.fill_(float("nan"))
+        got_b.fill_(float("nan"))
+        graph_b.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(got_b, want_b)
+        graph_a.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(got_a, want_a)
+        assert torch.equal(hk.fused_linear_scan(x, xg, ag, lam), want_a)  # eager launches in between
+
+
 def test_torch_compile_traces_the_ops_without_graph_breaks():
     (x, xg, ag), lam, gout = _leaves(1, 70, 64, "f32", seed=4)
     conv = hk.Conv1D(64, 4).cuda()
