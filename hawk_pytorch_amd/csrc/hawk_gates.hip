@@ -53,18 +53,8 @@ constexpr int kNumCU = 256;
 #define HAWK_GATE_SMALL_M 512
 #endif
 
-__device__ __forceinline__ float elem_to_f32(float v) { return v; }
-__device__ __forceinline__ float elem_to_f32(bf16_t v) { return __uint_as_float((uint32_t)v.bits << 16); }
-
-// Weight fetches go through a buffer resource (scalar base, one per-lane offset, scalar
-// per-access offset), with the default cache policy: every workgroup re-reads them.
-__device__ __forceinline__ float load_weight(rsrc_t r, uint32_t lane_bytes, uint32_t off_bytes, const float*) {
-    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, lane_bytes, off_bytes, kAuxDefault));
-}
-__device__ __forceinline__ float load_weight(rsrc_t r, uint32_t lane_bytes, uint32_t off_bytes, const bf16_t*) {
-    const uint16_t b = __builtin_bit_cast(uint16_t, __builtin_amdgcn_raw_buffer_load_b16(r, lane_bytes, off_bytes, kAuxDefault));
-    return __uint_as_float((uint32_t)b << 16);
-}
+// Weight fetches that go through a buffer resource (scalar base, one per-lane offset, scalar
+// per-access offset) use the default cache policy: every workgroup re-reads them.
 // eight consecutive weights as a bf16 MFMA operand (scaled by `live`, 0 or 1)
 __device__ __forceinline__ bf16x8_t load_weight8(rsrc_t r, uint32_t lane_bytes, uint32_t off_bytes, float live,
                                                  const float*) {
@@ -195,10 +185,7 @@ __global__ __launch_bounds__(kGateThreads, 1) void gate_proj_fwd_kernel(
     //      (lane % 32) and 8 consecutive input channels starting at 16 s + 8 (lane / 32)
     const int g = w >> 3, c = w & 7;
     const int blk = (32 * c) / BW;                 // block within the group
-    const int h = group * G + blk;                 // block of the layer
     const int col = lane & 31, khalf = 8 * (lane >> 5);
-    const int n = 32 * c - blk * BW + col;         // output column within the block
-    const WT* wsel = g ? w_a : w_i;
     const float* bsel = g ? b_a : b_i;
     const int ch = group * kGroup + 32 * c + col;  // channel of the layer
     const float bias = (bsel != nullptr && ch < D) ? bsel[ch] : 0.0f;
@@ -350,7 +337,7 @@ template <typename XT, typename WT, typename OT, int BW>
 __global__ __launch_bounds__(kSmallWaves* kWave, sizeof(XT) == 2 ? 4 : 2) void gate_proj_fwd_small_kernel(
     const XT* __restrict__ x, const WT* __restrict__ w_i, const float* __restrict__ b_i,
     const WT* __restrict__ w_a, const float* __restrict__ b_a, OT* __restrict__ out_i, OT* __restrict__ out_a,
-    int M, int D, int nb, int ntiles) {
+    int M, int D, int ntiles) {
     constexpr int KS = BW / 16;
     constexpr int kWRowBytes = BW * 2 + 16;        // one output column's bw weights + pad
     __shared__ __align__(16) unsigned char sW[32 * kWRowBytes];
@@ -794,7 +781,7 @@ int launch_gate_fwd(const void* x, const void* w_i, const float* b_i, const void
         hipLaunchKernelGGL((gate_proj_fwd_small_kernel<XT, WT, OT, BW>), dim3((unsigned)ncolblocks, (unsigned)rsplit),
                            dim3(kSmallWaves * kWave), 0, st, static_cast<const XT*>(x), static_cast<const WT*>(w_i),
                            b_i, static_cast<const WT*>(w_a), b_a, static_cast<OT*>(out_i), static_cast<OT*>(out_a), M,
-                           D, nb, ntiles);
+                           D, ntiles);
         return hipGetLastError() == hipSuccess ? HAWK_OK : HAWK_ERR_LAUNCH;
     }
     int nworkers = kNumCU / ngroups;
