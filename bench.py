@@ -66,6 +66,9 @@ WORKLOADS = {
     "long": (2, 32768, 4096, (0.99, 0.9999), False),
     "scan_conv": (8, 4096, 2560, (0.9, 0.999), True),
     "scan_gated": (8, 4096, 2560, (0.9, 0.999), False),
+    # fp32 activations and gate logits in, bf16 h and grad_out, fp32 gradients out (what the
+    # scan sees under bf16 autocast when its producers ran in fp32)
+    "scan_mixed": (8, 4096, 2560, (0.9, 0.999), False),
 }
 
 
@@ -529,13 +532,17 @@ def main():
     code = _lib.HAWK_DTYPE_BF16
     bf = torch.bfloat16
 
+    mixed = args.workload == "scan_mixed"
+    in_dt = torch.float32 if mixed else bf
+    in_code = _lib.HAWK_DTYPE_F32 if mixed else code
     gen = torch.Generator(device=dev).manual_seed(args.seed)
-    x, xg, ag, gout = (torch.randn(B, T, D, device=dev, generator=gen).to(bf) for _ in range(4))
+    x, xg, ag = (torch.randn(B, T, D, device=dev, generator=gen).to(in_dt) for _ in range(3))
+    gout = torch.randn(B, T, D, device=dev, generator=gen).to(bf)
     lam = lambda_for_a8_range(torch.Generator().manual_seed(args.seed), D, lo, hi).to(dev)
-    h = torch.empty_like(x)
+    h = torch.empty_like(gout)
     dx, dxg, dag = torch.empty_like(x), torch.empty_like(x), torch.empty_like(x)
     dlam = torch.empty(D, dtype=torch.float32, device=dev)
-    ws = torch.zeros(lib.hawk_scan_workspace_bytes(B, T, D, code), dtype=torch.uint8, device=dev)
+    ws = torch.zeros(lib.hawk_scan_workspace_bytes(B, T, D, in_code), dtype=torch.uint8, device=dev)
     if with_conv:
         W = 4
         cw = (torch.randn(W, D, device=dev, generator=gen) * 0.5).float()
@@ -559,6 +566,11 @@ def main():
                 x.data_ptr(), xg.data_ptr(), ag.data_ptr(), lam.data_ptr(), y.data_ptr(), 2 * D, h.data_ptr(),
                 gated_out.data_ptr(), None, B, T, D, code, code, ws.data_ptr(), ws.numel(), stream))
             return
+        if mixed:
+            _lib.check("scan_fwd_mixed", lib.hawk_rglru_scan_fwd_mixed(
+                x.data_ptr(), xg.data_ptr(), ag.data_ptr(), lam.data_ptr(), h.data_ptr(), B, T, D, in_code, code,
+                ws.data_ptr(), ws.numel(), stream))
+            return
         src = x
         if with_conv:
             _lib.check("conv_fwd", lib.hawk_conv1d_fwd(x.data_ptr(), cw.data_ptr(), cb.data_ptr(), None,
@@ -574,6 +586,12 @@ def main():
                 x.data_ptr(), xg.data_ptr(), ag.data_ptr(), lam.data_ptr(), y.data_ptr(), 2 * D, h.data_ptr(),
                 gout.data_ptr(), dx.data_ptr(), dxg.data_ptr(), dag.data_ptr(), dy.data_ptr(), D, dlam.data_ptr(),
                 B, T, D, code, code, ws.data_ptr(), ws.numel(), stream))
+            return
+        if mixed:
+            _lib.check("scan_bwd_mixed", lib.hawk_rglru_scan_bwd_mixed(
+                x.data_ptr(), xg.data_ptr(), ag.data_ptr(), lam.data_ptr(), h.data_ptr(), gout.data_ptr(),
+                dx.data_ptr(), dxg.data_ptr(), dag.data_ptr(), dlam.data_ptr(), B, T, D, in_code, code,
+                ws.data_ptr(), ws.numel(), stream))
             return
         src = u if with_conv else x
         _lib.check("scan_bwd", lib.hawk_rglru_scan_bwd(src.data_ptr(), xg.data_ptr(), ag.data_ptr(),
@@ -625,6 +643,8 @@ def main():
     # gated: the forward also reads y and writes out; the backward also reads y and writes dy
     fwd_bytes = (6 if gated else 4) * elem * N + (2 * elem * N if with_conv else 0)
     bwd_bytes = (10 if gated else 8) * elem * N
+    if mixed:  # three fp32 inputs + bf16 h; three fp32 inputs + bf16 h, grad_out, three fp32 gradients
+        fwd_bytes, bwd_bytes = (3 * 4 + 2) * N, (3 * 4 + 2 + 2 + 3 * 4) * N
     step_bytes = fwd_bytes + bwd_bytes + (3 * elem * N if with_conv else 0)
     bwd_gbs = bwd_bytes / (bwd_ms * 1e-3) / 1e9
 
@@ -639,13 +659,14 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "bf16 in/out, f32 state and accumulation",
+        "dtype": ("f32 inputs and gradients, bf16 h and grad_out, f32 state and accumulation" if mixed
+                  else "bf16 in/out, f32 state and accumulation"),
         "data": f"synthetic, seed {args.seed}: x, gate logits, grad ~ N(0,1); a^8 ~ U({lo},{hi})",
         "config": {
             "workload": f"{args.workload}: RG-LRU scan"
                         + (" + temporal conv1d (W=4)" if with_conv else "")
                         + (" fused with out = gelu(y) * h" if gated else "")
-                        + f" fwd+bwd, B={B}, T={T}, D={D}, bf16",
+                        + f" fwd+bwd, B={B}, T={T}, D={D}, " + ("f32 in / bf16 state" if mixed else "bf16"),
             "B": B, "T": T, "D": D,
         },
         "roofline": {
