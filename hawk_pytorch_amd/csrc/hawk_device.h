@@ -229,6 +229,11 @@ __device__ __forceinline__ uint32_t opaque(uint32_t x) {
     asm volatile("" : "+v"(x));
     return x;
 }
+__device__ __forceinline__ uint16_t opaque(uint16_t x) {
+    uint32_t w = x;
+    asm volatile("" : "+v"(w));
+    return (uint16_t)w;
+}
 
 __device__ __forceinline__ float clamp01(float z) { return fminf(fmaxf(z, 0.0f), 1.0f); }
 

@@ -515,14 +515,26 @@ __device__ __forceinline__ void bwd_tile(const IT* __restrict__ x, const IT* __r
         unpack(rag[j], fag);
         unpack(rgo[j], fgo);
         if constexpr (GATED) {
-            float fy[V];
+            // The gate is evaluated once.  gout gelu(y), the gradient that reaches h, takes
+            // gout's registers, and gout gelu'(y), which the replay multiplies by h_t to get
+            // dy, takes y's: both in the state dtype, which is also where an unfused
+            // gelu(y) * h backward would round them.
+            float fy[V], gd[V];
             unpack(ry[j], fy);
 #pragma unroll
             for (int v = 0; v < V; ++v) {
                 float cdf, e;
                 normal_cdf<PRECISE>(fy[v], cdf, e);
+                gd[v] = fgo[v] * fmaf(fy[v] * kInvSqrt2Pi, e, cdf);
                 fgo[v] *= fy[v] * cdf;
             }
+            // (pinned here: left alone, the compiler sinks the conversions to their uses after
+            // the exchange and keeps two floats per element alive instead of one packed word)
+            pack(fgo, rgo[j]);
+            pack(gd, ry[j]);
+            rgo[j] = opaque(rgo[j]);
+            ry[j] = opaque(ry[j]);
+            unpack(rgo[j], fgo);  // the chain must see exactly the gradient the replay will see
         }
         const bool ok = FULL || (t0 + j < T);
 #pragma unroll
@@ -541,6 +553,7 @@ __device__ __forceinline__ void bwd_tile(const IT* __restrict__ x, const IT* __r
             c_run[v] = alpha * (fgo[v] + c_run[v]);
             q_run[v] *= alpha;
         }
+        if constexpr (GATED) __builtin_amdgcn_sched_barrier(0);  // one row's gate temporaries at a time
     }
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -591,22 +604,16 @@ __device__ __forceinline__ void bwd_tile(const IT* __restrict__ x, const IT* __r
         unpack(rhp[j], fhp);
         float o4[V];
         if constexpr (GATED) {
-            // gelu(y) again (cheaper than a register per element across the exchange), its
-            // derivative, and h_t, which is the next row's h_{t-1}
-            float fy[V], fh[V];
+            // dy = (gout gelu'(y)) h_t; h_t is the next row's h_{t-1}
+            float fd[V], fh[V];
             if constexpr (sizeof(sraw_t) == 4 && sizeof(ST) == 2) {
-                unpack(opaque(ry[j]), fy);
+                unpack(opaque(ry[j]), fd);
             } else {
-                unpack(ry[j], fy);
+                unpack(ry[j], fd);
             }
             unpack(j == TC - 1 ? rh_end : rhp[j == TC - 1 ? j : j + 1], fh);
 #pragma unroll
-            for (int v = 0; v < V; ++v) {
-                float cdf, e;
-                normal_cdf<PRECISE>(fy[v], cdf, e);
-                o4[v] = (fgo[v] * fh[v]) * fmaf(fy[v] * kInvSqrt2Pi, e, cdf);
-                fgo[v] *= fy[v] * cdf;
-            }
+            for (int v = 0; v < V; ++v) o4[v] = fd[v] * fh[v];
         }
         const bool ok = FULL || (t0 + j < T);
         const uint32_t rpair = PACK_R ? opaque(rrh[j]) : 0u;
@@ -769,11 +776,12 @@ struct TileShape {
 #define HAWK_BWD_GATED_TC 10
 #endif
 #ifndef HAWK_BWD_GATED_TC1
-#define HAWK_BWD_GATED_TC1 8
+#define HAWK_BWD_GATED_TC1 12
 #endif
 constexpr int kFwdTC = HAWK_FWD_TC, kFwdNW = HAWK_FWD_NW;
 constexpr int kBwdTC = HAWK_BWD_TC, kBwdNW = HAWK_BWD_NW;
-// the gate adds a register per row and lane (two channels per lane), or two (one channel)
+// with two channels per lane the gate's operands cost two more registers per row and the tile
+// is two rows shorter; with one channel per lane the plain kernel's tile height still fits
 constexpr int kBwdGatedTC = HAWK_BWD_GATED_TC, kBwdGatedTC1 = HAWK_BWD_GATED_TC1;
 constexpr int kFwdGatedTC = HAWK_FWD_GATED_TC;  // two channels per lane; one channel keeps kFwdTC
 
@@ -939,12 +947,13 @@ int scan_bwd_impl(const void* x, const void* xg, const void* ag, const float* la
 
 size_t scan_workspace_bytes(int B, int T, int D, int dtype) {
     // one size serves every scan entry point: the longest chain (shortest tile) decides
-    const int rows[3] = {fwd_shape(D, dtype).rows(), bwd_shape(D, dtype).rows(), bwd_gated_shape(1).rows()};
+    const int rows[6] = {fwd_shape(D, dtype).rows(), fwd_gated_shape(1).rows(),   fwd_gated_shape(2).rows(),
+                         bwd_shape(D, dtype).rows(), bwd_gated_shape(1).rows(),   bwd_gated_shape(2).rows()};
     int n_chain = 0, n_dlam = 0;
-    for (int k = 0; k < 3; ++k) {
+    for (int k = 0; k < 6; ++k) {
         const int n = ceil_div(T, rows[k]);
         if (n > n_chain) n_chain = n;
-        if (k > 0 && n > n_dlam) n_dlam = n;
+        if (k >= 3 && n > n_dlam) n_dlam = n;  // only the backward kernels write dLambda partials
     }
     return layout_for(B, D, n_chain, n_dlam).total;
 }
