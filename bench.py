@@ -53,11 +53,13 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the backward scan kernel, from rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE runs of this file, each scaled by what the same counter reads for a plain
 # device copy of known size in the same run (FETCH x 2.000, WRITE x 1.000 on this part).
-# Sources: profiles/rglru_scan_B8_T4096_D2560_bf16.md, profiles/rglru_scan_B2_T32768_D4096_bf16.md.
+# Sources: profiles/rglru_scan_B8_T4096_D2560_bf16.md, profiles/rglru_scan_B2_T32768_D4096_bf16.md,
+# profiles/rglru_scan_gated_B8_T4096_D2560_bf16.md.
 MEASURED_BWD_TRAFFIC_BYTES = {
     "scan": 865.4e6 + 533.0e6,
     "scan_conv": 865.4e6 + 533.0e6,
     "long": 2776.5e6 + 1711.7e6,
+    "scan_gated": 1043.5e6 + 704.8e6,
 }
 
 WORKLOADS = {
