@@ -267,7 +267,6 @@ __global__ __launch_bounds__(kGateThreads, 1) void gate_proj_fwd_kernel(
 
     const int a_off = col * kARowBytes + (blk * BW + khalf) * 2;
     unsigned char* o_base = sO + (4 * (lane >> 5)) * kORowBytes + (g * kGroup + 32 * c + col) * (int)sizeof(OT);
-    const unsigned char* o_src = sO + lrow * kORowBytes + lc8 * 8 * (int)sizeof(OT);
 
     auto step = [&](int it, int cur, Row8<XT>& rnext) {
         // 32 x 32 output tile of this wave: A operands from LDS, B operands resident.  The A
@@ -295,17 +294,22 @@ __global__ __launch_bounds__(kGateThreads, 1) void gate_proj_fwd_kernel(
         stage_tile(cur ^ 1, rnext);
         load_tile(it + 3, rnext);
         __syncthreads();
-        const int row = (worker + it * nworkers) * kTileRows + lrow;
-        if (col_ok && row < M) {
-            constexpr int kVecs = (int)sizeof(OT) / 2;  // 16-byte pieces per 8 elements
-            OT* dst_i = out_i + (size_t)row * D + lcol;
-            OT* dst_a = out_a + (size_t)row * D + lcol;
+        // a gate's row of the group is 32 (bf16) or 64 (fp32) pieces of 16 bytes; consecutive
+        // threads take consecutive pieces, so that every store instruction writes whole rows
+        constexpr int kPieces = kGroup * (int)sizeof(OT) / 16;
+        constexpr int kPerThread = kTileRows * kPieces / kGateThreads;
 #pragma unroll
-            for (int q = 0; q < kVecs; ++q) {
-                const u32x4 vi = *reinterpret_cast<const u32x4*>(o_src + q * 16);
-                const u32x4 va = *reinterpret_cast<const u32x4*>(o_src + kGroup * (int)sizeof(OT) + q * 16);
-                __builtin_nontemporal_store(vi, reinterpret_cast<u32x4*>(dst_i) + q);
-                __builtin_nontemporal_store(va, reinterpret_cast<u32x4*>(dst_a) + q);
+        for (int q = 0; q < kPerThread; ++q) {
+            const int piece = tid + q * kGateThreads;
+            const int prow = piece / kPieces, pc = piece % kPieces;
+            const int row = (worker + it * nworkers) * kTileRows + prow;
+            const int ocol = group * kGroup + pc * (16 / (int)sizeof(OT));
+            if (ocol < D && row < M) {
+                const unsigned char* src = sO + prow * kORowBytes + pc * 16;
+                const u32x4 vi = *reinterpret_cast<const u32x4*>(src);
+                const u32x4 va = *reinterpret_cast<const u32x4*>(src + kGroup * (int)sizeof(OT));
+                __builtin_nontemporal_store(vi, reinterpret_cast<u32x4*>(out_i + (size_t)row * D + ocol));
+                __builtin_nontemporal_store(va, reinterpret_cast<u32x4*>(out_a + (size_t)row * D + ocol));
             }
         }
         __syncthreads();
