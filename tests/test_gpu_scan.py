@@ -284,3 +284,36 @@ def test_scan_launches_replay_correctly_from_a_hip_graph():
         for a, b in zip(again, eager):
             assert torch.equal(a, b), rep
     assert capi.workspace_flag(ws) == 0
+
+
+def test_two_streams_scan_concurrently_with_their_own_workspaces():
+    """Two scans of the benchmark size in flight at once on two streams, each with its own
+    workspace (the rule of the C ABI), several rounds: every result must equal the one obtained
+    alone.  A tile only ever waits for tiles of its own launch that have already started, so
+    two launches sharing the compute units cannot block each other."""
+    B, T, D = 8, 4096, 2560
+    g = torch.Generator(device="cuda").manual_seed(31)
+    lam = capi.to_dev(np.log(np.power(np.random.default_rng(31).uniform(0.9, 0.999, size=D), -1.0 / 8.0) - 1.0), "f32")
+    sets = []
+    for _ in range(2):
+        x, xg, ag, go = (torch.randn(B, T, D, device="cuda", generator=g).to(torch.bfloat16) for _ in range(4))
+        ws = capi.new_workspace(B, T, D, "bf16")
+        h = capi.scan_fwd(x, xg, ag, lam, ws)
+        grads = capi.scan_bwd(x, xg, ag, lam, h, go, ws)
+        sets.append((x, xg, ag, go, ws, h, grads))
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    for s in streams:
+        s.wait_stream(torch.cuda.current_stream())
+    for _ in range(3):
+        got = []
+        for (x, xg, ag, go, ws, _, _), s in zip(sets, streams):
+            with torch.cuda.stream(s):
+                h = capi.scan_fwd(x, xg, ag, lam, ws)
+                got.append((h, capi.scan_bwd(x, xg, ag, lam, h, go, ws)))
+        torch.cuda.synchronize()
+        for (h, grads), (_, _, _, _, ws, h_ref, grads_ref) in zip(got, sets):
+            assert capi.workspace_flag(ws) == 0
+            assert torch.equal(h, h_ref)
+            for a, b in zip(grads, grads_ref):
+                assert torch.equal(a, b)
