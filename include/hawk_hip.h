@@ -67,6 +67,11 @@ int hawk_scan_workspace_status(const void* workspace_device, void* stream, int* 
  * (hawk/scan_fused.py:319-360, :34-109).  Lambda stays fp32 for both dtypes.  Any D >= 1
  * is accepted (upstream requires D % 64 == 0); even D takes the two-channels-per-lane
  * path.  The workspace may be NULL when T fits one tile.
+ * Every scan entry point is reproducible: its outputs are a function of the inputs and of
+ * (B, T, D, dtypes) alone, never of timing, so two launches on the same data agree bit for
+ * bit.  The same sequence inside another batch size may differ in the last bit of fp32
+ * intermediate sums (launches with few independent chains group their carries in wider
+ * windows).
  * ------------------------------------------------------------------------------------- */
 int hawk_rglru_scan_fwd(const void* x, const void* x_rg_lru, const void* a_rg_lru,
                         const float* a_param, void* h, int B, int T, int D, int dtype,
