@@ -33,6 +33,40 @@ def test_library_exports_every_declared_symbol():
     assert lib.hawk_version() >= 100
 
 
+def test_header_is_plain_c_and_links_against_the_library(tmp_path):
+    """The boundary is a C ABI: the header must compile as C99 with no HIP or C++ headers, and a C
+    program that only validates arguments (no GPU needed) must link and run against the .so."""
+    import shutil
+    import subprocess
+
+    gcc = shutil.which("gcc")
+    if gcc is None:
+        pytest.skip("no gcc")
+    src = tmp_path / "caller.c"
+    src.write_text(
+        '#include <stdio.h>\n#include <string.h>\n#include "hawk_hip.h"\n'
+        "int main(void) {\n"
+        "    char x[16];\n"
+        "    if (hawk_version() < 100) return 1;\n"
+        "    if (strcmp(hawk_status_string(HAWK_OK), \"ok\") != 0) return 2;\n"
+        "    if (hawk_scan_workspace_bytes(8, 4096, 2560, HAWK_DTYPE_BF16) == 0) return 3;\n"
+        "    if (hawk_rglru_scan_fwd(NULL, x, x, (const float*)x, x, 1, 1, 64, HAWK_DTYPE_BF16, NULL, 0, NULL)\n"
+        "        != HAWK_ERR_NULL_POINTER) return 4;\n"
+        "    if (hawk_gate_proj_supported(2560, 10) != 1 || hawk_gate_proj_supported(2560, 3) != 0) return 5;\n"
+        '    puts("c caller ok");\n    return 0;\n}\n'
+    )
+    exe = tmp_path / "caller"
+    libdir = os.path.dirname(_lib.LIB_PATH)
+    _lib.load()  # builds the library if it is not there yet
+    subprocess.run(
+        [gcc, "-std=c99", "-Wall", "-Wextra", "-Werror", "-pedantic", "-I", os.path.join(ROOT, "include"), str(src),
+         "-o", str(exe), "-L", libdir, "-l:" + os.path.basename(_lib.LIB_PATH), "-Wl,-rpath," + libdir,
+         "-Wl,-rpath,/opt/rocm/lib", "-Wl,--allow-shlib-undefined"],
+        check=True, capture_output=True, text=True)
+    out = subprocess.run([str(exe)], check=True, capture_output=True, text=True)
+    assert "c caller ok" in out.stdout
+
+
 def test_status_strings_are_distinct():
     msgs = {_lib.status_string(s) for s in range(7)}
     assert len(msgs) == 7 and _lib.status_string(0) == "ok"
