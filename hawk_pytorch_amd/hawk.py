@@ -75,9 +75,13 @@ class RMSNorm(nn.Module):
         self.weight = nn.Parameter(torch.ones(dim))
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
-        xf = x.float()
-        normed = xf * torch.rsqrt(xf.square().mean(dim=-1, keepdim=True) + self.eps)
-        return normed.type_as(x) * self.weight
+        # hawk/hawk.py:53-58 normalises in fp32, rounds to x's dtype and multiplies by the weight,
+        # about eight eager kernels.  The library's rms_norm does it in one, in fp32 throughout
+        # (one rounding less), with the reference's output dtype: x's when the weight has it,
+        # fp32 when the weight is an fp32 parameter and x is not.
+        if self.weight.dtype == x.dtype:
+            return F.rms_norm(x, (x.shape[-1],), self.weight, self.eps)
+        return F.rms_norm(x.float(), (x.shape[-1],), self.weight.float(), self.eps)
 
 
 class MLP(nn.Module):
