@@ -62,6 +62,10 @@ MEASURED_BWD_TRAFFIC_BYTES = {
     "scan_gated": 1043.5e6 + 704.8e6,
 }
 
+# The same for the gates workload's dominant launch (weight-gradient kernel + its reduce kernel):
+# 503.4 + 63.2 MB read, 63.2 + 5.3 MB written (profiles/gate_proj_M32768_D2560_nb10_bf16.md).
+MEASURED_GATE_DW_TRAFFIC_BYTES = 503.4e6 + 63.2e6 + 63.2e6 + 5.3e6
+
 WORKLOADS = {
     # name: (B, T, D, a^8 range, includes conv)
     "scan": (8, 4096, 2560, (0.9, 0.999), False),
@@ -175,7 +179,8 @@ def run_gates(args, lib, dev):
             "bound": "hbm",
             "kernel": "gate_proj_bwd_weights_kernel (+ gate_proj_reduce_kernel, same launch call)",
             "achieved": gbs[2], "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs[2] / HBM_PEAK_GBS,
-            "traffic": None, "algorithmic_bytes_per_launch": alg[2], "launch_ms": ms[2],
+            "traffic": MEASURED_GATE_DW_TRAFFIC_BYTES,
+            "algorithmic_bytes_per_launch": alg[2], "launch_ms": ms[2],
         },
         "kernels": {name: {"ms": ms[i], "GBs": gbs[i], "frac": gbs[i] / HBM_PEAK_GBS,
                            "TFLOPs": flops[i] / (ms[i] * 1e-3) / 1e12}
