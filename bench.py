@@ -83,13 +83,14 @@ def lambda_for_a8_range(gen, D, lo, hi):
     return torch.log(u.pow(-1.0 / 8.0) - 1.0).float()
 
 
-def cpu_baseline(B, D, lo, hi, seed, budget_rows=512):
-    """PyTorch CPU loop (oracle/rglru_torch.py) on the first `budget_rows` time rows of the
-    workload's shape: forward plus autograd backward in fp32."""
+def cpu_baseline(B, D, lo, hi, seed, budget_elements=1536 * 8 * 2560):
+    """PyTorch CPU loop (oracle/rglru_torch.py) on the first time rows of the workload's shape,
+    about `budget_elements` element-steps (10-20 s on 16 host threads): forward plus autograd
+    backward in fp32."""
     from oracle import rglru_torch
 
     gen = torch.Generator().manual_seed(seed)
-    T = budget_rows
+    T = max(256, budget_elements // (B * D))
     x, xg, ag, go = (torch.randn(B, T, D, generator=gen) for _ in range(4))
     lam = lambda_for_a8_range(gen, D, lo, hi)
     rglru_torch.rglru_scan_fwd_bwd(x[:, :8], xg[:, :8], ag[:, :8], lam, go[:, :8])  # warm-up
@@ -625,16 +626,21 @@ def main():
             conv_bwd()
     torch.cuda.synchronize()
 
-    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
+    # Two events per step bracket the backward launch; the forward launch of step k runs from the
+    # end of step k-1 (its last event, or the event after the conv backward) to the first event of
+    # step k.
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3 if with_conv else 2)] for _ in range(args.steps)]
+    start = torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
+    start.record()
     for k in range(args.steps):
-        ev[k][0].record()
         fwd()
-        ev[k][1].record()
+        ev[k][0].record()
         bwd()
-        ev[k][2].record()
+        ev[k][1].record()
         if with_conv:
             conv_bwd()
+            ev[k][2].record()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
 
@@ -644,8 +650,9 @@ def main():
         print("bench.py: a scan tile gave up waiting for its carry; results are invalid", file=sys.stderr)
         sys.exit(1)
 
-    fwd_ms = float(np.mean([e[0].elapsed_time(e[1]) for e in ev]))
-    bwd_ms = float(np.mean([e[1].elapsed_time(e[2]) for e in ev]))
+    step_end = [start] + [e[-1] for e in ev]
+    fwd_ms = float(np.mean([step_end[k].elapsed_time(ev[k][0]) for k in range(args.steps)]))
+    bwd_ms = float(np.mean([e[0].elapsed_time(e[1]) for e in ev]))
     ms_per_step = wall * 1e3 / args.steps
     elem = 2  # bytes per bf16 activation element
     # gated: the forward also reads y and writes out; the backward also reads y and writes dy
