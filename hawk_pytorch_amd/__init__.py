@@ -6,6 +6,7 @@ from .cache import RNNCache
 from .external import (
     BlockDiagonalLinear,
     Conv1D,
+    decode_core_step,
     gate_projections,
     rglru_step,
     rglru_step_gated,
@@ -36,6 +37,7 @@ __all__ = [
     "RMSNorm",
     "RNNCache",
     "RNNLayer",
+    "decode_core_step",
     "fused_linear_scan",
     "gate_projections",
     "recurrent_core",

@@ -57,6 +57,12 @@ SIGNATURES = {
     "hawk_conv1d_step": (_c_int, [_c_void_p] * 5 + [_c_int] * 5 + [_c_void_p]),
     "hawk_rglru_step": (_c_int, [_c_void_p] * 6 + [_c_int] * 4 + [_c_void_p]),
     "hawk_gate_proj_supported": (_c_int, [_c_int, _c_int]),
+    "hawk_decode_core_supported": (_c_int, [_c_int] * 3),
+    "hawk_decode_core_step": (
+        _c_int,
+        [_c_void_p] * 2 + [ctypes.c_longlong] + [_c_void_p] * 8 + [ctypes.c_longlong] + [_c_void_p] * 2
+        + [_c_int] * 7 + [_c_void_p],
+    ),
     "hawk_gate_proj_fwd": (_c_int, [_c_void_p] * 7 + [_c_int] * 6 + [_c_void_p]),
     "hawk_gate_proj_bwd_input": (_c_int, [_c_void_p] * 6 + [_c_int] * 6 + [_c_void_p]),
     "hawk_gate_proj_bwd_weights_workspace_bytes": (_c_size_t, [_c_int] * 3),

@@ -215,6 +215,28 @@ int hawk_gate_proj_supported(int D, int num_blocks) {
     return hawk::gate_proj_block_width_supported(D / num_blocks) ? 1 : 0;
 }
 
+int hawk_decode_core_supported(int D, int num_blocks, int W) {
+    return (W >= 1 && W <= 8 && hawk_gate_proj_supported(D, num_blocks)) ? 1 : 0;
+}
+
+int hawk_decode_core_step(void* conv_state, const void* x_new, long long ldx, const float* conv_w,
+                          const float* conv_b, const void* w_i, const float* b_i, const void* w_a, const float* b_a,
+                          const float* a_param, const void* y, long long ldy, void* recc_state, void* out, int B, int D,
+                          int num_blocks, int W, int dtype, int w_dtype, int state_dtype, void* stream) {
+    if (!x_new || !conv_w || !conv_b || !w_i || !w_a || !a_param || !y || !recc_state || !out ||
+        (W > 1 && !conv_state))
+        return HAWK_ERR_NULL_POINTER;
+    if (dtype != HAWK_DTYPE_BF16 || !dtype_ok(w_dtype) || !dtype_ok(state_dtype)) return HAWK_ERR_BAD_DTYPE;
+    if (B < 1 || !hawk_decode_core_supported(D, num_blocks, W)) return HAWK_ERR_BAD_SHAPE;
+    // rows of x_new are read 16 bytes at a time
+    if (ldx < D || (ldx % 8) != 0 || ldx > kMaxRowStride || ldy < D || ldy > kMaxRowStride) return HAWK_ERR_BAD_SHAPE;
+    if (!aligned16(x_new) || (conv_state && !aligned16(conv_state)) || !aligned16(w_i) || !aligned16(w_a) ||
+        !aligned_elem(y, dtype) || !aligned_elem(recc_state, state_dtype) || !aligned_elem(out, dtype))
+        return HAWK_ERR_ALIGNMENT;
+    return hawk::decode_core_step(conv_state, x_new, ldx, conv_w, conv_b, w_i, b_i, w_a, b_a, a_param, y, ldy,
+                                  recc_state, out, B, D, num_blocks, W, w_dtype, state_dtype, as_stream(stream));
+}
+
 int hawk_gate_proj_fwd(const void* x, const void* w_i, const float* b_i, const void* w_a, const float* b_a,
                        void* x_rg_lru, void* a_rg_lru, int M, int D, int num_blocks, int x_dtype, int w_dtype,
                        int out_dtype, void* stream) {

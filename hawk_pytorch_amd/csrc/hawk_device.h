@@ -283,4 +283,21 @@ __device__ __forceinline__ void normal_cdf(float y, float& cdf, float& e) {
 }
 constexpr float kInvSqrt2Pi = 0.39894228040143268f;
 
+// One decode step of the RG-LRU for one channel (hawk/hawk.py:137-151, :196 upstream):
+//   h = alpha * state + sqrt(1 - alpha^2) * (sigmoid(xg) * x),  alpha = exp(-8 s sigmoid(ag)),
+// with s = softplus(Lambda) evaluated by the caller.
+__device__ __forceinline__ float rglru_step_value(float x, float xg, float ag, float s, float state) {
+    const float i = sigmoid_fast(xg);
+    const float r = sigmoid_fast(ag);
+    const float alpha = hw_exp2(-8.0f * kLog2e * s * r);
+    const float z = one_minus_exp(-16.0f * s * r);
+    return fmaf(alpha, state, hw_sqrt(z) * (i * x));
+}
+// gelu(y) * h with the exact (erf) GELU (hawk/hawk.py:134-135 upstream).
+__device__ __forceinline__ float gelu_times(float y, float h) {
+    float cdf, e;
+    normal_cdf<true>(y, cdf, e);
+    return (y * cdf) * h;
+}
+
 }  // namespace hawk

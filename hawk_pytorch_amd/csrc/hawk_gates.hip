@@ -421,6 +421,209 @@ __global__ __launch_bounds__(kSmallWaves* kWave, sizeof(XT) == 2 ? 4 : 2) void g
 }
 
 // ---------------------------------------------------------------------------------------
+// One decode step of a layer's whole recurrent core in one launch: the conv window roll and
+// conv, both gate projections, the RG-LRU state update and the output gate
+// (hawk/hawk.py:137-151, :169-182, :196-198 and hawk/cache.py:37-43 upstream; the three launches
+// hawk_conv1d_step, hawk_gate_proj_fwd, hawk_rglru_step_gated here).  Every kernel of a decode
+// step runs for about as long as it takes to start, so what this saves is two starts per layer.
+//
+// A workgroup of 8 waves owns 32 batch rows of one block of the projections, i.e. every
+// channel that those rows' outputs in the block depend on:
+//   1. all waves: conv of the rows' bw channels from the window in conv_state and the new row;
+//      the window is rolled in place, the result goes to LDS as bf16 (the MFMA A operand, and x
+//      of the recurrence);
+//   2. wave c < bw/32: the bw x 32 slices of both weight matrices that produce output columns
+//      32c.. of the block, transposed through a wave-private LDS region into B operands, one
+//      gate after the other (the second gate's weights travel while the first is multiplied);
+//   3. the same wave: biases, recurrence and gate on its 32 x 32 outputs straight from the
+//      accumulators; recc_state is updated in place.
+// Intermediate roundings are those of the three separate launches (conv output and logits to
+// bf16), so the two paths agree to the last bit or two of a bf16 result.
+// Where its time goes at 256 rows and a block width of 256 (19.5 us, as long as the three
+// launches it replaces; 10 us against 14.5 at a width of 128): 8.7 us for the launch, staging, matrix
+// products, operand loads and stores; 4.8 us fetching a block's 256 KiB of weights into one compute
+// unit (fetching the second gate's earlier does not shorten it); 2.9 us for the conv; 1.6 us
+// for the recurrence and gate.  One workgroup per (32 rows, block) is 80 workgroups here: what
+// the launch saves in starts it loses to running on a third of the device, so its gain is on
+// the host side (one call instead of three plus a copy).  Cutting a block's columns over more
+// workgroups would need the window roll out of the kernel: they would read rows that another
+// of them overwrites.
+// ---------------------------------------------------------------------------------------
+constexpr int kCoreWaves = 8;
+constexpr int kCoreMaxW = 8;
+
+template <int BW>
+struct CoreLds {
+    static constexpr int kRowBytes = BW * 2 + 16;                       // bf16 row + pad
+    static constexpr int kUBytes = kTileRows * kRowBytes;               // conv output tile
+    static constexpr int kWaveBytes = 32 * kRowBytes;                   // one wave's 32 weight columns
+    static constexpr int kWaves = BW / 32 < kCoreWaves ? BW / 32 : kCoreWaves;
+    static constexpr int kBytes = kUBytes + kWaves * kWaveBytes;
+};
+
+// all LDS traffic of this wave issued so far has completed, and the compiler keeps what
+// follows behind it
+__device__ __forceinline__ void wave_lds_fence() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
+
+template <typename WT, typename ST, int BW>
+__global__ __launch_bounds__(kCoreWaves* kWave, 1) void decode_core_kernel(
+    bf16_t* __restrict__ conv_state, const bf16_t* __restrict__ x_new, size_t ldx, const float* __restrict__ conv_w,
+    const float* __restrict__ conv_b, const WT* __restrict__ w_i, const float* __restrict__ b_i,
+    const WT* __restrict__ w_a, const float* __restrict__ b_a, const float* __restrict__ lam,
+    const bf16_t* __restrict__ y, size_t ldy, ST* __restrict__ state, bf16_t* __restrict__ out, int M, int D, int nb,
+    int W, int ntiles) {
+    static_assert(BW % 32 == 0 && BW <= 32 * kCoreWaves, "one wave per 32 output columns of a block");
+    constexpr int KS = BW / 16;
+    constexpr int NT = BW / 32;
+    constexpr int kRowBytes = CoreLds<BW>::kRowBytes;
+    constexpr int TPL = BW >= kWave ? BW / kWave : 1;   // weight tasks per lane and gate
+    extern __shared__ __align__(16) unsigned char core_smem[];
+    unsigned char* sU = core_smem;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & (kWave - 1);
+    const int w = __builtin_amdgcn_readfirstlane(tid / kWave);
+    const int h = (int)blockIdx.x / ntiles;
+    const int rt = (int)blockIdx.x - h * ntiles;
+    const bool computes = w < NT;
+
+    // This wave's slice of a weight matrix: thread -> (4 input channels, 8 consecutive output
+    // columns).  Sixteen lanes take sixteen consecutive channel quads of one column octet (their
+    // 8-byte LDS writes then cover every bank once), the next sixteen the next octet of the same
+    // rows, so that one load instruction touches 16 rows of 64 contiguous bytes and every
+    // cache line is asked for by one instruction only.
+    constexpr int KQN = BW / 4 < 16 ? BW / 4 : 16;
+    WeightQuad<WT> raw[TPL];
+    auto fetch_weights = [&](const WT* wsel) {
+#pragma unroll
+        for (int q = 0; q < TPL; ++q) {
+            const int task = lane + q * kWave;
+            const int tkq = task % KQN + KQN * (task / (4 * KQN)), tn8 = ((task / KQN) % 4) * 8;
+            if (task < BW) raw[q].load(wsel + ((size_t)h * BW + 4 * tkq) * BW + w * 32 + tn8, BW);
+            else raw[q].clear();
+        }
+    };
+    unsigned char* sW = core_smem + CoreLds<BW>::kUBytes + (computes ? w : 0) * CoreLds<BW>::kWaveBytes;
+    auto stage_weights = [&]() {
+#pragma unroll
+        for (int q = 0; q < TPL; ++q) {
+            const int task = lane + q * kWave;
+            const int tkq = task % KQN + KQN * (task / (4 * KQN)), tn8 = ((task / KQN) % 4) * 8;
+            if (task < BW) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e)
+                    *reinterpret_cast<u32x2*>(sW + (tn8 + e) * kRowBytes + tkq * 8) = raw[q].column(e);
+            }
+        }
+    };
+    if (computes) fetch_weights(w_i);
+
+    // ---- 1. conv window roll + conv: 16-byte chunks of 8 channels
+    {
+        constexpr int CH = BW / 8;
+        const int H = W - 1;
+        for (int task = tid; task < kTileRows * CH; task += kCoreWaves * kWave) {
+            const int rl = task / CH, ch = task - rl * CH;
+            const int row = rt * kTileRows + rl;
+            const int c = h * BW + ch * 8;
+            u32x4 ubits = {0u, 0u, 0u, 0u};
+            if (row < M) {
+                bf16_t* sb = conv_state + (size_t)row * H * D + c;
+                u32x4 win[kCoreMaxW - 1];
+#pragma unroll
+                for (int j = 0; j < kCoreMaxW - 1; ++j) {
+                    if (j < H) win[j] = *reinterpret_cast<const u32x4*>(sb + (size_t)j * D);
+                }
+                const u32x4 newest = *reinterpret_cast<const u32x4*>(x_new + (size_t)row * ldx + c);
+                float acc[8], xv[8];
+#pragma unroll
+                for (int v = 0; v < 8; ++v) acc[v] = conv_b[c + v];
+#pragma unroll
+                for (int j = 0; j < kCoreMaxW - 1; ++j) {
+                    if (j < H) {
+                        unpack(win[j], xv);
+#pragma unroll
+                        for (int v = 0; v < 8; ++v) acc[v] = fmaf(conv_w[(size_t)j * D + c + v], xv[v], acc[v]);
+                    }
+                }
+                unpack(newest, xv);
+#pragma unroll
+                for (int v = 0; v < 8; ++v) acc[v] = fmaf(conv_w[(size_t)H * D + c + v], xv[v], acc[v]);
+                pack(acc, ubits);
+#pragma unroll
+                for (int j = 0; j < kCoreMaxW - 1; ++j) {
+                    if (j + 1 < H) *reinterpret_cast<u32x4*>(sb + (size_t)j * D) = win[j + 1];
+                }
+                if (H > 0) *reinterpret_cast<u32x4*>(sb + (size_t)(H - 1) * D) = newest;
+            }
+            *reinterpret_cast<u32x4*>(sU + rl * kRowBytes + ch * 16) = ubits;
+        }
+    }
+
+    // ---- 2. gate projections of this wave's 32 output columns
+    const int col = lane & 31, khalf = 8 * (lane >> 5);
+    const int c_out = h * BW + (computes ? w : 0) * 32 + col;      // this lane's channel
+    const int row0 = rt * kTileRows + 4 * (lane >> 5);             // accumulator r: row0 + 8 (r / 4) + r % 4
+    typedef typename Raw<ST, 1>::type sraw_t;
+    uint16_t ybits[16];
+    sraw_t sold[16];
+    if (computes) {
+        stage_weights();
+        fetch_weights(w_a);
+        // operands of the recurrence travel during the matrix products
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int row = row0 + 8 * (r / 4) + (r % 4);
+            const bool ok = row < M;
+            ybits[r] = ok ? load_raw<bf16_t, 1>(y + (size_t)row * ldy + c_out) : (uint16_t)0;
+            sold[r] = ok ? load_raw<ST, 1>(state + (size_t)row * D + c_out) : raw_zero<sraw_t>();
+        }
+    }
+    wave_lds_fence();
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    if (!computes) return;
+
+    const unsigned char* asrc = sU + col * kRowBytes + khalf * 2;
+    const unsigned char* bsrc = sW + col * kRowBytes + khalf * 2;
+    f32x16 acc_i = {}, acc_a = {};
+#pragma unroll
+    for (int s = 0; s < KS; ++s)
+        acc_i = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*reinterpret_cast<const bf16x8*>(asrc + 32 * s),
+                                                        *reinterpret_cast<const bf16x8*>(bsrc + 32 * s), acc_i, 0, 0, 0);
+    wave_lds_fence();   // the first gate's operands have been read: the region can be overwritten
+    stage_weights();
+    wave_lds_fence();
+#pragma unroll
+    for (int s = 0; s < KS; ++s)
+        acc_a = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*reinterpret_cast<const bf16x8*>(asrc + 32 * s),
+                                                        *reinterpret_cast<const bf16x8*>(bsrc + 32 * s), acc_a, 0, 0, 0);
+
+    // ---- 3. biases, recurrence, output gate
+    const float bias_i = b_i != nullptr ? b_i[c_out] : 0.0f;
+    const float bias_a = b_a != nullptr ? b_a[c_out] : 0.0f;
+    const float sp = softplus_precise(lam[c_out]);
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        const int rl = 4 * (lane >> 5) + 8 * (r / 4) + (r % 4);
+        const int row = rt * kTileRows + rl;
+        if (row >= M) continue;
+        const float u = __uint_as_float(
+            (uint32_t) * reinterpret_cast<const uint16_t*>(sU + rl * kRowBytes + (w * 32 + col) * 2) << 16);
+        const float xg = __uint_as_float((uint32_t)to_bf16_bits(acc_i[r] + bias_i) << 16);
+        const float ag = __uint_as_float((uint32_t)to_bf16_bits(acc_a[r] + bias_a) << 16);
+        float so[1], fy[1], hn[1];
+        unpack(sold[r], so);
+        unpack(ybits[r], fy);
+        hn[0] = rglru_step_value(u, xg, ag, sp, so[0]);
+        sraw_t rs;
+        pack(hn, rs);
+        *reinterpret_cast<sraw_t*>(state + (size_t)row * D + c_out) = rs;
+        *reinterpret_cast<uint16_t*>(out + (size_t)row * D + c_out) = to_bf16_bits(gelu_times(fy[0], hn[0]));
+    }
+}
+
+// ---------------------------------------------------------------------------------------
 // Input gradient of the two projections:
 //   dx[m, h*bw + i] = sum_j dxg[m, h*bw + j] w_i[h, i, j] + sum_j dag[m, h*bw + j] w_a[h, i, j]
 //                     (+ addend[m, h*bw + i], the gradient x receives from its other consumers)
@@ -895,9 +1098,55 @@ int gate_bwd_weights_bw(const void* x, const void* dg_i, const void* dg_a, float
     }
 }
 
+template <typename WT, typename ST, int BW>
+int launch_decode_core(void* conv_state, const void* x_new, long long ldx, const float* conv_w, const float* conv_b,
+                       const void* w_i, const float* b_i, const void* w_a, const float* b_a, const float* lam,
+                       const void* y, long long ldy, void* state, void* out, int B, int D, int nb, int W,
+                       hipStream_t st) {
+    const int ntiles = ceil_div(B, kTileRows);
+    const long long grid = (long long)nb * ntiles;
+    if (grid > 0x7fffffffLL) return HAWK_ERR_BAD_SHAPE;
+    constexpr auto kernel = decode_core_kernel<WT, ST, BW>;
+    constexpr size_t smem = CoreLds<BW>::kBytes;
+    if (!allow_dynamic_lds<kernel>(smem)) return HAWK_ERR_LAUNCH;
+    hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(kCoreWaves * kWave), smem, st,
+                       static_cast<bf16_t*>(conv_state), static_cast<const bf16_t*>(x_new), (size_t)ldx, conv_w,
+                       conv_b, static_cast<const WT*>(w_i), b_i, static_cast<const WT*>(w_a), b_a, lam,
+                       static_cast<const bf16_t*>(y), (size_t)ldy, static_cast<ST*>(state), static_cast<bf16_t*>(out),
+                       B, D, nb, W, ntiles);
+    return hipGetLastError() == hipSuccess ? HAWK_OK : HAWK_ERR_LAUNCH;
+}
+
+template <typename WT, typename ST>
+int decode_core_bw(void* conv_state, const void* x_new, long long ldx, const float* conv_w, const float* conv_b,
+                   const void* w_i, const float* b_i, const void* w_a, const float* b_a, const float* lam,
+                   const void* y, long long ldy, void* state, void* out, int B, int D, int nb, int W, hipStream_t st) {
+    switch (D / nb) {
+        case 32: return launch_decode_core<WT, ST, 32>(conv_state, x_new, ldx, conv_w, conv_b, w_i, b_i, w_a, b_a, lam, y, ldy, state, out, B, D, nb, W, st);
+        case 64: return launch_decode_core<WT, ST, 64>(conv_state, x_new, ldx, conv_w, conv_b, w_i, b_i, w_a, b_a, lam, y, ldy, state, out, B, D, nb, W, st);
+        case 128: return launch_decode_core<WT, ST, 128>(conv_state, x_new, ldx, conv_w, conv_b, w_i, b_i, w_a, b_a, lam, y, ldy, state, out, B, D, nb, W, st);
+        case 256: return launch_decode_core<WT, ST, 256>(conv_state, x_new, ldx, conv_w, conv_b, w_i, b_i, w_a, b_a, lam, y, ldy, state, out, B, D, nb, W, st);
+        default: return HAWK_ERR_BAD_SHAPE;
+    }
+}
+
 }  // namespace
 
 bool gate_proj_block_width_supported(int bw) { return bw == 32 || bw == 64 || bw == 128 || bw == 256; }
+
+int decode_core_step(void* conv_state, const void* x_new, long long ldx, const float* conv_w, const float* conv_b,
+                     const void* w_i, const float* b_i, const void* w_a, const float* b_a, const float* lam,
+                     const void* y, long long ldy, void* state, void* out, int B, int D, int nb, int W, int w_dtype,
+                     int state_dtype, hipStream_t st) {
+    if (w_dtype == HAWK_DTYPE_BF16) {
+        if (state_dtype == HAWK_DTYPE_BF16)
+            return decode_core_bw<bf16_t, bf16_t>(conv_state, x_new, ldx, conv_w, conv_b, w_i, b_i, w_a, b_a, lam, y, ldy, state, out, B, D, nb, W, st);
+        return decode_core_bw<bf16_t, float>(conv_state, x_new, ldx, conv_w, conv_b, w_i, b_i, w_a, b_a, lam, y, ldy, state, out, B, D, nb, W, st);
+    }
+    if (state_dtype == HAWK_DTYPE_BF16)
+        return decode_core_bw<float, bf16_t>(conv_state, x_new, ldx, conv_w, conv_b, w_i, b_i, w_a, b_a, lam, y, ldy, state, out, B, D, nb, W, st);
+    return decode_core_bw<float, float>(conv_state, x_new, ldx, conv_w, conv_b, w_i, b_i, w_a, b_a, lam, y, ldy, state, out, B, D, nb, W, st);
+}
 
 int gate_proj_fwd(const void* x, const void* w_i, const float* b_i, const void* w_a, const float* b_a, void* out_i,
                   void* out_a, int M, int D, int nb, int x_dtype, int w_dtype, int out_dtype, hipStream_t st) {

@@ -51,6 +51,12 @@ int gate_proj_fwd(const void* x, const void* w_i, const float* b_i, const void* 
                   void* out_a, int M, int D, int nb, int x_dtype, int w_dtype, int out_dtype, hipStream_t st);
 int gate_proj_bwd_input(const void* dxg, const void* dag, const void* w_i, const void* w_a, const void* addend,
                         void* dx, int M, int D, int nb, int g_dtype, int w_dtype, int dx_dtype, hipStream_t st);
+// conv window roll + conv, both projections, state update and output gate of one decode step
+// (bf16 activations and conv window; W <= 8)
+int decode_core_step(void* conv_state, const void* x_new, long long ldx, const float* conv_w, const float* conv_b,
+                     const void* w_i, const float* b_i, const void* w_a, const float* b_a, const float* lam,
+                     const void* y, long long ldy, void* state, void* out, int B, int D, int nb, int W, int w_dtype,
+                     int state_dtype, hipStream_t st);
 size_t gate_proj_bwd_weights_workspace_bytes(int M, int D, int nb);
 int gate_proj_bwd_weights(const void* x, const void* dg_i, const void* dg_a, float* dw_i, float* db_i, float* dw_a,
                           float* db_a, int M, int D, int nb, int x_dtype, int g_dtype, void* ws, size_t ws_bytes,

@@ -99,12 +99,7 @@ __global__ __launch_bounds__(256) void rglru_step_kernel(const ET* __restrict__ 
     for (int v = 0; v < V; ++v) {
         if (bias_i != nullptr) fxg[v] += bias_i[c0 + v];
         if (bias_a != nullptr) fag[v] += bias_a[c0 + v];
-        const float s = softplus_precise(lam[c0 + v]);
-        const float i = sigmoid_fast(fxg[v]);
-        const float r = sigmoid_fast(fag[v]);
-        const float alpha = hw_exp2(-8.0f * kLog2e * s * r);
-        const float z = one_minus_exp(-16.0f * s * r);
-        hn[v] = fmaf(alpha, fs[v], hw_sqrt(z) * (i * fx[v]));
+        hn[v] = rglru_step_value(fx[v], fxg[v], fag[v], softplus_precise(lam[c0 + v]), fs[v]);
     }
     eraw_t rh;
     sraw_t rs;
@@ -116,11 +111,7 @@ __global__ __launch_bounds__(256) void rglru_step_kernel(const ET* __restrict__ 
         float fy[V], g[V];
         unpack(load_raw<ET, V>(y + (size_t)b * ldy + c0), fy);
 #pragma unroll
-        for (int v = 0; v < V; ++v) {
-            float cdf, e;
-            normal_cdf<true>(fy[v], cdf, e);
-            g[v] = (fy[v] * cdf) * hn[v];
-        }
+        for (int v = 0; v < V; ++v) g[v] = gelu_times(fy[v], hn[v]);
         eraw_t ro;
         pack(g, ro);
         *reinterpret_cast<eraw_t*>(out + o) = ro;

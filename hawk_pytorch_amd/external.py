@@ -254,6 +254,70 @@ def rglru_step_gated(x, x_rg_lru, a_rg_lru, a_param, recc_state, y, bias_i=None,
     return out.reshape(shape)
 
 
+def decode_core_supported(x_new: torch.Tensor, conv: "Conv1D", gate: "BlockDiagonalLinear",
+                          conv_state: torch.Tensor) -> bool:
+    """Whether ``decode_core_step`` serves these operands: bf16 activations and conv window, a
+    block width of 32..256 (the fused projections' rule) and a window of at most 8 rows."""
+    if x_new.device.type != "cuda" or x_new.dtype != torch.bfloat16 or conv_state.dtype != torch.bfloat16:
+        return False
+    if gate.w.dtype not in (torch.bfloat16, torch.float32):
+        return False
+    W = conv.w.shape[0]
+    return (1 <= W <= MAX_TEMPORAL_WIDTH and gate.width % gate.num_blocks == 0
+            and gate.block_width in _GATE_BLOCK_WIDTHS)
+
+
+def decode_core_step(conv_state, x_new, conv: "Conv1D", input_gate: "BlockDiagonalLinear",
+                     a_gate: "BlockDiagonalLinear", a_param, recc_state, y):
+    """One decode step of a Hawk block's recurrent core in one launch.
+
+    ``conv_state`` [B, W-1, D] is rolled in place and ``recc_state`` [B, 1, D] or [B, D] is
+    overwritten with the new state; returns ``gelu(y) * h`` in x_new's shape.  Same result
+    (to the last bit or two of bf16) as ``temporal_conv1d_step`` + ``gate_projections`` +
+    ``rglru_step_gated``; upstream: hawk/hawk.py:134-151, :169-182, :196-198 and
+    hawk/cache.py:29-43.  ``x_new`` and ``y`` may be the two halves of the input projection,
+    passed in place.
+    """
+    W, D = conv.w.shape
+    shape = x_new.shape
+    B = x_new.numel() // D
+    assert conv_state.shape == (B, W - 1, D) and conv_state.is_contiguous(), (
+        f"conv_state must be a contiguous [B, W-1, D] = {(B, W - 1, D)}, got {tuple(conv_state.shape)}"
+    )
+    assert recc_state.numel() == B * D and recc_state.is_contiguous()
+    assert x_new.dtype == torch.bfloat16 and conv_state.dtype == torch.bfloat16, "the fused step runs on bf16"
+    dev = _lib.require_cuda(conv_state, x_new, conv.w, input_gate.w, a_gate.w, a_param, recc_state, y)
+
+    def rows(t):
+        """[B, D] view with unit column stride and its row stride, copying only if it must."""
+        t2 = t.reshape(B, D) if t.dtype == torch.bfloat16 else t.reshape(B, D).to(torch.bfloat16)
+        if t2.stride(1) != 1 or (B > 1 and t2.stride(0) < D):
+            t2 = t2.contiguous()
+        return t2, (t2.stride(0) if B > 1 else D)
+
+    xn, ldx = rows(x_new)
+    if ldx % 8 != 0 or xn.data_ptr() % 16 != 0:
+        xn, ldx = _lib.dense16(xn.contiguous()), D
+    y2, ldy = rows(y)
+    w32, b32 = _lib.dense16(conv.w.detach().float()), _lib.dense16(conv.b.detach().float())
+    w_i, w_a = _lib.dense16(input_gate.w.detach()), _lib.dense16(a_gate.w.detach())
+    if w_a.dtype != w_i.dtype:
+        w_a = w_a.to(w_i.dtype)
+    b_i = _lib.dense16(input_gate.b.detach().float().reshape(D))
+    b_a = _lib.dense16(a_gate.b.detach().float().reshape(D))
+    lam = _lib.dense16(a_param.detach().float())
+    out = torch.empty((B, D), dtype=torch.bfloat16, device=dev)
+    with torch.cuda.device(dev):
+        status = _lib.load().hawk_decode_core_step(
+            conv_state.data_ptr(), xn.data_ptr(), ldx, w32.data_ptr(), b32.data_ptr(), w_i.data_ptr(),
+            b_i.data_ptr(), w_a.data_ptr(), b_a.data_ptr(), lam.data_ptr(), y2.data_ptr(), ldy,
+            recc_state.data_ptr(), out.data_ptr(), B, D, input_gate.num_blocks, W, _lib.HAWK_DTYPE_BF16,
+            _lib.dtype_code(w_i.dtype), _lib.dtype_code(recc_state.dtype), _lib.stream_ptr(dev),
+        )
+    _lib.check("hawk_decode_core_step", status)
+    return out.reshape(shape)
+
+
 # ---------------------------------------------------------------------------------------
 # Pieces of the harness model that are not on the hot path (library GEMMs, initialisers).
 # ---------------------------------------------------------------------------------------

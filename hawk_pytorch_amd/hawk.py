@@ -31,6 +31,8 @@ from .cache import RNNCache
 from .external import (
     BlockDiagonalLinear,
     Conv1D,
+    decode_core_step,
+    decode_core_supported,
     gate_projections,
     gate_projections_supported,
     rglru_step,
@@ -58,6 +60,9 @@ class HawkConfig:
     # not an upstream field: both gate projections in one matrix-core kernel when the arithmetic
     # is bf16 anyway (bf16 tensors or bf16 autocast); hawk/hawk.py:181-182
     fused_gates: bool = True
+    # not an upstream field: with both of the above, a decode step's conv, projections, state
+    # update and output gate as one launch (hawk/hawk.py:137-151, :169-182, :196-198)
+    fused_decode_core: bool = True
 
     def __post_init__(self):
         if self.post_norm:
@@ -135,6 +140,12 @@ class Hawk(nn.Module):
             fused_gates = self.config.fused_gates and gate_projections_supported(branch, self.rg_lru_input_gate)
             gate_branch = gate_branch[:, -1:, :]
             layer_past.current_cache_size = 1
+            if (fused_gates and self.config.fused_epilogue and self.config.fused_decode_core
+                    and decode_core_supported(branch, self.conv1d, self.rg_lru_input_gate, layer_past.conv_state)):
+                gated = decode_core_step(layer_past.conv_state, branch[:, -1:, :], self.conv1d,
+                                         self.rg_lru_input_gate, self.rg_lru_a_gate, self.rg_lru_a_param,
+                                         layer_past.recc_state, gate_branch)
+                return self.resid_proj(gated), layer_past
             if fused_gates:
                 u = temporal_conv1d_step(layer_past.conv_state, branch[:, -1:, :], self.conv1d.w, self.conv1d.b,
                                          torch.bfloat16)

@@ -200,6 +200,32 @@ int hawk_rglru_step_gated(const void* x, const void* x_rg_lru, const void* a_rg_
  * 32, 64, 128 or 256.  Other shapes stay with the caller's library GEMM. */
 int hawk_gate_proj_supported(int D, int num_blocks);
 
+/* 1 if hawk_decode_core_step serves the shape: a (D, num_blocks) pair the gate projections
+ * serve and a conv window of 1 <= W <= 8 rows. */
+int hawk_decode_core_supported(int D, int num_blocks, int W);
+
+/* One decode step of a layer's whole recurrent core, one launch instead of
+ * hawk_conv1d_step + hawk_gate_proj_fwd + hawk_rglru_step_gated (upstream: the window concat,
+ * RNNCache.update_conv_cache, Conv1D, the two BlockDiagonalLinear calls evaluated twice,
+ * Hawk.inference_prologue, the step, RNNCache.update_cache and Hawk.epilogue's gate:
+ * hawk/hawk.py:134-151, :169-182, :196-198, hawk/cache.py:29-43):
+ *   conv_state [B, W-1, D]  rolled up one row in place, x_new written last
+ *   x_new      [B, D], rows ldx >= D elements apart, ldx a multiple of 8 (the x half of the
+ *              input projection, passed in place); 16-byte aligned
+ *   conv_w [W, D], conv_b [D] fp32; w_i, w_a [num_blocks, bw, bw] of w_dtype (16-byte
+ *              aligned); b_i, b_a [D] fp32 or NULL; a_param [D] fp32
+ *   y          [B, D], rows ldy >= D elements apart (the gate half of the input projection)
+ *   recc_state [B, D] of state_dtype: read, then overwritten with the new state h
+ *   out        [B, D] <- gelu(y) * h
+ * conv_state, x_new, y and out are bf16 (`dtype` must be HAWK_DTYPE_BF16).  The conv output
+ * and the two logits are rounded to bf16 where the three separate calls round them, so both
+ * routes agree to the last bit or two of a bf16 result. */
+int hawk_decode_core_step(void* conv_state, const void* x_new, long long ldx, const float* conv_w,
+                          const float* conv_b, const void* w_i, const float* b_i, const void* w_a,
+                          const float* b_a, const float* a_param, const void* y, long long ldy,
+                          void* recc_state, void* out, int B, int D, int num_blocks, int W,
+                          int dtype, int w_dtype, int state_dtype, void* stream);
+
 /* Both gate logits of M = B*T tokens in one pass over x:
  *   x_rg_lru[m, h*bw+j] = b_i[h*bw+j] + sum_i x[m, h*bw+i] w_i[h, i, j]     (same for a_rg_lru)
  * Replaces the two BlockDiagonalLinear calls of hawk/hawk.py:181-182 (einsum + bias,

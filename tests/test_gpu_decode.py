@@ -117,3 +117,61 @@ def test_prefill_then_steps_track_the_full_scan(dtype):
     for k in range(K):
         y = capi.conv_step(conv_state, d[0][:, T + k].contiguous(), w, b)
         assert max_rel(capi.to_np(y), capi.to_np(y_full[:, T + k])) < TOL[dtype]
+
+
+def _core_operands(B, D, nb, W, w_dtype, state_dtype, seed):
+    rng = np.random.default_rng(seed)
+    bw = D // nb
+    wide = capi.to_dev(rng.standard_normal((B, 2 * D)), "bf16")   # the input projection: [x | y]
+    conv_state = capi.to_dev(rng.standard_normal((B, W - 1, D)), "bf16")
+    conv_w = capi.to_dev(rng.standard_normal((W, D)) * 0.5, "f32")
+    conv_b = capi.to_dev(rng.standard_normal(D) * 0.1, "f32")
+    w_i = capi.to_dev(rng.standard_normal((nb, bw, bw)) / np.sqrt(bw), w_dtype)
+    w_a = capi.to_dev(rng.standard_normal((nb, bw, bw)) / np.sqrt(bw), w_dtype)
+    b_i = capi.to_dev(rng.standard_normal(D), "f32")
+    b_a = capi.to_dev(rng.standard_normal(D), "f32")
+    lam = capi.to_dev(np.log(np.power(rng.uniform(0.9, 0.999, size=D), -1.0 / 8.0) - 1.0), "f32")
+    state = capi.to_dev(rng.standard_normal((B, D)), state_dtype)
+    return wide, conv_state, conv_w, conv_b, w_i, b_i, w_a, b_a, lam, state
+
+
+@pytest.mark.parametrize("w_dtype,state_dtype", [("bf16", "bf16"), ("f32", "bf16"), ("bf16", "f32"), ("f32", "f32")])
+@pytest.mark.parametrize("B,D,nb,W", [(256, 2560, 10, 4), (1, 2560, 10, 4), (33, 512, 16, 4), (5, 256, 4, 2),
+                                      (70, 256, 2, 8), (3, 64, 2, 1), (64, 1024, 4, 4)])
+def test_decode_core_step_matches_the_three_separate_launches(B, D, nb, W, w_dtype, state_dtype):
+    """One launch against hawk_conv1d_step + hawk_gate_proj_fwd + hawk_rglru_step_gated on the
+    same operands (x and y are the two halves of one [B, 2D] tensor): the conv window exactly,
+    state and output to the last bits of their dtype, over three consecutive tokens."""
+    wide, cs, conv_w, conv_b, w_i, b_i, w_a, b_a, lam, st = _core_operands(B, D, nb, W, w_dtype, state_dtype, B + D + W)
+    cs_ref, st_ref = cs.clone(), st.clone()
+    rng = np.random.default_rng(7)
+    for step in range(3):
+        x_new, y = wide[:, :D], wide[:, D:]
+        out = capi.decode_core_step(cs if W > 1 else None, x_new, conv_w, conv_b, w_i, b_i, w_a, b_a, lam, y, st)
+        u = capi.conv_step(cs_ref, x_new.contiguous(), conv_w, conv_b, torch.bfloat16)
+        xg, ag = capi.gate_proj_fwd(u, w_i, b_i, w_a, b_a, torch.bfloat16)
+        out_ref, _ = capi.rglru_step_gated(u, xg, ag, None, None, lam, y, st_ref)
+        torch.cuda.synchronize()
+        assert torch.equal(cs, cs_ref), step
+        tol = 2.0 ** -7 if state_dtype == "bf16" else 1e-5
+        assert max_rel(capi.to_np(st), capi.to_np(st_ref)) <= tol, step
+        assert max_rel(capi.to_np(out), capi.to_np(out_ref)) <= 2.0 ** -7, step
+        wide = capi.to_dev(rng.standard_normal((B, 2 * D)), "bf16")
+
+
+def test_decode_core_step_against_the_oracle():
+    """The same launch against the fp64 restatement: conv step, block-diagonal projections with
+    their biases, the recurrence and the gate."""
+    B, D, nb, W = 37, 512, 4, 4
+    wide, cs, conv_w, conv_b, w_i, b_i, w_a, b_a, lam, st = _core_operands(B, D, nb, W, "f32", "f32", 99)
+    x_new, y = wide[:, :D], wide[:, D:]
+    n = capi.to_np
+    u_ref, cs_next = oracle.conv1d_step(n(cs), n(x_new), n(conv_w), n(conv_b))
+    xg = oracle.block_diagonal_linear(u_ref, n(w_i), n(b_i))
+    ag = oracle.block_diagonal_linear(u_ref, n(w_a), n(b_a))
+    h_ref = oracle.rglru_step(u_ref, xg, ag, n(lam), n(st))
+    out_ref = oracle.gelu(n(y)) * h_ref
+    out = capi.decode_core_step(cs, x_new, conv_w, conv_b, w_i, b_i, w_a, b_a, lam, y, st)
+    assert np.array_equal(n(cs), cs_next.astype(np.float32))
+    assert max_rel(n(st), h_ref) < TOL["bf16"]
+    assert max_rel(n(out), out_ref) < TOL["bf16"]
