@@ -217,6 +217,61 @@ def test_model_prefill_then_decode_matches_full_forward():
             assert max_rel(capi.to_np(step_logits[:, 0]), capi.to_np(full_logits[:, T + k])) < 1e-3
 
 
+@pytest.mark.parametrize("weights", ["bf16", "f32 under autocast"])
+def test_bf16_decode_takes_the_same_steps_on_every_route(weights):
+    """A bf16 model with a warm cache: the single fused launch per layer, the three launches and
+    the unfused modules must produce the same tokens' logits (to bf16 accuracy) and leave the
+    same caches behind."""
+    cfg = hk.HawkConfig(vocab_size=512, hidden_size=256, intermediate_size=512, num_hidden_layers=3,
+                        recurrent_size=256, num_blocks=2, conv_width=4)
+    torch.manual_seed(2)
+    model = hk.HawkModel(cfg, use_cache=True).cuda().eval()
+    _randomise_zero_inits(model)
+    if weights == "bf16":
+        model = model.to(torch.bfloat16)
+    B, T, K = 5, 33, 4
+    ids = torch.randint(1, cfg.vocab_size, (B, T + K), device="cuda", generator=torch.Generator("cuda").manual_seed(3))
+
+    def run(fused_decode_core, fused_gates):
+        cfg.fused_decode_core, cfg.fused_gates = fused_decode_core, fused_gates
+        out = []
+        with torch.no_grad(), torch.autocast(device_type="cuda", dtype=torch.bfloat16,
+                                             enabled=weights != "bf16"):
+            _, caches = model(ids[:, :T], layer_past=model.new_cache(B))
+            for k in range(K):
+                logits, caches = model(ids[:, T + k: T + k + 1], layer_past=caches)
+                out.append(logits[:, 0].float())
+        return torch.stack(out), caches
+
+    import hawk_pytorch_amd.hawk as hm
+
+    calls = []
+    real = hm.decode_core_step
+
+    def counted(*args, **kwargs):
+        calls.append(1)
+        return real(*args, **kwargs)
+
+    try:
+        hm.decode_core_step = counted
+        one, caches_one = run(True, True)
+        assert len(calls) == K * cfg.num_hidden_layers   # the fused launch is what ran
+        three, caches_three = run(False, True)
+        plain, _ = run(False, False)
+        assert len(calls) == K * cfg.num_hidden_layers
+    finally:
+        hm.decode_core_step = real
+        cfg.fused_decode_core, cfg.fused_gates = True, True
+    assert torch.isfinite(one).all()
+    scale = float(plain.abs().max())
+    assert float((one - three).abs().max()) < 2e-2 * scale
+    assert float((one - plain).abs().max()) < 4e-2 * scale
+    for a, b in zip(caches_one, caches_three):
+        assert torch.equal(a.conv_state, b.conv_state)
+        assert float((a.recc_state.float() - b.recc_state.float()).abs().max()) < 2e-2 * float(
+            b.recc_state.float().abs().max())
+
+
 @pytest.mark.parametrize("fused_epilogue", [True, False])
 def test_model_gradients_match_a_pure_torch_model_of_the_same_weights(fused_epilogue):
     """End-to-end fwd+bwd of the small model in fp32 against the same model with the scan
