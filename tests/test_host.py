@@ -273,3 +273,35 @@ def test_argument_validation_of_the_gated_and_projection_entry_points():
         == E.HAWK_ERR_WORKSPACE
     assert lib.hawk_gate_proj_bwd_weights_workspace_bytes(32768, 2560, 10) > 0
     assert lib.hawk_gate_proj_bwd_weights_workspace_bytes(32768, 2560, 7) == 0
+
+
+def test_argument_validation_of_the_fused_decode_step():
+    lib = _lib.load()
+    buf = (ctypes.c_char * 4096)()
+    p = (ctypes.addressof(buf) + 15) & ~15
+    E = _lib
+    # (conv_state, x_new, ldx, conv_w, conv_b, w_i, b_i, w_a, b_a, a_param, y, ldy, recc_state, out,
+    #  B, D, num_blocks, W, dtype, w_dtype, state_dtype, stream)
+    ok = [p, p, 512, p, p, p, None, p, None, p, p, 512, p, p, 1, 256, 2, 4, 0, 0, 0, None]
+
+    def step(**kw):
+        a = list(ok)
+        for k, v in kw.items():
+            a[int(k[1:])] = v
+        return lib.hawk_decode_core_step(*a)
+
+    assert step(a1=None) == E.HAWK_ERR_NULL_POINTER          # x_new
+    assert step(a0=None) == E.HAWK_ERR_NULL_POINTER          # a window of 3 rows needs its state
+    assert step(a0=None, a17=1, a1=p + 2) == E.HAWK_ERR_ALIGNMENT  # no window, no state: the next check fails
+    assert step(a18=1) == E.HAWK_ERR_BAD_DTYPE               # activations must be bf16
+    assert step(a19=7) == E.HAWK_ERR_BAD_DTYPE
+    assert step(a17=9) == E.HAWK_ERR_BAD_SHAPE               # window too wide
+    assert step(a16=3) == E.HAWK_ERR_BAD_SHAPE               # 256 channels do not split in 3 blocks
+    assert step(a2=255) == E.HAWK_ERR_BAD_SHAPE              # row stride below D
+    assert step(a2=260) == E.HAWK_ERR_BAD_SHAPE              # rows of x_new must stay 16-byte aligned
+    assert step(a11=100) == E.HAWK_ERR_BAD_SHAPE
+    assert step(a1=p + 2) == E.HAWK_ERR_ALIGNMENT
+    assert step(a10=p + 1) == E.HAWK_ERR_ALIGNMENT           # y must be element aligned
+    assert lib.hawk_decode_core_supported(2560, 10, 4) == 1
+    assert lib.hawk_decode_core_supported(2560, 10, 9) == 0
+    assert lib.hawk_decode_core_supported(2560, 7, 4) == 0
