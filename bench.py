@@ -83,7 +83,7 @@ def lambda_for_a8_range(gen, D, lo, hi):
     return torch.log(u.pow(-1.0 / 8.0) - 1.0).float()
 
 
-def cpu_baseline(B, D, lo, hi, seed, budget_elements=1536 * 8 * 2560):
+def cpu_baseline(B, D, lo, hi, seed, budget_elements=1024 * 8 * 2560):
     """PyTorch CPU loop (oracle/rglru_torch.py) on the first time rows of the workload's shape,
     about `budget_elements` element-steps (10-20 s on 16 host threads): forward plus autograd
     backward in fp32."""
