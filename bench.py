@@ -56,10 +56,10 @@ HBM_PEAK_GBS = 8000.0
 # Sources: profiles/rglru_scan_B8_T4096_D2560_bf16.md, profiles/rglru_scan_B2_T32768_D4096_bf16.md,
 # profiles/rglru_scan_gated_B8_T4096_D2560_bf16.md.
 MEASURED_BWD_TRAFFIC_BYTES = {
-    "scan": 865.4e6 + 533.0e6,
-    "scan_conv": 865.4e6 + 533.0e6,
+    "scan": 876.9e6 + 545.0e6,
+    "scan_conv": 876.9e6 + 545.0e6,
     "long": 2776.5e6 + 1711.7e6,
-    "scan_gated": 1043.5e6 + 704.8e6,
+    "scan_gated": 1050.4e6 + 712.7e6,
 }
 
 # The same for the gates workload's dominant launch (weight-gradient kernel + its reduce kernel):

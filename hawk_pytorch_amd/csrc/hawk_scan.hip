@@ -783,6 +783,18 @@ constexpr int kBwdTC = HAWK_BWD_TC, kBwdNW = HAWK_BWD_NW;
 // with two channels per lane the gate's operands cost two more registers per row and the tile
 // is two rows shorter; with one channel per lane the plain kernel's tile height still fits
 constexpr int kBwdGatedTC = HAWK_BWD_GATED_TC, kBwdGatedTC1 = HAWK_BWD_GATED_TC1;
+// With many independent chains in a launch (B x channel tiles) the backward runs 1-3 % faster on
+// 64-row tiles: more, shorter-lived tiles, and enough chains to keep the memory system busy
+// while each waits on its carry.  With few chains the longer carry chain of short tiles
+// costs more than that (4 % at B=2, T=32768, D=4096), so those keep the tall tiles.
+#ifndef HAWK_BWD_MANY_TC
+#define HAWK_BWD_MANY_TC 8
+#endif
+#ifndef HAWK_BWD_MANY_CHAINS
+#define HAWK_BWD_MANY_CHAINS 128
+#endif
+constexpr int kBwdManyTC = HAWK_BWD_MANY_TC;
+constexpr int kManyChains = HAWK_BWD_MANY_CHAINS;
 constexpr int kFwdGatedTC = HAWK_FWD_GATED_TC;  // two channels per lane; one channel keeps kFwdTC
 
 #ifndef HAWK_MAX_V
@@ -791,9 +803,14 @@ constexpr int kFwdGatedTC = HAWK_FWD_GATED_TC;  // two channels per lane; one ch
 int pick_v(int D, int dtype) { return (HAWK_MAX_V >= 2 && dtype == HAWK_DTYPE_BF16 && (D % 2) == 0) ? 2 : 1; }
 
 TileShape fwd_shape(int D, int dtype) { return TileShape{pick_v(D, dtype), kFwdTC, kFwdNW}; }
-TileShape bwd_shape(int D, int dtype) { return TileShape{pick_v(D, dtype), kBwdTC, kBwdNW}; }
+bool many_chains(int B, int D, int V) { return (long long)B * ((D + kWave * V - 1) / (kWave * V)) >= kManyChains; }
+TileShape bwd_shape(int D, int dtype, bool many) {
+    return TileShape{pick_v(D, dtype), many ? kBwdManyTC : kBwdTC, kBwdNW};
+}
 TileShape fwd_gated_shape(int V) { return TileShape{V, V == 2 ? kFwdGatedTC : kFwdTC, kFwdNW}; }
-TileShape bwd_gated_shape(int V) { return TileShape{V, V == 2 ? kBwdGatedTC : kBwdGatedTC1, kBwdNW}; }
+TileShape bwd_gated_shape(int V, bool many) {
+    return TileShape{V, many ? kBwdManyTC : (V == 2 ? kBwdGatedTC : kBwdGatedTC1), kBwdNW};
+}
 
 int ceil_div(int a, int b) { return (a + b - 1) / b; }
 
@@ -906,17 +923,13 @@ int scan_fwd_impl(const void* x, const void* xg, const void* ag, const float* la
     return launch_fwd<float, float, 1, kFwdTC, kFwdNW, true, GATED>(x, xg, ag, lam, h, g, B, T, D, nseg, nct, p, st);
 }
 
-template <bool GATED>
-int scan_bwd_impl(const void* x, const void* xg, const void* ag, const float* lam, const void* hs, const void* gout,
-                  void* dx, void* dxg, void* dag, float* dlam, const GateBwdHost& g, int B, int T, int D,
-                  int in_dtype, int state_dtype, void* ws, size_t ws_bytes, hipStream_t st) {
-    constexpr int TC2 = GATED ? kBwdGatedTC : kBwdTC, TC1 = GATED ? kBwdGatedTC1 : kBwdTC;
-    TileShape s = bwd_shape(D, in_dtype);
-    if (GATED) {
-        const bool pairs_aligned = (g.ldy % 2) == 0 && (g.lddy % 2) == 0 &&
-                                   ((reinterpret_cast<uintptr_t>(g.y) | reinterpret_cast<uintptr_t>(g.dy)) & 3u) == 0;
-        s = bwd_gated_shape(pairs_aligned ? s.V : 1);
-    }
+template <bool GATED, bool MANY>
+int scan_bwd_shaped(const void* x, const void* xg, const void* ag, const float* lam, const void* hs, const void* gout,
+                    void* dx, void* dxg, void* dag, float* dlam, const GateBwdHost& g, int B, int T, int D,
+                    int in_dtype, int state_dtype, int V, void* ws, size_t ws_bytes, hipStream_t st) {
+    constexpr int TC2 = MANY ? kBwdManyTC : (GATED ? kBwdGatedTC : kBwdTC);
+    constexpr int TC1 = MANY ? kBwdManyTC : (GATED ? kBwdGatedTC1 : kBwdTC);
+    const TileShape s = GATED ? bwd_gated_shape(V, MANY) : TileShape{V, MANY ? kBwdManyTC : kBwdTC, kBwdNW};
     const int nseg = ceil_div(T, s.rows());
     const int nct = ceil_div(D, s.chans());
     const WsLayout l = layout_for(B, D, nseg, nseg);
@@ -943,12 +956,31 @@ int scan_bwd_impl(const void* x, const void* xg, const void* ag, const float* la
     return hipGetLastError() == hipSuccess ? HAWK_OK : HAWK_ERR_LAUNCH;
 }
 
+template <bool GATED>
+int scan_bwd_impl(const void* x, const void* xg, const void* ag, const float* lam, const void* hs, const void* gout,
+                  void* dx, void* dxg, void* dag, float* dlam, const GateBwdHost& g, int B, int T, int D,
+                  int in_dtype, int state_dtype, void* ws, size_t ws_bytes, hipStream_t st) {
+    int V = pick_v(D, in_dtype);
+    if (GATED) {
+        const bool pairs_aligned = (g.ldy % 2) == 0 && (g.lddy % 2) == 0 &&
+                                   ((reinterpret_cast<uintptr_t>(g.y) | reinterpret_cast<uintptr_t>(g.dy)) & 3u) == 0;
+        if (!pairs_aligned) V = 1;
+    }
+    if (many_chains(B, D, V))
+        return scan_bwd_shaped<GATED, true>(x, xg, ag, lam, hs, gout, dx, dxg, dag, dlam, g, B, T, D, in_dtype,
+                                            state_dtype, V, ws, ws_bytes, st);
+    return scan_bwd_shaped<GATED, false>(x, xg, ag, lam, hs, gout, dx, dxg, dag, dlam, g, B, T, D, in_dtype,
+                                         state_dtype, V, ws, ws_bytes, st);
+}
+
 }  // namespace
 
 size_t scan_workspace_bytes(int B, int T, int D, int dtype) {
     // one size serves every scan entry point: the longest chain (shortest tile) decides
-    const int rows[6] = {fwd_shape(D, dtype).rows(), fwd_gated_shape(1).rows(),   fwd_gated_shape(2).rows(),
-                         bwd_shape(D, dtype).rows(), bwd_gated_shape(1).rows(),   bwd_gated_shape(2).rows()};
+    const int V = pick_v(D, dtype);
+    const bool many1 = many_chains(B, D, 1), manyv = many_chains(B, D, V);
+    const int rows[6] = {fwd_shape(D, dtype).rows(),        fwd_gated_shape(1).rows(),       fwd_gated_shape(2).rows(),
+                         bwd_shape(D, dtype, manyv).rows(), bwd_gated_shape(1, many1).rows(), bwd_gated_shape(2, manyv).rows()};
     int n_chain = 0, n_dlam = 0;
     for (int k = 0; k < 6; ++k) {
         const int n = ceil_div(T, rows[k]);
