@@ -83,8 +83,14 @@ __device__ __forceinline__ bool try_read(const unsigned long long* p, uint32_t t
 // tiles) to keep the memory system busy while each chain waits on its hops, 8 when there are
 // few and the hops themselves set the pace (one long sequence of a narrow model: 8 chains run
 // 22 % faster, 16 chains 4 %); with 60 or more chains the wider window costs 2-3 % instead.
+// With 128 or more chains the distance is 2: a tile then reads at most two predecessors'
+// words, and even at one memory round trip per two positions the chain stays ahead of the
+// rate at which the launch gets through a position of all its chains (0.5 % faster).
 constexpr int kMaxLookback = 8;
 constexpr int kFewChains = 24;
+#ifndef HAWK_LOOKBACK_MANY
+#define HAWK_LOOKBACK_MANY 2
+#endif
 
 __device__ __forceinline__ bool is_checkpoint(int pos, int lookback) { return (pos & (lookback - 1)) == 0; }
 __device__ __forceinline__ int checkpoint_before(int pos, int lookback) { return (pos - 1) & ~(lookback - 1); }
@@ -831,7 +837,8 @@ int lookback_for(int B, int nct) {
 #ifdef HAWK_LOOKBACK
     return HAWK_LOOKBACK;
 #else
-    return (long long)B * nct <= kFewChains ? kMaxLookback : 4;
+    const long long chains = (long long)B * nct;
+    return chains <= kFewChains ? kMaxLookback : (chains >= kManyChains ? HAWK_LOOKBACK_MANY : 4);
 #endif
 }
 ScanWsPtrs carve(void* ws, const WsLayout& l, int lookback) {
