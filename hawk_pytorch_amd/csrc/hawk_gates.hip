@@ -470,8 +470,8 @@ __global__ __launch_bounds__(kCoreWaves* kWave, 1) void decode_core_kernel(
     bf16_t* __restrict__ conv_state, const bf16_t* __restrict__ x_new, size_t ldx, const float* __restrict__ conv_w,
     const float* __restrict__ conv_b, const WT* __restrict__ w_i, const float* __restrict__ b_i,
     const WT* __restrict__ w_a, const float* __restrict__ b_a, const float* __restrict__ lam,
-    const bf16_t* __restrict__ y, size_t ldy, ST* __restrict__ state, bf16_t* __restrict__ out, int M, int D, int nb,
-    int W, int ntiles) {
+    const bf16_t* __restrict__ y, size_t ldy, ST* __restrict__ state, bf16_t* __restrict__ out, int M, int D, int W,
+    int ntiles) {
     static_assert(BW % 32 == 0 && BW <= 32 * kCoreWaves, "one wave per 32 output columns of a block");
     constexpr int KS = BW / 16;
     constexpr int NT = BW / 32;
@@ -1113,7 +1113,7 @@ int launch_decode_core(void* conv_state, const void* x_new, long long ldx, const
                        static_cast<bf16_t*>(conv_state), static_cast<const bf16_t*>(x_new), (size_t)ldx, conv_w,
                        conv_b, static_cast<const WT*>(w_i), b_i, static_cast<const WT*>(w_a), b_a, lam,
                        static_cast<const bf16_t*>(y), (size_t)ldy, static_cast<ST*>(state), static_cast<bf16_t*>(out),
-                       B, D, nb, W, ntiles);
+                       B, D, W, ntiles);
     return hipGetLastError() == hipSuccess ? HAWK_OK : HAWK_ERR_LAUNCH;
 }
 
