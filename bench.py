@@ -22,6 +22,10 @@ on a 1 x 2048 batch under bf16 autocast, with and without the fused gate / epilo
 10 gate blocks, vocabulary 32000, bf16 weights) at batch 256 after a 1024-token prefill,
 eagerly and as a replayed HIP graph, plus the two hot-path kernels of a layer on their own.
 
+The kernel workloads (scan*, long, gates, block) run ``--settle-steps`` untimed steps (default 100)
+before the ``--warmup`` ones: for about 50 steps (20 ms) after the GPU leaves idle the same kernels
+run up to 12 % slower than they do from then on.
+
 Prints one JSON line:
   value        tokens/s = B*T / (wall time per step), whole job on one GPU
   roofline     for the dominant kernel (the backward scan): algorithmic bytes per launch
@@ -144,7 +148,7 @@ def run_gates(args, lib, dev):
         for _ in range(3):
             oi.copy_(x)
         torch.cuda.synchronize()
-    for _ in range(args.warmup):
+    for _ in range(args.settle_steps + args.warmup):
         fwd(), bwd_input(), bwd_weights()
     torch.cuda.synchronize()
     ev = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(args.steps)]
@@ -170,7 +174,8 @@ def run_gates(args, lib, dev):
         "metric": "fused gate projections fwd+bwd tokens/s, 1 GPU",
         "value": M / (ms_per_step * 1e-3),
         "unit": "tokens/s",
-        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step,
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "settle_steps": args.settle_steps,
+        "ms_per_step": ms_per_step,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16 operands, f32 accumulation",
         "data": f"synthetic, seed {args.seed}: activations and gradients ~ N(0,1), weights ~ N(0, 1/bw)",
@@ -238,7 +243,7 @@ def run_block(args, lib, dev):
         _lib.check("conv_bwd", lib.hawk_conv1d_bwd(p(du), p(xin), p(cw), p(dxin), p(dcw), p(dcb), B, T, D, W, code,
                                                    code, p(cws), cws.numel(), st))
 
-    for _ in range(args.warmup):
+    for _ in range(args.settle_steps + args.warmup):
         fwd(), bwd()
     torch.cuda.synchronize()
     ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
@@ -263,7 +268,8 @@ def run_block(args, lib, dev):
     print(json.dumps({
         "metric": "Hawk recurrent core (conv, gate projections, gated scan) fwd+bwd tokens/s, 1 GPU",
         "value": B * T / (ms_per_step * 1e-3), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
-        "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak",
+        "warmup": args.warmup, "settle_steps": args.settle_steps, "ms_per_step": ms_per_step,
+        "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "bf16 activations, f32 parameters, state and accumulation",
         "data": f"synthetic, seed {args.seed}",
         "config": {"workload": f"block: conv1d(4) + gate projections ({nb} blocks) + scan fused with gelu(y)*h, "
@@ -500,8 +506,10 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=100,
-                    help="untimed steps; kernel durations settle about 50 steps (20 ms) after the GPU leaves idle")
+    ap.add_argument("--warmup", type=int, default=10, help="untimed steps before the timed ones")
+    ap.add_argument("--settle-steps", type=int, default=100,
+                    help="further untimed steps run before the warm-up in the kernel workloads (scan*, long, gates, "
+                         "block): kernel durations settle about 50 steps (20 ms) after the GPU leaves idle")
     ap.add_argument("--workload", choices=sorted(WORKLOADS) + ["block", "decode", "gates", "model"], default="scan")
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -619,7 +627,7 @@ def main():
             h.copy_(x)  # reads 2*N bytes, writes 2*N bytes
         torch.cuda.synchronize()
 
-    for _ in range(args.warmup):
+    for _ in range(args.settle_steps + args.warmup):
         fwd()
         bwd()
         if with_conv:
@@ -670,6 +678,7 @@ def main():
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
+        "settle_steps": args.settle_steps,
         "ms_per_step": ms_per_step,
         "higher_is_better": True,
         "scaling": "weak",
