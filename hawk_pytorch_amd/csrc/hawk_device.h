@@ -23,6 +23,7 @@ typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x8 __attribute__((ext_vector_type(8)));
 
 // Two fp32 -> packed bf16 pair, round-to-nearest-even (one v_cvt_pk_bf16_f32 on gfx950).
 __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
@@ -63,6 +64,8 @@ template <>
 struct Raw<float, 2> { typedef f32x2 type; };
 template <>
 struct Raw<float, 4> { typedef f32x4 type; };
+template <>
+struct Raw<float, 8> { typedef f32x8 type; };
 
 __device__ __forceinline__ void unpack(uint16_t r, float (&o)[1]) { o[0] = __uint_as_float((uint32_t)r << 16); }
 __device__ __forceinline__ void unpack(uint32_t r, float (&o)[2]) { o[0] = bf16_lo(r); o[1] = bf16_hi(r); }
@@ -76,6 +79,10 @@ __device__ __forceinline__ void unpack(u32x4 r, float (&o)[8]) {
 __device__ __forceinline__ void unpack(float r, float (&o)[1]) { o[0] = r; }
 __device__ __forceinline__ void unpack(f32x2 r, float (&o)[2]) { o[0] = r.x; o[1] = r.y; }
 __device__ __forceinline__ void unpack(f32x4 r, float (&o)[4]) { o[0] = r.x; o[1] = r.y; o[2] = r.z; o[3] = r.w; }
+__device__ __forceinline__ void unpack(f32x8 r, float (&o)[8]) {
+#pragma unroll
+    for (int k = 0; k < 8; ++k) o[k] = r[k];
+}
 
 __device__ __forceinline__ void pack(const float (&v)[1], uint16_t& r) { r = to_bf16_bits(v[0]); }
 __device__ __forceinline__ void pack(const float (&v)[2], uint32_t& r) { r = pack_bf16x2(v[0], v[1]); }
@@ -89,6 +96,10 @@ __device__ __forceinline__ void pack(const float (&v)[8], u32x4& r) {
 __device__ __forceinline__ void pack(const float (&v)[1], float& r) { r = v[0]; }
 __device__ __forceinline__ void pack(const float (&v)[2], f32x2& r) { r.x = v[0]; r.y = v[1]; }
 __device__ __forceinline__ void pack(const float (&v)[4], f32x4& r) { r.x = v[0]; r.y = v[1]; r.z = v[2]; r.w = v[3]; }
+__device__ __forceinline__ void pack(const float (&v)[8], f32x8& r) {
+#pragma unroll
+    for (int k = 0; k < 8; ++k) r[k] = v[k];
+}
 
 template <typename R>
 __device__ __forceinline__ R raw_zero() {

@@ -435,19 +435,23 @@ __global__ __launch_bounds__(kSmallWaves* kWave, sizeof(XT) == 2 ? 4 : 2) void g
 //   2. wave c < bw/32: the bw x 32 slices of both weight matrices that produce output columns
 //      32c.. of the block, transposed through a wave-private LDS region into B operands, one
 //      gate after the other (the second gate's weights travel while the first is multiplied);
-//   3. the same wave: biases, recurrence and gate on its 32 x 32 outputs straight from the
-//      accumulators; recc_state is updated in place.
+//   3. the same wave adds the biases and leaves its 32 x 32 logits in LDS as bf16, over the
+//      weights, which are done with by then;
+//   4. all waves: recurrence and output gate, thread -> (row, 8 consecutive channels) with
+//      16-byte accesses to y, recc_state (updated in place) and out.  (Applied straight to the
+//      accumulators, with 2-byte gathers and scatters per element, this step alone made the
+//      kernel 13 us slower at a block width of 32 and 2 us at 128.)
 // Intermediate roundings are those of the three separate launches (conv output and logits to
-// bf16), so the two paths agree to the last bit or two of a bf16 result.
-// Where its time goes at 256 rows and a block width of 256 (19.5 us, as long as the three
-// launches it replaces; 10 us against 14.5 at a width of 128): 8.7 us for the launch, staging, matrix
-// products, operand loads and stores; 4.8 us fetching a block's 256 KiB of weights into one compute
-// unit (fetching the second gate's earlier does not shorten it); 2.9 us for the conv; 1.6 us
-// for the recurrence and gate.  One workgroup per (32 rows, block) is 80 workgroups here: what
-// the launch saves in starts it loses to running on a third of the device, so its gain is on
-// the host side (one call instead of three plus a copy).  Cutting a block's columns over more
-// workgroups would need the window roll out of the kernel: they would read rows that another
-// of them overwrites.
+// bf16), so the two paths give the same bits.
+// At 256 rows, replayed from a graph: 18.6 us at a block width of 256 against 19.4 us for the
+// three launches it replaces, 8.4 against 14.5 us at a width of 128, 8.9 against 14.1 us at 32.
+// At 256 the time is the launch, staging, matrix products, operand loads and stores (8 us),
+// fetching a block's 256 KiB of weights into one compute unit (4.8 us; fetching the second
+// gate's earlier does not shorten it), the conv (2.9 us) and the recurrence (1.6 us).  One
+// workgroup per (32 rows, block) is 80 workgroups there: what the launch saves in starts it
+// loses to running on a third of the device, and its gain is on the host side (one call
+// instead of three plus a copy).  Cutting a block's columns over more workgroups would need the
+// window roll out of the kernel: they would read rows that another of them overwrites.
 // ---------------------------------------------------------------------------------------
 constexpr int kCoreWaves = 8;
 constexpr int kCoreMaxW = 8;
@@ -458,7 +462,10 @@ struct CoreLds {
     static constexpr int kUBytes = kTileRows * kRowBytes;               // conv output tile
     static constexpr int kWaveBytes = 32 * kRowBytes;                   // one wave's 32 weight columns
     static constexpr int kWaves = BW / 32 < kCoreWaves ? BW / 32 : kCoreWaves;
-    static constexpr int kBytes = kUBytes + kWaves * kWaveBytes;
+    static constexpr int kORowBytes = 2 * BW * 2 + 16;                  // both gates' logits of one row + pad
+    static constexpr int kWeightBytes = kWaves * kWaveBytes;
+    static constexpr int kLogitBytes = kTileRows * kORowBytes;          // reuses the weights' space
+    static constexpr int kBytes = kUBytes + (kWeightBytes > kLogitBytes ? kWeightBytes : kLogitBytes);
 };
 
 // all LDS traffic of this wave issued so far has completed, and the compiler keeps what
@@ -471,7 +478,7 @@ __global__ __launch_bounds__(kCoreWaves* kWave, 1) void decode_core_kernel(
     const float* __restrict__ conv_b, const WT* __restrict__ w_i, const float* __restrict__ b_i,
     const WT* __restrict__ w_a, const float* __restrict__ b_a, const float* __restrict__ lam,
     const bf16_t* __restrict__ y, size_t ldy, ST* __restrict__ state, bf16_t* __restrict__ out, int M, int D, int W,
-    int ntiles) {
+    int ntiles, bool vec_io) {
     static_assert(BW % 32 == 0 && BW <= 32 * kCoreWaves, "one wave per 32 output columns of a block");
     constexpr int KS = BW / 16;
     constexpr int NT = BW / 32;
@@ -562,64 +569,112 @@ __global__ __launch_bounds__(kCoreWaves* kWave, 1) void decode_core_kernel(
 
     // ---- 2. gate projections of this wave's 32 output columns
     const int col = lane & 31, khalf = 8 * (lane >> 5);
-    const int c_out = h * BW + (computes ? w : 0) * 32 + col;      // this lane's channel
-    const int row0 = rt * kTileRows + 4 * (lane >> 5);             // accumulator r: row0 + 8 (r / 4) + r % 4
-    typedef typename Raw<ST, 1>::type sraw_t;
-    uint16_t ybits[16];
-    sraw_t sold[16];
+    // softplus(Lambda) of the block's channels, once per workgroup
+    float* sSp = reinterpret_cast<float*>(core_smem + CoreLds<BW>::kBytes);
+    if (tid < BW) sSp[tid] = softplus_precise(lam[h * BW + tid]);
     if (computes) {
         stage_weights();
         fetch_weights(w_a);
-        // operands of the recurrence travel during the matrix products
+    }
+    wave_lds_fence();
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+
+    f32x16 acc_i = {}, acc_a = {};
+    if (computes) {
+        const unsigned char* asrc = sU + col * kRowBytes + khalf * 2;
+        const unsigned char* bsrc = sW + col * kRowBytes + khalf * 2;
+#pragma unroll
+        for (int s = 0; s < KS; ++s)
+            acc_i = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*reinterpret_cast<const bf16x8*>(asrc + 32 * s),
+                                                            *reinterpret_cast<const bf16x8*>(bsrc + 32 * s), acc_i, 0, 0,
+                                                            0);
+        wave_lds_fence();   // the first gate's operands have been read: the region can be overwritten
+        stage_weights();
+        wave_lds_fence();
+#pragma unroll
+        for (int s = 0; s < KS; ++s)
+            acc_a = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*reinterpret_cast<const bf16x8*>(asrc + 32 * s),
+                                                            *reinterpret_cast<const bf16x8*>(bsrc + 32 * s), acc_a, 0, 0,
+                                                            0);
+    }
+
+    // ---- 3. the logits (biases added, rounded to bf16) go to LDS over the weights, which every
+    //         wave has finished with, so that the recurrence can run on all threads with 16-byte
+    //         accesses: thread -> (row, 8 consecutive channels), as in the conv
+    constexpr int kORowBytes = CoreLds<BW>::kORowBytes;
+    unsigned char* sO = core_smem + CoreLds<BW>::kUBytes;
+    wave_lds_fence();
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    if (computes) {
+        const int c_out = h * BW + w * 32 + col;
+        const float bias_i = b_i != nullptr ? b_i[c_out] : 0.0f;
+        const float bias_a = b_a != nullptr ? b_a[c_out] : 0.0f;
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-            const int row = row0 + 8 * (r / 4) + (r % 4);
-            const bool ok = row < M;
-            ybits[r] = ok ? load_raw<bf16_t, 1>(y + (size_t)row * ldy + c_out) : (uint16_t)0;
-            sold[r] = ok ? load_raw<ST, 1>(state + (size_t)row * D + c_out) : raw_zero<sraw_t>();
+            const int rl = 4 * (lane >> 5) + 8 * (r / 4) + (r % 4);
+            unsigned char* o = sO + rl * kORowBytes + (w * 32 + col) * 2;
+            *reinterpret_cast<uint16_t*>(o) = to_bf16_bits(acc_i[r] + bias_i);
+            *reinterpret_cast<uint16_t*>(o + BW * 2) = to_bf16_bits(acc_a[r] + bias_a);
         }
     }
     wave_lds_fence();
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
-    if (!computes) return;
 
-    const unsigned char* asrc = sU + col * kRowBytes + khalf * 2;
-    const unsigned char* bsrc = sW + col * kRowBytes + khalf * 2;
-    f32x16 acc_i = {}, acc_a = {};
+    // ---- 4. recurrence and output gate
+    {
+        typedef typename Raw<ST, 8>::type sraw8_t;
+        constexpr int CH = BW / 8;
+        for (int task = tid; task < kTileRows * CH; task += kCoreWaves * kWave) {
+            const int rl = task / CH, ch = task - rl * CH;
+            const int row = rt * kTileRows + rl;
+            if (row >= M) continue;
+            const int c = h * BW + ch * 8;
+            float u[8], xg[8], ag[8], fy[8], so[8], hn[8], go[8];
+            unpack(*reinterpret_cast<const u32x4*>(sU + rl * kRowBytes + ch * 16), u);
+            unpack(*reinterpret_cast<const u32x4*>(sO + rl * kORowBytes + ch * 16), xg);
+            unpack(*reinterpret_cast<const u32x4*>(sO + rl * kORowBytes + BW * 2 + ch * 16), ag);
+            const bf16_t* yp = y + (size_t)row * ldy + c;
+            ST* sp = state + (size_t)row * D + c;
+            bf16_t* op = out + (size_t)row * D + c;
+            if (vec_io) {
+                unpack(load_raw<bf16_t, 8>(yp), fy);
+                unpack(load_raw<ST, 8>(sp), so);
+            } else {
 #pragma unroll
-    for (int s = 0; s < KS; ++s)
-        acc_i = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*reinterpret_cast<const bf16x8*>(asrc + 32 * s),
-                                                        *reinterpret_cast<const bf16x8*>(bsrc + 32 * s), acc_i, 0, 0, 0);
-    wave_lds_fence();   // the first gate's operands have been read: the region can be overwritten
-    stage_weights();
-    wave_lds_fence();
+                for (int v = 0; v < 8; ++v) {
+                    float t1[1], t2[1];
+                    unpack(load_raw<bf16_t, 1>(yp + v), t1);
+                    unpack(load_raw<ST, 1>(sp + v), t2);
+                    fy[v] = t1[0];
+                    so[v] = t2[0];
+                }
+            }
 #pragma unroll
-    for (int s = 0; s < KS; ++s)
-        acc_a = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*reinterpret_cast<const bf16x8*>(asrc + 32 * s),
-                                                        *reinterpret_cast<const bf16x8*>(bsrc + 32 * s), acc_a, 0, 0, 0);
-
-    // ---- 3. biases, recurrence, output gate
-    const float bias_i = b_i != nullptr ? b_i[c_out] : 0.0f;
-    const float bias_a = b_a != nullptr ? b_a[c_out] : 0.0f;
-    const float sp = softplus_precise(lam[c_out]);
+            for (int v = 0; v < 8; ++v) {
+                hn[v] = rglru_step_value(u[v], xg[v], ag[v], sSp[ch * 8 + v], so[v]);
+                go[v] = gelu_times(fy[v], hn[v]);
+            }
+            if (vec_io) {
+                sraw8_t rs;
+                u32x4 ro;
+                pack(hn, rs);
+                pack(go, ro);
+                *reinterpret_cast<sraw8_t*>(sp) = rs;
+                *reinterpret_cast<u32x4*>(op) = ro;
+            } else {
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-        const int rl = 4 * (lane >> 5) + 8 * (r / 4) + (r % 4);
-        const int row = rt * kTileRows + rl;
-        if (row >= M) continue;
-        const float u = __uint_as_float(
-            (uint32_t) * reinterpret_cast<const uint16_t*>(sU + rl * kRowBytes + (w * 32 + col) * 2) << 16);
-        const float xg = __uint_as_float((uint32_t)to_bf16_bits(acc_i[r] + bias_i) << 16);
-        const float ag = __uint_as_float((uint32_t)to_bf16_bits(acc_a[r] + bias_a) << 16);
-        float so[1], fy[1], hn[1];
-        unpack(sold[r], so);
-        unpack(ybits[r], fy);
-        hn[0] = rglru_step_value(u, xg, ag, sp, so[0]);
-        sraw_t rs;
-        pack(hn, rs);
-        *reinterpret_cast<sraw_t*>(state + (size_t)row * D + c_out) = rs;
-        *reinterpret_cast<uint16_t*>(out + (size_t)row * D + c_out) = to_bf16_bits(gelu_times(fy[0], hn[0]));
+                for (int v = 0; v < 8; ++v) {
+                    const float h1[1] = {hn[v]};
+                    typename Raw<ST, 1>::type r1;
+                    pack(h1, r1);
+                    *reinterpret_cast<typename Raw<ST, 1>::type*>(sp + v) = r1;
+                    *reinterpret_cast<uint16_t*>(op + v) = to_bf16_bits(go[v]);
+                }
+            }
+        }
     }
 }
 
@@ -1107,13 +1162,16 @@ int launch_decode_core(void* conv_state, const void* x_new, long long ldx, const
     const long long grid = (long long)nb * ntiles;
     if (grid > 0x7fffffffLL) return HAWK_ERR_BAD_SHAPE;
     constexpr auto kernel = decode_core_kernel<WT, ST, BW>;
-    constexpr size_t smem = CoreLds<BW>::kBytes;
+    constexpr size_t smem = CoreLds<BW>::kBytes + BW * sizeof(float);   // + softplus(Lambda) of the block
+    // 16-byte accesses to y, recc_state and out when their rows allow it
+    const bool vec_io = (ldy % 8) == 0 && (reinterpret_cast<uintptr_t>(y) & 15u) == 0 &&
+                        (reinterpret_cast<uintptr_t>(state) & 31u) == 0 && (reinterpret_cast<uintptr_t>(out) & 15u) == 0;
     if (!allow_dynamic_lds<kernel>(smem)) return HAWK_ERR_LAUNCH;
     hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(kCoreWaves * kWave), smem, st,
                        static_cast<bf16_t*>(conv_state), static_cast<const bf16_t*>(x_new), (size_t)ldx, conv_w,
                        conv_b, static_cast<const WT*>(w_i), b_i, static_cast<const WT*>(w_a), b_a, lam,
                        static_cast<const bf16_t*>(y), (size_t)ldy, static_cast<ST*>(state), static_cast<bf16_t*>(out),
-                       B, D, W, ntiles);
+                       B, D, W, ntiles, vec_io);
     return hipGetLastError() == hipSuccess ? HAWK_OK : HAWK_ERR_LAUNCH;
 }
 

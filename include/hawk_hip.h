@@ -219,7 +219,8 @@ int hawk_decode_core_supported(int D, int num_blocks, int W);
  *   out        [B, D] <- gelu(y) * h
  * conv_state, x_new, y and out are bf16 (`dtype` must be HAWK_DTYPE_BF16).  The conv output
  * and the two logits are rounded to bf16 where the three separate calls round them, so both
- * routes agree to the last bit or two of a bf16 result. */
+ * routes give the same result.  y, recc_state and out are accessed 16 bytes at a time when
+ * they are 16-byte aligned (32 for an fp32 recc_state) and ldy is a multiple of 8. */
 int hawk_decode_core_step(void* conv_state, const void* x_new, long long ldx, const float* conv_w,
                           const float* conv_b, const void* w_i, const float* b_i, const void* w_a,
                           const float* b_a, const float* a_param, const void* y, long long ldy,

@@ -175,3 +175,27 @@ def test_decode_core_step_against_the_oracle():
     assert np.array_equal(n(cs), cs_next.astype(np.float32))
     assert max_rel(n(st), h_ref) < TOL["bf16"]
     assert max_rel(n(out), out_ref) < TOL["bf16"]
+
+
+@pytest.mark.parametrize("state_dtype", ["bf16", "f32"])
+def test_decode_core_step_with_operands_that_forbid_16_byte_accesses(state_dtype):
+    """y with an odd row stride, recc_state and out 8 bytes off a 16-byte boundary: the step
+    falls back to element-wise accesses for them and gives the same result."""
+    B, D, nb, W = 45, 512, 4, 4
+    wide, cs, conv_w, conv_b, w_i, b_i, w_a, b_a, lam, st = _core_operands(B, D, nb, W, "bf16", state_dtype, 21)
+    x_new = wide[:, :D]
+    y_odd = torch.zeros(B, D + 1, dtype=torch.bfloat16, device="cuda")
+    y_odd[:, :D] = wide[:, D:]
+    y = y_odd[:, :D]
+    assert y.stride(0) % 2 == 1
+    off = 8 // st.element_size()
+    st_buf = torch.zeros(B * D + off, dtype=st.dtype, device="cuda")
+    st_off = st_buf[off:].view(B, D)
+    st_off.copy_(st)
+    assert st_off.data_ptr() % 16 == 8
+    cs_ref, st_ref = cs.clone(), st.clone()
+    out = capi.decode_core_step(cs, x_new, conv_w, conv_b, w_i, b_i, w_a, b_a, lam, y, st_off)
+    out_ref = capi.decode_core_step(cs_ref, x_new, conv_w, conv_b, w_i, b_i, w_a, b_a, lam, wide[:, D:], st_ref)
+    assert torch.equal(cs, cs_ref)
+    assert torch.equal(st_off, st_ref)
+    assert torch.equal(out, out_ref)
