@@ -305,3 +305,14 @@ def test_argument_validation_of_the_fused_decode_step():
     assert lib.hawk_decode_core_supported(2560, 10, 4) == 1
     assert lib.hawk_decode_core_supported(2560, 10, 9) == 0
     assert lib.hawk_decode_core_supported(2560, 7, 4) == 0
+
+
+def test_bench_refuses_more_than_one_gpu():
+    import subprocess
+    import sys
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"],
+                       capture_output=True, text=True, timeout=300, cwd=root)
+    assert r.returncode == 2
+    assert "one GPU" in r.stderr and r.stdout.strip() == ""
