@@ -431,18 +431,19 @@ def fused_linear_scan_gated(x, x_rg_lru, a_rg_lru, a_param, y, return_last_state
 class RecurrentCore(Function):
     @staticmethod
     def forward(ctx, u, w_i, b_i, w_a, b_a, a_param, y, want_last):
-        from .external import _gate_proj_fwd_op  # deferred: external imports nothing from here
+        from .external import _gate_proj_fwd_op, kernel_weights  # deferred: external imports nothing from here
 
         assert u.dtype == torch.bfloat16, "the fused core runs on bf16 activations"
         uc = u if u.is_contiguous() else u.contiguous()
         lam = a_param.float().contiguous()
+        ctx.dtypes = (w_i.dtype, b_i.dtype, w_a.dtype, b_a.dtype, a_param.dtype, y.dtype)
+        w_i, w_a = kernel_weights(w_i, w_a, uc.numel() // uc.shape[-1])
         xg, ag = _gate_proj_fwd_op(uc, w_i, b_i.float().reshape(-1), w_a, b_a.float().reshape(-1), True)
         _check_shapes(uc, xg, ag, a_param)
         want_h = any(ctx.needs_input_grad[:7])
         out, h, h_last = _rglru_scan_gated_fwd_op(uc, xg, ag, lam, y, True, want_h, bool(want_last))
         if want_h:
             ctx.save_for_backward(uc, xg, ag, h, y, w_i, w_a, a_param)
-        ctx.dtypes = (w_i.dtype, b_i.dtype, w_a.dtype, b_a.dtype, a_param.dtype, y.dtype)
         ctx.mark_non_differentiable(h_last)
         return out, h_last
 

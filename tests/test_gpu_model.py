@@ -593,3 +593,39 @@ def test_recurrent_core_matches_its_parts():
         assert a.shape == b.shape, name
         assert max_rel(capi.to_np(a), capi.to_np(b)) < 1e-2, (name, max_rel(capi.to_np(a), capi.to_np(b)))
     assert torch.equal(got[0], want[0])  # the forward is the very same pair of kernels
+
+
+def test_rounding_fp32_gate_weights_once_per_forward_changes_no_bit():
+    """From 8192 rows on the host hands the projection kernels bf16 copies of fp32 weights
+    instead of letting every workgroup round them: outputs and all gradients must be the same."""
+    import hawk_pytorch_amd.external as he
+
+    B, T, D, nb = 2, 4096, 512, 2
+    g = torch.Generator(device="cuda").manual_seed(31)
+    x = torch.randn(B, T, D, device="cuda", generator=g).to(torch.bfloat16).requires_grad_(True)
+    gi = he.BlockDiagonalLinear(D, nb, device="cuda")
+    ga = he.BlockDiagonalLinear(D, nb, device="cuda")
+    with torch.no_grad():
+        gi.b.normal_(generator=g)
+        ga.b.normal_(generator=g)
+    go_i = torch.randn(B, T, D, device="cuda", generator=g).to(torch.bfloat16)
+    go_a = torch.randn(B, T, D, device="cuda", generator=g).to(torch.bfloat16)
+
+    def run():
+        for t in (x, gi.w, gi.b, ga.w, ga.b):
+            t.grad = None
+        with torch.autocast(device_type="cuda", dtype=torch.bfloat16):
+            xg, ag = he.gate_projections(x, gi, ga, torch.bfloat16)
+        torch.autograd.backward([xg, ag], [go_i, go_a])
+        return [xg.detach(), ag.detach()] + [t.grad.clone() for t in (x, gi.w, gi.b, ga.w, ga.b)]
+
+    assert B * T >= he._CAST_WEIGHTS_MIN_ROWS
+    cast = run()
+    keep = he._CAST_WEIGHTS_MIN_ROWS
+    try:
+        he._CAST_WEIGHTS_MIN_ROWS = 1 << 40
+        plain = run()
+    finally:
+        he._CAST_WEIGHTS_MIN_ROWS = keep
+    for a, b in zip(cast, plain):
+        assert torch.equal(a, b)
