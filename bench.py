@@ -14,7 +14,8 @@ y being one half of a [B, T, 2D] projection), 12 + 20 bytes per element;
 forward, input gradient, weight gradients) on 32768 tokens, D = 2560, 10 blocks, bf16;
 ``--workload block`` chains the whole recurrent core of one layer at B=8, T=4096, D=2560 (conv,
 both gate projections, scan fused with the output gate, and the backward of all of them)
-through the C ABI, seven launches that move 31 activation-sized tensors;
+through the C ABI, seven launches that move 31 activation-sized tensors (plus two casts of the
+fp32 gate weights to bf16, as the Python host does at this size);
 ``--workload model`` runs full training steps (forward, backward, AdamW) of the upstream
 README model (vocabulary 32000, hidden = recurrent = 512, MLP 1024, 8 layers, 16 gate blocks)
 on a 1 x 2048 batch under bf16 autocast, with and without the fused gate / epilogue kernels;
