@@ -23,6 +23,7 @@ HAWK_ERR_BAD_DTYPE = 3
 HAWK_ERR_WORKSPACE = 4
 HAWK_ERR_LAUNCH = 5
 HAWK_ERR_ALIGNMENT = 6
+HAWK_ERR_SCRATCH_LIMIT = 7
 
 HAWK_DTYPE_BF16 = 0
 HAWK_DTYPE_F32 = 1
@@ -39,6 +40,7 @@ SIGNATURES = {
     "hawk_scan_workspace_init": (_c_int, [_c_void_p, _c_size_t, _c_void_p]),
     "hawk_scan_workspace_status": (_c_int, [_c_void_p, _c_void_p, ctypes.POINTER(_c_int)]),
     "hawk_rglru_scan_fwd": (_c_int, [_c_void_p] * 5 + [_c_int] * 4 + [_c_void_p, _c_size_t, _c_void_p]),
+    "hawk_rglru_scan_fwd_static": (_c_int, [_c_void_p] * 5 + [_c_int] * 4 + [_c_void_p]),
     "hawk_rglru_scan_bwd": (_c_int, [_c_void_p] * 10 + [_c_int] * 4 + [_c_void_p, _c_size_t, _c_void_p]),
     "hawk_rglru_scan_fwd_mixed": (_c_int, [_c_void_p] * 5 + [_c_int] * 5 + [_c_void_p, _c_size_t, _c_void_p]),
     "hawk_rglru_scan_bwd_mixed": (_c_int, [_c_void_p] * 10 + [_c_int] * 5 + [_c_void_p, _c_size_t, _c_void_p]),

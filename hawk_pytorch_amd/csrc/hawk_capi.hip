@@ -42,6 +42,9 @@ const char* hawk_status_string(int status) {
         case HAWK_ERR_WORKSPACE: return "workspace is NULL or smaller than the size query reports";
         case HAWK_ERR_LAUNCH: return "the HIP runtime refused a kernel launch or copy";
         case HAWK_ERR_ALIGNMENT: return "tensor pointers must be 16-byte aligned";
+        case HAWK_ERR_SCRATCH_LIMIT:
+            return "shape needs more carry words than the library's fixed 16 MiB scratch array holds: "
+                   "ceil(T/128) * B * D * 24 + 256 bytes must fit; use the entry point that takes a workspace";
         default: return "unknown status";
     }
 }
@@ -59,7 +62,8 @@ int hawk_scan_workspace_init(void* workspace_device, size_t workspace_bytes, voi
 }
 
 int hawk_scan_workspace_status(const void* workspace_device, void* stream, int* flag) {
-    if (workspace_device == nullptr || flag == nullptr) return HAWK_ERR_NULL_POINTER;
+    if (flag == nullptr) return HAWK_ERR_NULL_POINTER;
+    if (workspace_device == nullptr) return hawk::static_scratch_status(as_stream(stream), flag);
     return hawk::workspace_status(workspace_device, as_stream(stream), flag);
 }
 
@@ -81,6 +85,15 @@ int hawk_rglru_scan_fwd(const void* x, const void* x_rg_lru, const void* a_rg_lr
                         void* stream) {
     return hawk_rglru_scan_fwd_mixed(x, x_rg_lru, a_rg_lru, a_param, h, B, T, D, dtype, dtype, workspace_device,
                                      workspace_bytes, stream);
+}
+
+int hawk_rglru_scan_fwd_static(const void* x, const void* x_rg_lru, const void* a_rg_lru, const float* a_param,
+                               void* h, int B, int T, int D, int dtype, void* stream) {
+    if (!x || !x_rg_lru || !a_rg_lru || !a_param || !h) return HAWK_ERR_NULL_POINTER;
+    if (!dtype_ok(dtype)) return HAWK_ERR_BAD_DTYPE;
+    if (int rc = check_scan_shape(B, T, D)) return rc;
+    if (!aligned16(x) || !aligned16(x_rg_lru) || !aligned16(a_rg_lru) || !aligned16(h)) return HAWK_ERR_ALIGNMENT;
+    return hawk::scan_fwd_static(x, x_rg_lru, a_rg_lru, a_param, h, B, T, D, dtype, as_stream(stream));
 }
 
 int hawk_rglru_scan_bwd_mixed(const void* x, const void* x_rg_lru, const void* a_rg_lru, const float* a_param,

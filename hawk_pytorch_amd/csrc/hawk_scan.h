@@ -20,6 +20,10 @@ int scan_fwd(const void* x, const void* xg, const void* ag, const float* lam, vo
 int scan_bwd(const void* x, const void* xg, const void* ag, const float* lam, const void* hs, const void* gout,
              void* dx, void* dxg, void* dag, float* dlam, int B, int T, int D, int in_dtype, int state_dtype,
              void* ws, size_t ws_bytes, hipStream_t st);
+// Forward scan on the library's fixed per-device carry array; allocates nothing.
+int scan_fwd_static(const void* x, const void* xg, const void* ag, const float* lam, void* h, int B, int T, int D,
+                    int dtype, hipStream_t st);
+int static_scratch_status(hipStream_t st, int* flag);
 // Gated variants: out = gelu(y) * h.  y (and dy) are [B, T, D] with ldy (lddy) elements between rows.
 int scan_gated_fwd(const void* x, const void* xg, const void* ag, const float* lam, const void* y, long long ldy,
                    void* h, void* out, void* h_last, int B, int T, int D, int in_dtype, int out_dtype, void* ws,

@@ -34,6 +34,8 @@
 
 #include <stdint.h>
 
+#include <mutex>
+
 #include "hawk_device.h"
 
 namespace hawk {
@@ -1013,6 +1015,73 @@ int workspace_status(const void* ws, hipStream_t st, int* flag) {
     if (hipStreamSynchronize(st) != hipSuccess) return HAWK_ERR_LAUNCH;
     *flag = (int)v;
     return HAWK_OK;
+}
+
+// ---------------------------------------------------------------------------------------
+// Forward scan on the library's own carry buffer, for callers that cannot allocate.
+// `scratch` is one fixed array per GPU (each device that loads this code object holds its
+// own copy at its own address, from the first use of the library on that device until the
+// process ends).  On the host the array's name is only a handle: the device address is
+// asked for once per device, with that device current, and kept; kernels, fills and copies
+// only ever see that address.
+// ---------------------------------------------------------------------------------------
+namespace {
+
+static __device__ __align__(256) unsigned char scratch[HAWK_STATIC_SCRATCH_BYTES];
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[kMaxDevices] = {};
+
+// Device address of the current device's scratch array; *fresh is set when this call is the
+// one that looked it up.
+int static_scratch_ptr(void** out, bool* fresh) {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return HAWK_ERR_LAUNCH;
+    std::lock_guard<std::mutex> guard(g_scratch_mutex);
+    *fresh = false;
+    if (g_scratch_ptr[dev] == nullptr) {
+        void* p = nullptr;
+        if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || p == nullptr) return HAWK_ERR_LAUNCH;
+        g_scratch_ptr[dev] = p;
+        *fresh = true;
+    }
+    *out = g_scratch_ptr[dev];
+    return HAWK_OK;
+}
+
+}  // namespace
+
+int scan_fwd_static(const void* x, const void* xg, const void* ag, const float* lam, void* h, int B, int T, int D,
+                    int dtype, hipStream_t st) {
+    const TileShape s = fwd_shape(D, dtype);
+    const int nseg = ceil_div(T, s.rows());
+    if (nseg > 1 && layout_for(B, D, nseg, 0).total > (size_t)HAWK_STATIC_SCRATCH_BYTES) return HAWK_ERR_SCRATCH_LIMIT;
+    void* ws = nullptr;
+    bool fresh = false;
+    if (int rc = static_scratch_ptr(&ws, &fresh)) return rc;
+    if (fresh) {
+        // The array starts as zeros like any object of static storage; the first use on a
+        // device clears it all the same (with a fill kernel, ordered before the scan on the
+        // caller's stream) unless that stream is being captured: a fill recorded into a graph
+        // would rewind the launch epoch at every replay.  Afterwards nothing needs clearing:
+        // the ticket half of the control word is back at zero when a launch ends, and words
+        // of earlier calls carry older launch tags.
+        hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(st, &cap) != hipSuccess) return HAWK_ERR_LAUNCH;
+        if (cap == hipStreamCaptureStatusNone) {
+            if (int rc = workspace_init(ws, HAWK_STATIC_SCRATCH_BYTES, st)) return rc;
+        }
+    }
+    return scan_fwd_impl<false>(x, xg, ag, lam, h, GateFwdHost{}, B, T, D, dtype, dtype, ws,
+                                (size_t)HAWK_STATIC_SCRATCH_BYTES, st);
+}
+
+int static_scratch_status(hipStream_t st, int* flag) {
+    void* ws = nullptr;
+    bool fresh = false;
+    if (int rc = static_scratch_ptr(&ws, &fresh)) return rc;
+    return workspace_status(ws, st, flag);
 }
 
 bool scan_dtypes_supported(int in_dtype, int state_dtype) {

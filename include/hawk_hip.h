@@ -31,7 +31,9 @@ typedef enum hawk_status {
     HAWK_ERR_BAD_DTYPE = 3,     /* dtype is not a hawk_dtype this entry point supports */
     HAWK_ERR_WORKSPACE = 4,     /* workspace missing or smaller than the size query says */
     HAWK_ERR_LAUNCH = 5,        /* the HIP runtime refused a launch or copy */
-    HAWK_ERR_ALIGNMENT = 6      /* a tensor pointer is not aligned to its element size */
+    HAWK_ERR_ALIGNMENT = 6,     /* a tensor pointer is not aligned to its element size */
+    HAWK_ERR_SCRATCH_LIMIT = 7  /* the problem needs more carry words than the library's fixed
+                                   scratch array holds (hawk_rglru_scan_fwd_static only) */
 } hawk_status;
 
 typedef enum hawk_dtype {
@@ -56,7 +58,8 @@ size_t hawk_scan_workspace_bytes(int B, int T, int D, int dtype);
 int hawk_scan_workspace_init(void* workspace_device, size_t workspace_bytes, void* stream);
 /* Synchronises `stream` and reports in *flag whether any scan on this workspace gave up
  * waiting for a carry (0 = all carries arrived).  A non-zero flag means results of that
- * launch are invalid and the workspace must be re-initialised. */
+ * launch are invalid and the workspace must be re-initialised.  workspace_device == NULL
+ * asks about the current device's fixed scratch array (hawk_rglru_scan_fwd_static). */
 int hawk_scan_workspace_status(const void* workspace_device, void* stream, int* flag);
 
 /* ---------------------------------------------------------------------------------------
@@ -76,6 +79,26 @@ int hawk_scan_workspace_status(const void* workspace_device, void* stream, int* 
 int hawk_rglru_scan_fwd(const void* x, const void* x_rg_lru, const void* a_rg_lru,
                         const float* a_param, void* h, int B, int T, int D, int dtype,
                         void* workspace_device, size_t workspace_bytes, void* stream);
+
+/* hawk_rglru_scan_fwd for callers that cannot allocate device memory (code under HIP graph
+ * capture, serving loops, harnesses that forbid allocation).  It has no counterpart
+ * upstream.  Same kernels, same arguments and same results bit for bit, but the carry words
+ * live in an array of HAWK_STATIC_SCRATCH_BYTES that is part of the library's device code:
+ * every GPU the library is used on holds one such array from the first call there until the
+ * process ends.  The call allocates and frees nothing.
+ *   limit   ceil(T / 128) * B * D * 24 bytes + 256 must not exceed HAWK_STATIC_SCRATCH_BYTES
+ *           (T <= 128 always fits); beyond it the call returns HAWK_ERR_SCRATCH_LIMIT and
+ *           launches nothing.  B=8, T=4096, D=2560 needs 15.0 MiB.
+ *   sharing every call on a GPU uses that GPU's one array, so calls must not overlap there:
+ *           order them on one stream (or with events).  Two overlapping calls race.
+ *   set-up  the first call on a device looks up the array's device address (the device must
+ *           be current, as for every call) and clears the array with a fill kernel ahead of
+ *           the scan on `stream`; when that first call is being captured into a graph the
+ *           fill is left out and the array's zero initialisation is relied on. */
+#define HAWK_STATIC_SCRATCH_BYTES (16u << 20)
+int hawk_rglru_scan_fwd_static(const void* x, const void* x_rg_lru, const void* a_rg_lru,
+                               const float* a_param, void* h, int B, int T, int D, int dtype,
+                               void* stream);
 
 /* RG-LRU scan backward (reverse time).  Inputs are the forward's inputs, the saved h and
  * the upstream gradient; outputs are dx, dx_rg_lru, da_rg_lru in `dtype` and
