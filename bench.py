@@ -27,6 +27,10 @@ The kernel workloads (scan*, long, gates, block) run ``--settle-steps`` untimed 
 before the ``--warmup`` ones: for about 50 steps (20 ms) after the GPU leaves idle the same kernels
 run up to 12 % slower than they do from then on.
 
+The default workload's line also carries, under "also", records for the long-context and the
+scan + conv configurations, timed after the headline region in the same process (``--no-also``
+leaves them out).
+
 Prints one JSON line:
   value        tokens/s = B*T / (wall time per step), whole job on one GPU
   roofline     for the dominant kernel (the backward scan): algorithmic bytes per launch
@@ -55,21 +59,62 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0
 
-# HBM bytes per launch of the backward scan kernel, from rocprofv3 --pmc FETCH_SIZE and
-# WRITE_SIZE runs of this file, each scaled by what the same counter reads for a plain
-# device copy of known size in the same run (FETCH x 2.000, WRITE x 1.000 on this part).
-# Sources: profiles/rglru_scan_B8_T4096_D2560_bf16.md, profiles/rglru_scan_B2_T32768_D4096_bf16.md,
-# profiles/rglru_scan_gated_B8_T4096_D2560_bf16.md.
-MEASURED_BWD_TRAFFIC_BYTES = {
-    "scan": 876.9e6 + 545.0e6,
-    "scan_conv": 876.9e6 + 545.0e6,
-    "long": 2776.5e6 + 1711.7e6,
-    "scan_gated": 1050.4e6 + 712.7e6,
-}
+# HBM bytes per launch of each workload's dominant kernel, as rocprofv3 counted them
+# (--pmc FETCH_SIZE, then WRITE_SIZE, each scaled by what the same counter reads for a plain
+# device copy of known size in the same run), are kept in profiles/hbm_traffic.json together
+# with the digest of the kernel sources they were measured on.  A record taken on other
+# sources is stale and is not reported.
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+KERNEL_SOURCES = ("hawk_scan.hip", "hawk_gates.hip", "hawk_conv.hip", "hawk_device.h")
 
-# The same for the gates workload's dominant launch (weight-gradient kernel + its reduce kernel):
-# 503.4 + 63.2 MB read, 63.2 + 5.3 MB written (profiles/gate_proj_M32768_D2560_nb10_bf16.md).
-MEASURED_GATE_DW_TRAFFIC_BYTES = 503.4e6 + 63.2e6 + 63.2e6 + 5.3e6
+
+def kernel_source_digest():
+    import hashlib
+
+    h = hashlib.sha256()
+    for name in KERNEL_SOURCES:
+        with open(os.path.join(ROOT, "hawk_pytorch_amd", "csrc", name), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
+
+
+def measured_traffic(workload):
+    """FETCH + WRITE bytes per launch recorded for `workload`, or None (no record, or a record
+    taken on kernel sources other than the present ones)."""
+    try:
+        with open(TRAFFIC_FILE) as f:
+            rec = json.load(f).get(workload)
+    except (OSError, ValueError):
+        return None
+    if not rec or rec.get("kernel_source_digest") != kernel_source_digest():
+        return None
+    return float(rec["fetch_bytes"]) + float(rec["write_bytes"])
+
+
+def record_traffic(workload, fetch_bytes, write_bytes, note):
+    """Write one record of profiles/hbm_traffic.json (used after a rocprofv3 --pmc pass)."""
+    import datetime
+    import subprocess
+
+    try:
+        with open(TRAFFIC_FILE) as f:
+            data = json.load(f)
+    except (OSError, ValueError):
+        data = {}
+    try:
+        commit = subprocess.run(["git", "-C", ROOT, "rev-parse", "--short", "HEAD"], capture_output=True,
+                                text=True).stdout.strip() or None
+    except OSError:
+        commit = None
+    data[workload] = {
+        "fetch_bytes": float(fetch_bytes), "write_bytes": float(write_bytes),
+        "kernel_source_digest": kernel_source_digest(), "commit_before": commit,
+        "date": datetime.date.today().isoformat(), "note": note,
+    }
+    with open(TRAFFIC_FILE, "w") as f:
+        json.dump(data, f, indent=1, sort_keys=True)
+        f.write("\n")
+
 
 WORKLOADS = {
     # name: (B, T, D, a^8 range, includes conv)
@@ -89,9 +134,17 @@ def lambda_for_a8_range(gen, D, lo, hi):
 
 
 def cpu_baseline(B, D, lo, hi, seed, budget_elements=1024 * 8 * 2560):
-    """PyTorch CPU loop (oracle/rglru_torch.py) on the first time rows of the workload's shape,
-    about `budget_elements` element-steps (10-20 s on 16 host threads): forward plus autograd
-    backward in fp32."""
+    """The recurrence on this host's cores, on the first time rows of the workload's shape
+    (about `budget_elements` element-steps), forward plus backward in fp32, two ways:
+
+    * `value`: the PyTorch loop over time (oracle/rglru_torch.py: the one-token step of
+      hawk/hawk.py:137-151, :196 iterated, autograd for the backward), 10-20 s on 16 host
+      threads.  Its rate falls with the sample's length, because the autograd tape grows.
+    * `scalar_c`: the single-threaded C restatement of the two kernels' arithmetic
+      (oracle_rglru_scan_{fwd,bwd}_f32, following hawk/scan_fused.py:44-109 and :123-317), whose
+      rate does not depend on the length of the sample.
+    """
+    import oracle
     from oracle import rglru_torch
 
     gen = torch.Generator().manual_seed(seed)
@@ -102,6 +155,13 @@ def cpu_baseline(B, D, lo, hi, seed, budget_elements=1024 * 8 * 2560):
     t0 = time.perf_counter()
     rglru_torch.rglru_scan_fwd_bwd(x, xg, ag, lam, go)
     dt = time.perf_counter() - t0
+
+    xn, xgn, agn, gon, lamn = (t.numpy() for t in (x, xg, ag, go, lam))
+    oracle.rglru_scan_fwd(xn[:, :8], xgn[:, :8], agn[:, :8], lamn, precision="f32")  # loads the library
+    t0 = time.perf_counter()
+    hn = oracle.rglru_scan_fwd(xn, xgn, agn, lamn, precision="f32")
+    oracle.rglru_scan_bwd(xn, xgn, agn, lamn, hn, gon, precision="f32")
+    dt_c = time.perf_counter() - t0
     return {
         "value": B * T / dt,
         "unit": "tokens/s",
@@ -109,6 +169,10 @@ def cpu_baseline(B, D, lo, hi, seed, budget_elements=1024 * 8 * 2560):
         "kind": "port",
         "sample": f"first {T} of the time rows at B={B}, D={D}, fp32, forward + autograd backward, "
                   f"{dt:.2f} s, host has {os.cpu_count()} logical cpus",
+        "scalar_c": {
+            "value": B * T / dt_c, "unit": "tokens/s", "cores": 1, "kind": "port",
+            "sample": f"the same {T} rows through the scalar C port of both kernels, fp32, {dt_c:.2f} s",
+        },
     }
 
 
@@ -186,7 +250,7 @@ def run_gates(args, lib, dev):
             "bound": "hbm",
             "kernel": "gate_proj_bwd_weights_kernel (+ gate_proj_reduce_kernel, same launch call)",
             "achieved": gbs[2], "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs[2] / HBM_PEAK_GBS,
-            "traffic": MEASURED_GATE_DW_TRAFFIC_BYTES,
+            "traffic": measured_traffic("gates"),
             "algorithmic_bytes_per_launch": alg[2], "launch_ms": ms[2],
         },
         "kernels": {name: {"ms": ms[i], "GBs": gbs[i], "frac": gbs[i] / HBM_PEAK_GBS,
@@ -509,54 +573,16 @@ def run_decode(args, lib, dev):
     print(json.dumps(out_json))
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=10, help="untimed steps before the timed ones")
-    ap.add_argument("--settle-steps", type=int, default=100,
-                    help="further untimed steps run before the warm-up in the kernel workloads (scan*, long, gates, "
-                         "block): kernel durations settle about 50 steps (20 ms) after the GPU leaves idle")
-    ap.add_argument("--workload", choices=sorted(WORKLOADS) + ["block", "decode", "gates", "model"], default="scan")
-    ap.add_argument("--seed", type=int, default=0)
-    ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--calibration-copy", action="store_true",
-                    help="also run three plain device-to-device copies of one activation tensor (outside the "
-                         "timed region) so that a rocprofv3 --pmc run has a kernel of known traffic to scale "
-                         "FETCH_SIZE / WRITE_SIZE by")
-    args = ap.parse_args()
-
-    if args.gpus != 1:
-        print("bench.py: this build runs on exactly one GPU (the path needs no collective); "
-              "--gpus must be 1", file=sys.stderr)
-        sys.exit(2)
-    if not torch.cuda.is_available():
-        print("bench.py: no GPU visible; the HIP kernels have no CPU fallback", file=sys.stderr)
-        sys.exit(1)
-
+def run_scan(args, lib, dev, name, steps, warmup, settle, calibration_copy=False):
+    """Times `steps` forward + backward steps of scan workload `name`; returns the record."""
     from hawk_pytorch_amd import _lib
 
-    lib = _lib.load()
-    dev = torch.device("cuda:0")
-    torch.cuda.set_device(dev)
-    if args.workload == "decode":
-        run_decode(args, lib, dev)
-        return
-    if args.workload == "gates":
-        run_gates(args, lib, dev)
-        return
-    if args.workload == "model":
-        run_model(args, lib, dev)
-        return
-    if args.workload == "block":
-        run_block(args, lib, dev)
-        return
-    B, T, D, (lo, hi), with_conv = WORKLOADS[args.workload]
+    B, T, D, (lo, hi), with_conv = WORKLOADS[name]
     N = B * T * D
     code = _lib.HAWK_DTYPE_BF16
     bf = torch.bfloat16
 
-    mixed = args.workload == "scan_mixed"
+    mixed = name == "scan_mixed"
     in_dt = torch.float32 if mixed else bf
     in_code = _lib.HAWK_DTYPE_F32 if mixed else code
     gen = torch.Generator(device=dev).manual_seed(args.seed)
@@ -576,7 +602,7 @@ def main():
         dw = torch.empty(W, D, device=dev)
         db = torch.empty(D, device=dev)
         cws = torch.empty(lib.hawk_conv1d_bwd_workspace_bytes(B, T, D, W), dtype=torch.uint8, device=dev)
-    gated = args.workload == "scan_gated"
+    gated = name == "scan_gated"
     if gated:
         xy = torch.randn(B, T, 2 * D, device=dev, generator=gen).to(bf)
         y = xy[..., D:]               # the gate half of the block's input projection, in place
@@ -629,12 +655,12 @@ def main():
                                                    dw.data_ptr(), db.data_ptr(), B, T, D, W, code, code,
                                                    cws.data_ptr(), cws.numel(), stream))
 
-    if args.calibration_copy:
+    if calibration_copy:
         for _ in range(3):
             h.copy_(x)  # reads 2*N bytes, writes 2*N bytes
         torch.cuda.synchronize()
 
-    for _ in range(args.settle_steps + args.warmup):
+    for _ in range(settle + warmup):
         fwd()
         bwd()
         if with_conv:
@@ -644,11 +670,11 @@ def main():
     # Two events per step bracket the backward launch; the forward launch of step k runs from the
     # end of step k-1 (its last event, or the event after the conv backward) to the first event of
     # step k.
-    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3 if with_conv else 2)] for _ in range(args.steps)]
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3 if with_conv else 2)] for _ in range(steps)]
     start = torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
     start.record()
-    for k in range(args.steps):
+    for k in range(steps):
         fwd()
         ev[k][0].record()
         bwd()
@@ -666,9 +692,9 @@ def main():
         sys.exit(1)
 
     step_end = [start] + [e[-1] for e in ev]
-    fwd_ms = float(np.mean([step_end[k].elapsed_time(ev[k][0]) for k in range(args.steps)]))
+    fwd_ms = float(np.mean([step_end[k].elapsed_time(ev[k][0]) for k in range(steps)]))
     bwd_ms = float(np.mean([e[0].elapsed_time(e[1]) for e in ev]))
-    ms_per_step = wall * 1e3 / args.steps
+    ms_per_step = wall * 1e3 / steps
     elem = 2  # bytes per bf16 activation element
     # gated: the forward also reads y and writes out; the backward also reads y and writes dy
     fwd_bytes = (6 if gated else 4) * elem * N + (2 * elem * N if with_conv else 0)
@@ -683,9 +709,9 @@ def main():
         "value": B * T / (ms_per_step * 1e-3),
         "unit": "tokens/s",
         "n_gpus": 1,
-        "steps": args.steps,
-        "warmup": args.warmup,
-        "settle_steps": args.settle_steps,
+        "steps": steps,
+        "warmup": warmup,
+        "settle_steps": settle,
         "ms_per_step": ms_per_step,
         "higher_is_better": True,
         "scaling": "weak",
@@ -694,7 +720,7 @@ def main():
                   else "bf16 in/out, f32 state and accumulation"),
         "data": f"synthetic, seed {args.seed}: x, gate logits, grad ~ N(0,1); a^8 ~ U({lo},{hi})",
         "config": {
-            "workload": f"{args.workload}: RG-LRU scan"
+            "workload": f"{name}: RG-LRU scan"
                         + (" + temporal conv1d (W=4)" if with_conv else "")
                         + (" fused with out = gelu(y) * h" if gated else "")
                         + f" fwd+bwd, B={B}, T={T}, D={D}, " + ("f32 in / bf16 state" if mixed else "bf16"),
@@ -708,7 +734,7 @@ def main():
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": bwd_gbs / HBM_PEAK_GBS,
-            "traffic": MEASURED_BWD_TRAFFIC_BYTES.get(args.workload),
+            "traffic": measured_traffic(name),
             "algorithmic_bytes_per_launch": bwd_bytes,
             "launch_ms": bwd_ms,
         },
@@ -717,8 +743,76 @@ def main():
         "step_hbm": {"GBs": step_bytes / (ms_per_step * 1e-3) / 1e9,
                      "frac": step_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS},
     }
+    out["_cpu_args"] = (B, D, lo, hi)
+    return out
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=10, help="untimed steps before the timed ones")
+    ap.add_argument("--settle-steps", type=int, default=100,
+                    help="further untimed steps run before the warm-up in the kernel workloads (scan*, long, gates, "
+                         "block): kernel durations settle about 50 steps (20 ms) after the GPU leaves idle")
+    ap.add_argument("--workload", choices=sorted(WORKLOADS) + ["block", "decode", "gates", "model"], default="scan")
+    ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-also", action="store_true",
+                    help="default workload only: skip the sub-records for the long and scan_conv configurations")
+    ap.add_argument("--record-traffic", nargs=3, metavar=("FETCH_BYTES", "WRITE_BYTES", "NOTE"),
+                    help="no GPU run: store a measured HBM traffic figure for --workload in "
+                         "profiles/hbm_traffic.json, stamped with the digest of the present kernel sources")
+    ap.add_argument("--calibration-copy", action="store_true",
+                    help="also run three plain device-to-device copies of one activation tensor (outside the "
+                         "timed region) so that a rocprofv3 --pmc run has a kernel of known traffic to scale "
+                         "FETCH_SIZE / WRITE_SIZE by")
+    args = ap.parse_args()
+
+    if args.record_traffic:
+        record_traffic(args.workload, float(args.record_traffic[0]), float(args.record_traffic[1]),
+                       args.record_traffic[2])
+        return
+    if args.gpus != 1:
+        print("bench.py: this build runs on exactly one GPU (the path needs no collective); "
+              "--gpus must be 1", file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the HIP kernels have no CPU fallback", file=sys.stderr)
+        sys.exit(1)
+
+    from hawk_pytorch_amd import _lib
+
+    lib = _lib.load()
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    if args.workload == "decode":
+        run_decode(args, lib, dev)
+        return
+    if args.workload == "gates":
+        run_gates(args, lib, dev)
+        return
+    if args.workload == "model":
+        run_model(args, lib, dev)
+        return
+    if args.workload == "block":
+        run_block(args, lib, dev)
+        return
+    out = run_scan(args, lib, dev, args.workload, args.steps, args.warmup, args.settle_steps, args.calibration_copy)
+    cpu_args = out.pop("_cpu_args")
+    if args.workload == "scan" and not args.no_also:
+        # the other scan configurations of the benchmark definition, timed after the headline
+        # region in the same process (fewer steps; the GPU is already at its steady clocks)
+        also = {}
+        for other in ("long", "scan_conv"):
+            torch.cuda.empty_cache()
+            rec = run_scan(args, lib, dev, other, max(20, args.steps // 4), args.warmup, max(10, args.settle_steps // 4))
+            rec.pop("_cpu_args")
+            also[other] = {k: rec[k] for k in ("config", "value", "unit", "ms_per_step", "steps", "warmup",
+                                               "settle_steps", "roofline", "fwd", "step_hbm")}
+        out["also"] = also
     if not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline(B, D, lo, hi, args.seed)
+        out["cpu_baseline"] = cpu_baseline(*cpu_args, args.seed)
     print(json.dumps(out))
 
 

@@ -2,6 +2,7 @@
 operator / module surface of fattorib/hawk-pytorch (``from hawk import HawkModel, HawkConfig``
 becomes ``from hawk_pytorch_amd import HawkModel, HawkConfig``)."""
 
+from ._lib import HawkHipError, check_scan_status, release_workspaces
 from .cache import RNNCache
 from .external import (
     BlockDiagonalLinear,
@@ -32,15 +33,18 @@ __all__ = [
     "GatedDiagonalRecurrence",
     "Hawk",
     "HawkConfig",
+    "HawkHipError",
     "HawkModel",
     "MLP",
     "RMSNorm",
     "RNNCache",
     "RNNLayer",
+    "check_scan_status",
     "decode_core_step",
     "fused_linear_scan",
     "gate_projections",
     "recurrent_core",
+    "release_workspaces",
     "fused_linear_scan_gated",
     "rglru_step",
     "rglru_step_gated",

@@ -159,6 +159,15 @@ def dense16(t: torch.Tensor) -> torch.Tensor:
 # Scans that share a workspace must be ordered on one stream, hence the key.
 # ---------------------------------------------------------------------------------------
 _workspaces: dict = {}
+# Workspaces handed to launches recorded into HIP graphs: (device index, tensor).  They belong to
+# the graph's memory pool; a reference is kept so that their carry-timeout flag can be read
+# after a replay.  At most _MAX_CAPTURED are remembered (oldest dropped first).
+_captured: list = []
+_MAX_CAPTURED = 256
+
+
+def _device_index(dev: torch.device) -> int:
+    return dev.index if dev.index is not None else torch.cuda.current_device()
 
 
 def scan_workspace(dev: torch.device, nbytes: int) -> torch.Tensor:
@@ -168,22 +177,58 @@ def scan_workspace(dev: torch.device, nbytes: int) -> torch.Tensor:
         # code or another graph also uses, whatever stream it is replayed on and in whatever
         # order graphs are replayed.  (A cached buffer created during a capture would hold
         # nothing until that one graph had been replayed.)
-        return torch.zeros(max(nbytes, 256), dtype=torch.uint8, device=dev)
-    key = (dev.index if dev.index is not None else torch.cuda.current_device(), stream_ptr(dev))
-    ws = _workspaces.get(key)
-    if ws is None or ws.numel() < nbytes:
-        ws = torch.zeros(max(nbytes, 1 << 20), dtype=torch.uint8, device=dev)
-        _workspaces[key] = ws
+        ws = torch.zeros(max(nbytes, 256), dtype=torch.uint8, device=dev)
+        with _lock:
+            _captured.append((_device_index(dev), ws))
+            del _captured[:-_MAX_CAPTURED]
+        return ws
+    key = (_device_index(dev), stream_ptr(dev))
+    with _lock:
+        ws = _workspaces.get(key)
+        if ws is None or ws.numel() < nbytes:
+            ws = torch.zeros(max(nbytes, 1 << 20), dtype=torch.uint8, device=dev)
+            _workspaces[key] = ws
     return ws
+
+
+def release_workspaces() -> None:
+    """Drop every cached scan workspace (they are re-created on demand)."""
+    with _lock:
+        _workspaces.clear()
+        _captured.clear()
+
+
+def _flag_of(ws: torch.Tensor, dev: torch.device) -> int:
+    flag = ctypes.c_int(0)
+    with torch.cuda.device(dev):
+        check("hawk_scan_workspace_status",
+              load().hawk_scan_workspace_status(ws.data_ptr(), stream_ptr(dev), ctypes.byref(flag)))
+    return flag.value
 
 
 def scan_workspace_status(dev: torch.device) -> int:
     """Synchronising check of the carry-timeout flag of the current stream's workspace."""
-    key = (dev.index if dev.index is not None else torch.cuda.current_device(), stream_ptr(dev))
-    ws = _workspaces.get(key)
-    if ws is None:
-        return 0
-    flag = ctypes.c_int(0)
-    check("hawk_scan_workspace_status",
-          load().hawk_scan_workspace_status(ws.data_ptr(), stream_ptr(dev), ctypes.byref(flag)))
-    return flag.value
+    with _lock:
+        ws = _workspaces.get((_device_index(dev), stream_ptr(dev)))
+    return 0 if ws is None else _flag_of(ws, dev)
+
+
+def check_scan_status(device=None) -> None:
+    """Raise HawkHipError if any scan launched through this package on `device` (default: the
+    current one) gave up waiting for a carry, in which case that launch's results are wrong.
+
+    The kernels bound their wait so that a lost carry cannot hang the GPU; this is the call that
+    turns such an event into an error.  It synchronises the device, so call it where the program
+    synchronises anyway (end of a training step, after a graph replay, before results are used).
+    Covers the cached workspaces of every stream and those of launches captured into HIP graphs.
+    """
+    dev = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
+    idx = _device_index(dev)
+    with _lock:
+        todo = [ws for (d, _s), ws in _workspaces.items() if d == idx] + [ws for d, ws in _captured if d == idx]
+    torch.cuda.synchronize(dev)
+    for ws in todo:
+        if _flag_of(ws, dev) != 0:
+            raise HawkHipError("hawk_scan_workspace_status", HAWK_ERR_WORKSPACE,
+                               "a scan tile gave up waiting for its carry: the results of that launch are "
+                               "invalid; call release_workspaces() before the next scan")

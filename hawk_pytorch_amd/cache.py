@@ -7,8 +7,11 @@ are generalised: any batch size B (upstream asserts B == 1) and any temporal con
 (upstream ignores its ``temporal_conv_width`` argument and always uses 4).  With B == 1
 and width 4 the buffers are exactly upstream's.
 
-The decode kernels read and write ``recc_state`` / ``conv_state`` in place, so both are
-kept contiguous and are never re-bound to views of other tensors.
+The decode kernels read and write ``recc_state`` / ``conv_state`` in place and need them
+contiguous.  This package never re-binds them, but upstream's own ``Hawk.forward`` does
+(``layer_past.conv_state = x[:, -3:, ...]``, hawk/hawk.py:174, a strided view of the input
+projection), and its torch-only decode branch works on such a view; ``own_buffers`` turns a
+re-bound view back into a contiguous buffer of the cache's own before a kernel touches it.
 """
 
 from __future__ import annotations
@@ -59,6 +62,14 @@ class RNNCache:
         if self.conv_cache_size > 1:
             self.conv_state[:, :-1, :] = self.conv_state[:, 1:, :].clone()
         self.conv_state[:, -1:, :] = new_state
+
+    def own_buffers(self) -> None:
+        """Make ``recc_state`` and ``conv_state`` contiguous tensors that the cache alone
+        refers to (a copy is made only for a buffer that was re-bound to a strided view)."""
+        if not self.conv_state.is_contiguous():
+            self.conv_state = self.conv_state.contiguous()
+        if not self.recc_state.is_contiguous():
+            self.recc_state = self.recc_state.contiguous()
 
     def seed_conv_state(self, x: torch.Tensor) -> None:
         """Prefill: keep the last W-1 pre-conv rows of x [B,T,D]; a shorter prompt is

@@ -21,6 +21,8 @@ constexpr long long kMaxRowStride = 1LL << 24;  // elements; keeps 16 rows of an
 
 int check_scan_shape(int B, int T, int D) {
     if (B < 1 || T < 1 || D < 1) return HAWK_ERR_BAD_SHAPE;
+    // the kernels form row and tile byte offsets in 32 bits
+    if (D > kMaxRowStride) return HAWK_ERR_BAD_SHAPE;
     // tiles are at least 64 rows x 64 channels; the flattened grid must fit 31 bits
     const long long tiles = (long long)B * ((T + 63) / 64) * ((D + 63) / 64);
     if (tiles > kMaxTiles) return HAWK_ERR_BAD_SHAPE;

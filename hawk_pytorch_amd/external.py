@@ -383,10 +383,11 @@ def _gate_workspace(dev: torch.device, nbytes: int) -> torch.Tensor:
     if torch.cuda.is_current_stream_capturing():
         return torch.empty(nbytes, dtype=torch.uint8, device=dev)  # the graph's own scratch, from its pool
     key = (dev.index if dev.index is not None else torch.cuda.current_device(), _lib.stream_ptr(dev))
-    ws = _gate_ws.get(key)
-    if ws is None or ws.numel() < nbytes:
-        ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
-        _gate_ws[key] = ws
+    with _lib._lock:
+        ws = _gate_ws.get(key)
+        if ws is None or ws.numel() < nbytes:
+            ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+            _gate_ws[key] = ws
     return ws
 
 

@@ -135,8 +135,15 @@ class Hawk(nn.Module):
         branch, gate_branch = self.input_xy(x).chunk(2, dim=-1)
 
         if warm:
-            # one new token per batch row; only the last position is used, as upstream
+            # One new token per batch row.  (Upstream accepts more and silently keeps only the
+            # last position, hawk/hawk.py:178-179, with a conv window that then spans the new
+            # rows; nothing sensible can be returned for the other positions, so refuse.)
             assert layer_past is not None
+            assert x.shape[1] == 1, (
+                f"a warm cache takes one new token per call, got {x.shape[1]}; "
+                "feed longer inputs with a fresh RNNCache (prefill)"
+            )
+            layer_past.own_buffers()
             fused_gates = self.config.fused_gates and gate_projections_supported(branch, self.rg_lru_input_gate)
             gate_branch = gate_branch[:, -1:, :]
             layer_past.current_cache_size = 1

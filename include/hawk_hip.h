@@ -4,8 +4,10 @@
  * Plain pointers and sizes only.  Every pointer named "device" must be device memory of
  * the GPU that is current when the call is made.  All calls are asynchronous on `stream`
  * (a hipStream_t passed as void*; NULL is the default stream) unless stated otherwise,
- * never synchronise the device, never allocate or free memory, keep no host-side state,
- * and may be called from any host thread.  Every function returns a hawk_status; nothing
+ * never synchronise the device, never allocate or free memory, and may be called from any
+ * host thread.  The only host-side state is bookkeeping that no caller can observe: a bit per
+ * device recording that a kernel's dynamic-LDS limit has been raised there, and the device
+ * address of the fixed scratch array of hawk_rglru_scan_fwd_static.  Every function returns a hawk_status; nothing
  * throws or aborts.
  *
  * Tensors are dense row-major: activations [B,T,D] (strides T*D, D, 1), Lambda [D] fp32,
@@ -27,7 +29,8 @@ extern "C" {
 typedef enum hawk_status {
     HAWK_OK = 0,
     HAWK_ERR_NULL_POINTER = 1,  /* a required pointer is NULL */
-    HAWK_ERR_BAD_SHAPE = 2,     /* a size is < 1, too large, or breaks a stated divisibility rule */
+    HAWK_ERR_BAD_SHAPE = 2,     /* a size is < 1, too large (D and row strides above 2^24 elements,
+                                   more than 2^31 - 1 tiles), or breaks a stated divisibility rule */
     HAWK_ERR_BAD_DTYPE = 3,     /* dtype is not a hawk_dtype this entry point supports */
     HAWK_ERR_WORKSPACE = 4,     /* workspace missing or smaller than the size query says */
     HAWK_ERR_LAUNCH = 5,        /* the HIP runtime refused a launch or copy */

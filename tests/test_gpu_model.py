@@ -314,11 +314,41 @@ def test_model_gradients_match_a_pure_torch_model_of_the_same_weights(fused_epil
         assert max_rel(capi.to_np(got[n]), capi.to_np(p.grad)) < 1e-3, n
 
 
+def _tensor_max_rel(a, b):
+    """max |a - b| / max |b| over one tensor (the benchmark's parity metric), on the GPU."""
+    a, b = a.float(), b.float()
+    return float((a - b).abs().max() / b.abs().max().clamp_min(1e-30))
+
+
+def _tensor_rel_l2(a, b):
+    a, b = a.float(), b.float()
+    return float((a - b).norm() / b.norm().clamp_min(1e-30))
+
+
 def test_readme_model_config_bf16_autocast_training_step():
     """The upstream README's model (vocab 32000, hidden = recurrent = 512, MLP 1024, 8 layers,
-    16 gate blocks, conv 4) on a 1 x 2048 batch under bf16 autocast, forward and backward,
-    for every combination of the fused-kernel switches, against the same weights run in fp32
-    with the torch-loop scan, the library conv and the library gate GEMMs."""
+    16 gate blocks, conv 4) on a 1 x 2048 batch under bf16 autocast, forward and backward, for
+    every combination of the fused-kernel switches.
+
+    Two references run the same weights with the torch-loop scan, a torch conv and the library
+    gate GEMMs in place of the kernels: one in fp32 throughout, one under the same bf16
+    autocast (scan operands rounded to bf16 with fp32 state, as upstream's
+    custom_fwd(cast_inputs=bfloat16) arranges, hawk/scan_fused.py:428; conv output in fp32, as
+    upstream's promotion gives, hawk/external.py:90).
+
+    The benchmark's bound for the hot path (max-rel 2e-2 per tensor) is what the kernel tests
+    assert, operator by operator.  It cannot be asserted on this whole model: under bf16
+    autocast every GEMM of eight layers rounds, and the two references above, which share the
+    scan and the conv, already differ by 1.3e-2 to 4.4e-2 per tensor (measured on an MI355X).
+    What is asserted per parameter instead:
+      * max-rel against the fp32 reference below 8e-2 (observed: up to 5.6e-2; a gradient off
+        by 10 % in scale fails); against the autocast reference the figure is only printed,
+        both sides of that comparison carrying bf16's noise (up to 7.5e-2 was seen);
+      * relative L2 error against the fp32 reference at most 1.5 times that of the autocast
+        reference (plus 5e-3), i.e. the kernels add no error of their own beyond bf16's, which
+        a wrong constant factor of a few per cent on any tensor would;
+      * cosine above 0.99.
+    """
     torch.manual_seed(3)
     cfg = hk.HawkConfig(vocab_size=32000, hidden_size=512, intermediate_size=1024, num_hidden_layers=8,
                         recurrent_size=512, num_blocks=16, conv_width=4)
@@ -330,21 +360,39 @@ def test_readme_model_config_bf16_autocast_training_step():
     import hawk_pytorch_amd.external as he
 
     def ref_scan(x, xg, ag, lam):
+        if torch.is_autocast_enabled():
+            with torch.autocast(device_type="cuda", enabled=False):
+                r = lambda t: t.to(torch.bfloat16).float()  # noqa: E731
+                return rglru_torch.rglru_scan_loop(r(x), r(xg), r(ag), lam.float()).to(torch.bfloat16)
         return rglru_torch.rglru_scan_loop(x, xg, ag, lam)
 
     def ref_conv(self, x, state=None):
-        return rglru_torch.conv1d_library(x, self.w, self.b)
+        # shifted slices times per-channel weights, promoted to fp32 (hawk/external.py:78-93)
+        W, T = self.w.shape[0], x.shape[1]
+        y = self.b.float().expand_as(x).clone()
+        for s_ in range(min(W, T)):
+            y[:, s_:, :] += x[:, : T - s_, :].float() * self.w[W - 1 - s_].float()
+        return y
 
-    cfg.fused_gates, cfg.fused_epilogue = False, False
-    old = hm.fused_linear_scan, he.Conv1D.forward
-    try:
-        hm.fused_linear_scan, he.Conv1D.forward = ref_scan, ref_conv
-        ref_loss = model(ids, ids)
-        ref_loss.backward()
-    finally:
-        hm.fused_linear_scan, he.Conv1D.forward = old
-    want = {n: p.grad.detach().float().clone() for n, p in model.named_parameters()}
+    def reference(autocast):
+        cfg.fused_gates, cfg.fused_epilogue = False, False
+        old = hm.fused_linear_scan, he.Conv1D.forward
+        model.zero_grad()
+        try:
+            hm.fused_linear_scan, he.Conv1D.forward = ref_scan, ref_conv
+            with torch.autocast(device_type="cuda", dtype=torch.bfloat16, enabled=autocast):
+                loss = model(ids, ids)
+            loss.backward()
+        finally:
+            hm.fused_linear_scan, he.Conv1D.forward = old
+        return loss.item(), {n: p.grad.detach().float().clone() for n, p in model.named_parameters()}
 
+    loss32, want32 = reference(False)
+    loss_ac, want_ac = reference(True)
+    ref_l2 = {n: _tensor_rel_l2(want_ac[n], want32[n]) for n in want32}
+    between = max(_tensor_max_rel(want_ac[n], want32[n]) for n in want32)
+
+    worst_ac, worst32, worst_l2 = 0.0, 0.0, 0.0
     for fused_gates, fused_epilogue in [(True, True), (True, False), (False, True), (False, False)]:
         cfg.fused_gates, cfg.fused_epilogue = fused_gates, fused_epilogue
         model.zero_grad()
@@ -352,12 +400,21 @@ def test_readme_model_config_bf16_autocast_training_step():
             loss = model(ids, ids)
         loss.backward()
         case = (fused_gates, fused_epilogue)
-        assert abs(loss.item() - ref_loss.item()) < 2e-2 * abs(ref_loss.item()), case
+        assert abs(loss.item() - loss_ac) < 2e-2 * abs(loss_ac), case
+        assert abs(loss.item() - loss32) < 2e-2 * abs(loss32), case
         for n, p in model.named_parameters():
-            a, b = p.grad.float().flatten(), want[n].flatten()
-            assert torch.isfinite(a).all(), (case, n)
+            assert torch.isfinite(p.grad).all(), (case, n)
+            e_ac, e32 = _tensor_max_rel(p.grad, want_ac[n]), _tensor_max_rel(p.grad, want32[n])
+            l2 = _tensor_rel_l2(p.grad, want32[n])
+            worst_ac, worst32, worst_l2 = max(worst_ac, e_ac), max(worst32, e32), max(worst_l2, l2 / ref_l2[n])
+            assert e32 < 8e-2, (case, n, e32, e_ac)
+            assert l2 <= 1.5 * ref_l2[n] + 5e-3, (case, n, l2, ref_l2[n])
+            a, b = p.grad.float().flatten(), want32[n].flatten()
             cos = float(torch.dot(a, b) / (a.norm() * b.norm() + 1e-30))
             assert cos > 0.99, (case, n, cos)
+    print(f"cfg1 gradients, worst per-tensor max-rel: {worst_ac:.2e} vs the autocast reference, "
+          f"{worst32:.2e} vs the fp32 reference (the two references differ by up to {between:.2e}); "
+          f"worst ratio of relative L2 errors, kernels / autocast reference: {worst_l2:.2f}")
 
 
 def test_training_step_replays_from_a_hip_graph():
@@ -629,3 +686,102 @@ def test_rounding_fp32_gate_weights_once_per_forward_changes_no_bit():
         he._CAST_WEIGHTS_MIN_ROWS = keep
     for a, b in zip(cast, plain):
         assert torch.equal(a, b)
+
+
+def test_upstream_decode_call_sequence_runs_on_this_cache_and_matches_the_fused_path():
+    """Upstream's own Hawk.forward, prefill and decode branches (hawk/hawk.py:153-203), replayed
+    call by call on this package's RNNCache, Conv1D, BlockDiagonalLinear and fused_linear_scan:
+    the re-binding of conv_state to a view of the input projection (:174), the window concat
+    (:169), update_conv_cache (:170), the conv over the 4-row window and its last row (:176-179),
+    the torch-op recurrence step (:137-151, :196) and update_cache (:190, :198).  Its outputs
+    must match the fused decode path, and a cache that went through the upstream sequence
+    (conv_state left as a strided view) must be accepted by the fused path afterwards."""
+    cfg = hk.HawkConfig(vocab_size=64, hidden_size=128, intermediate_size=256, num_hidden_layers=1,
+                        recurrent_size=256, num_blocks=4, conv_width=4)
+    torch.manual_seed(11)
+    block = hk.Hawk(cfg, use_cache=True).cuda()
+    torch.nn.init.normal_(block.resid_proj.weight, std=0.05)
+    torch.nn.init.normal_(block.rg_lru_input_gate.b, std=0.3)
+    torch.nn.init.normal_(block.rg_lru_a_gate.b, std=0.3)
+    block = block.to(torch.bfloat16).eval()
+    B, T, K, R = 2, 19, 5, cfg.recurrent_size
+    gen = torch.Generator("cuda").manual_seed(12)
+    xs = torch.randn(B, T + K + 1, cfg.hidden_size, device="cuda", generator=gen).to(torch.bfloat16)
+
+    def upstream_forward(x, layer_past):
+        warm = layer_past.current_cache_size > 0
+        xy = block.input_xy(x)
+        xb, yb = xy.chunk(2, dim=-1)
+        if warm:
+            xb = torch.cat([layer_past.conv_state, xb], dim=1)
+            layer_past.update_conv_cache(xb[:, -1:, ...])
+        else:
+            layer_past.conv_state = xb[:, -3:, ...]
+        u = block.conv1d(xb)
+        if warm:
+            u = u[:, -1:, ...]
+        if not warm:
+            xg, ag = block.rg_lru_input_gate(u), block.rg_lru_a_gate(u)
+            h = hk.fused_linear_scan(u, xg, ag, block.rg_lru_a_param.float())
+            layer_past.update_cache(h[:, -1:, :])
+        else:
+            gate_x = torch.sigmoid(block.rg_lru_input_gate(u))
+            gate_a = torch.sigmoid(block.rg_lru_a_gate(u))
+            log_a = -8.0 * gate_a.float() * F.softplus(block.rg_lru_a_param.float())
+            a = torch.exp(log_a)
+            normalized_x = u * gate_x * torch.sqrt(1.0 - torch.exp(2.0 * log_a)).to(u.dtype)
+            h = (a * layer_past.recc_state + normalized_x).to(u.dtype)
+            layer_past.update_cache(h[:, -1:, :])
+        return block.resid_proj(F.gelu(yb) * h)
+
+    with torch.no_grad():
+        up_cache = hk.RNNCache(R, xs.device, cfg.conv_width, batch_size=B)
+        fused_cache = hk.RNNCache(R, xs.device, cfg.conv_width, batch_size=B)
+        up_out = [upstream_forward(xs[:, :T], up_cache)]
+        assert not up_cache.conv_state.is_contiguous()          # the re-bound view of hawk/hawk.py:174
+        fused_out = [block(xs[:, :T], fused_cache)[0]]
+        for k in range(K):
+            step = xs[:, T + k: T + k + 1]
+            up_out.append(upstream_forward(step, up_cache))
+            fused_out.append(block(step, fused_cache)[0])
+        for k, (a, b) in enumerate(zip(up_out, fused_out)):
+            scale = float(a.float().abs().max())
+            assert float((a.float() - b.float()).abs().max()) < 2e-2 * scale, k
+        assert float((up_cache.conv_state.float() - fused_cache.conv_state.float()).abs().max()) == 0.0
+        err = (up_cache.recc_state.float() - fused_cache.recc_state.float()).abs().max()
+        assert float(err) < 2e-2 * float(fused_cache.recc_state.float().abs().max())
+        # the cache that upstream's sequence left behind (strided conv_state) now goes through
+        # the fused path
+        last = xs[:, T + K: T + K + 1]
+        a = block(last, up_cache)[0]
+        b = block(last, fused_cache)[0]
+        assert up_cache.conv_state.is_contiguous()
+        assert float((a.float() - b.float()).abs().max()) < 2e-2 * float(b.float().abs().max())
+
+
+def test_warm_cache_refuses_more_than_one_new_token():
+    cfg = _small_config()
+    model = hk.HawkModel(cfg, use_cache=True).cuda().eval()
+    ids = torch.randint(1, cfg.vocab_size, (1, 9), device="cuda")
+    with torch.no_grad():
+        _, caches = model(ids[:, :6], layer_past=model.new_cache(1))
+        with pytest.raises(AssertionError, match="one new token"):
+            model(ids[:, 6:9], layer_past=caches)
+
+
+def test_check_scan_status_reads_every_cached_workspace():
+    x, xg, ag, lam, _ = make_scan_inputs(2, 300, 128, seed=4)
+    dev = [capi.to_dev(a, "bf16") for a in (x, xg, ag)] + [capi.to_dev(lam, "f32")]
+    hk.fused_linear_scan(*dev)
+    hk.check_scan_status()           # all carries arrived: returns silently
+    from hawk_pytorch_amd import _lib
+    key = next(iter(_lib._workspaces))
+    ws = _lib._workspaces[key]
+    ws.view(torch.int32)[2] = 1      # what a tile that exhausted its wait leaves behind
+    try:
+        with pytest.raises(hk.HawkHipError, match="carry"):
+            hk.check_scan_status()
+    finally:
+        hk.release_workspaces()
+    hk.fused_linear_scan(*dev)
+    hk.check_scan_status()

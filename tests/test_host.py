@@ -68,8 +68,8 @@ def test_header_is_plain_c_and_links_against_the_library(tmp_path):
 
 
 def test_status_strings_are_distinct():
-    msgs = {_lib.status_string(s) for s in range(7)}
-    assert len(msgs) == 7 and _lib.status_string(0) == "ok"
+    msgs = {_lib.status_string(s) for s in range(8)}
+    assert len(msgs) == 8 and _lib.status_string(0) == "ok"
     assert "unknown" in _lib.status_string(99)
 
 
@@ -99,6 +99,27 @@ def test_argument_validation_needs_no_gpu():
     assert lib.hawk_rglru_scan_fwd_mixed(*args, 1, 8, 64, 0, 1, None, 0, None) == _lib.HAWK_ERR_BAD_DTYPE
     assert lib.hawk_rglru_scan_bwd_mixed(*bwd, 1, 8, 64, 0, 1, p, 1 << 20, None) == _lib.HAWK_ERR_BAD_DTYPE
     assert lib.hawk_rglru_scan_bwd_mixed(*bwd, 1, 8, 64, 1, 0, None, 0, None) == _lib.HAWK_ERR_WORKSPACE
+
+
+def test_scan_shape_limits_are_checked_before_any_launch():
+    """Row and tile byte offsets are formed in 32 bits inside the kernels: D and row strides
+    beyond 2^24 elements are refused, as are shapes whose carries do not fit the fixed scratch
+    array of the entry point that allocates nothing."""
+    lib = _lib.load()
+    buf = (ctypes.c_char * 4096)()
+    p = (ctypes.addressof(buf) + 15) & ~15
+    args = [p, p, p, p, p]
+    big_d = (1 << 24) + 64
+    assert lib.hawk_rglru_scan_fwd(*args, 1, 8, big_d, 0, None, 0, None) == _lib.HAWK_ERR_BAD_SHAPE
+    assert lib.hawk_rglru_scan_fwd(*args, 1, 8, big_d, 1, None, 0, None) == _lib.HAWK_ERR_BAD_SHAPE
+    assert lib.hawk_rglru_scan_bwd(*([p] * 10), 1, 8, big_d, 0, p, 1 << 20, None) == _lib.HAWK_ERR_BAD_SHAPE
+    assert lib.hawk_scan_workspace_bytes(1, 8, big_d, 0) == 0
+    assert lib.hawk_scan_workspace_bytes(1, 8, 1 << 24, 0) > 0
+    assert lib.hawk_rglru_scan_fwd_static(*args, 1, 8, big_d, 0, None) == _lib.HAWK_ERR_BAD_SHAPE
+    # 64 tiles in time x 8 x 2560 channels x 24 bytes = 31.5 MB of carry words > 16 MiB
+    assert lib.hawk_rglru_scan_fwd_static(*args, 8, 8192, 2560, 0, None) == _lib.HAWK_ERR_SCRATCH_LIMIT
+    assert lib.hawk_rglru_scan_fwd_static(None, p, p, p, p, 1, 8, 64, 0, None) == _lib.HAWK_ERR_NULL_POINTER
+    assert lib.hawk_rglru_scan_fwd_static(*args, 1, 8, 64, 5, None) == _lib.HAWK_ERR_BAD_DTYPE
 
 
 def test_workspace_size_queries():
