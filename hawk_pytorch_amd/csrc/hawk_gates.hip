@@ -52,6 +52,11 @@ constexpr int kNumCU = 256;
 #ifndef HAWK_GATE_SMALL_M
 #define HAWK_GATE_SMALL_M 512
 #endif
+// Tiles in flight per workgroup of the weight-gradient kernel (bf16 operands; half as many fp32).
+#ifndef HAWK_GATE_DW_SETS
+#define HAWK_GATE_DW_SETS 2
+#endif
+
 
 // Weight fetches that go through a buffer resource (scalar base, one per-lane offset, scalar
 // per-access offset) use the default cache policy: every workgroup re-reads them.
@@ -812,7 +817,8 @@ __global__ __launch_bounds__(kGateThreads, 1) void gate_proj_bwd_input_kernel(
 // Weight and bias gradients:
 //   dw_g[h, i, j] = sum_m x[m, h*bw + i] dg[m, h*bw + j],   db_g[c] = sum_m dg[m, c]
 // The contraction runs over the rows, so both operands are needed "column-wise".  A
-// workgroup (msplit, 256-channel group, gate) walks over its share of the rows 32 at a time;
+// workgroup (msplit, 256-channel group, gate) walks over its share of the row tiles (32 rows
+// each, dealt round-robin to the splits);
 // waves 0-7 fetch the x tile and waves 8-15 the gradient tile, each lane 8 rows of two
 // adjacent channels, transpose them in registers and write them to LDS as
 // [8-row chunk][channel][8 rows], which is exactly the 16 bytes an MFMA operand lane needs
@@ -824,19 +830,6 @@ constexpr int kChunkBytes = kGroup * 16;          // one 8-row chunk of a transp
 constexpr int kTTileBytes = 4 * kChunkBytes;      // 32 rows
 
 template <typename ET>
-__device__ __forceinline__ void load_pair(const ET* p, bool ok, uint32_t (&raw)[2]);
-template <>
-__device__ __forceinline__ void load_pair<bf16_t>(const bf16_t* p, bool ok, uint32_t (&raw)[2]) {
-    raw[0] = ok ? *reinterpret_cast<const uint32_t*>(p) : 0u;
-    raw[1] = 0u;
-}
-template <>
-__device__ __forceinline__ void load_pair<float>(const float* p, bool ok, uint32_t (&raw)[2]) {
-    const u32x2 v = ok ? *reinterpret_cast<const u32x2*>(p) : u32x2{0u, 0u};
-    raw[0] = v.x;
-    raw[1] = v.y;
-}
-template <typename ET>
 __device__ __forceinline__ uint32_t pair_as_bf16(const uint32_t (&raw)[2]) {
     if constexpr (sizeof(ET) == 2) return raw[0];
     return pack_bf16x2(__uint_as_float(raw[0]), __uint_as_float(raw[1]));
@@ -845,7 +838,7 @@ __device__ __forceinline__ uint32_t pair_as_bf16(const uint32_t (&raw)[2]) {
 template <typename XT, typename GT, int BW>
 __global__ __launch_bounds__(kGateThreads, 1) void gate_proj_bwd_weights_kernel(
     const XT* __restrict__ x, const GT* __restrict__ dg_i, const GT* __restrict__ dg_a, float* __restrict__ part_w,
-    float* __restrict__ part_b, int M, int D, int nb, int rows_per_split) {
+    float* __restrict__ part_b, int M, int D, int nb) {
     constexpr int G = kGroup / BW;                 // blocks per group
     constexpr int NT = BW / 32;                    // 32-wide tiles per block side
     constexpr int TI = BW >= 256 ? 2 : 1;          // output tiles per wave: TI x TJ
@@ -860,9 +853,12 @@ __global__ __launch_bounds__(kGateThreads, 1) void gate_proj_bwd_weights_kernel(
     const int w = __builtin_amdgcn_readfirstlane(tid / kWave);
     const int split = blockIdx.x, group = blockIdx.y, gate = blockIdx.z;
     const GT* dg = gate ? dg_a : dg_i;
-    const int row_begin = split * rows_per_split;
-    const int row_end = min(row_begin + rows_per_split, M);
-    const int ntiles = (row_end - row_begin + kTileRows - 1) / kTileRows;
+    // Row tiles are dealt out round-robin: split s takes tiles s, s + nsplit, ...  All workgroups
+    // of the launch then read neighbouring rows at any moment, three sequential streams (x and
+    // the two gradients) instead of three per split; memory serves few streams faster.
+    const int nsplit = gridDim.x;
+    const int all_tiles = (M + kTileRows - 1) / kTileRows;
+    const int ntiles = split < all_tiles ? (all_tiles - split + nsplit - 1) / nsplit : 0;
 
     // ---- loader role: 8 rows x 2 channels per lane
     const bool loads_x = w < 8;
@@ -870,18 +866,46 @@ __global__ __launch_bounds__(kGateThreads, 1) void gate_proj_bwd_weights_kernel(
     const int c2 = (w & 1) * 64 + lane;                          // channel pair within the group
     const int lch = group * kGroup + 2 * c2;
     const bool ch_ok = lch < D;
-    uint32_t ra[8][RAWW], rb[8][RAWW];
+    // Register sets that hold tiles on their way from memory: tile k lands in set k % kSets and is
+    // staged into LDS kSets - 1 steps after its loads were issued.  A step lasts well under a
+    // microsecond and a load under traffic takes several, so the depth of this ring, not the
+    // arithmetic, sets the pace of the loop.
+    constexpr int kSets = (RAWW == 1) ? HAWK_GATE_DW_SETS : (HAWK_GATE_DW_SETS / 4 >= 1 ? (HAWK_GATE_DW_SETS / 4) * 2 : 2);
+    static_assert(kSets >= 2 && kSets % 2 == 0, "an even number of register sets");
+    uint32_t rs[kSets][8][RAWW];
+    // Loads go through a buffer resource that covers the rows of the tile which exist: rows past
+    // M, tiles past the last one and the channels past D of the last group read as zeros without a
+    // branch, so the loop body is straight-line code and the compiler can wait for exactly the
+    // loads a step needs while younger ones stay in flight.
+    constexpr bool kSameWidth = sizeof(XT) == sizeof(GT);
+    const char* src = loads_x ? reinterpret_cast<const char*>(x) : reinterpret_cast<const char*>(dg);
+    const uint32_t esz = loads_x ? (uint32_t)sizeof(XT) : (uint32_t)sizeof(GT);
+    const uint32_t row_bytes = (uint32_t)D * esz;
+    const uint32_t lane_bytes = ch_ok ? (uint32_t)lch * esz : 0x80000000u;
     auto load_rows = [&](int t, uint32_t (&r)[8][RAWW]) {
-        const int row0 = row_begin + t * kTileRows + 8 * q;
+        const int row0 = min((split + t * nsplit) * kTileRows + 8 * q, M);
+        const int rows = (t < ntiles) ? min(M - row0, 8) : 0;
+        const rsrc_t rs_ = make_rsrc(src + (size_t)row0 * row_bytes, (uint32_t)rows * row_bytes);
+        auto narrow = [&](int k) {
+            r[k][0] = __builtin_amdgcn_raw_buffer_load_b32(rs_, lane_bytes, k * row_bytes, kAuxDefault);
+            if (RAWW > 1) r[k][RAWW - 1] = 0u;
+        };
+        auto wide = [&](int k) {
+            const u32x2 v = __builtin_bit_cast(u32x2, __builtin_amdgcn_raw_buffer_load_b64(rs_, lane_bytes, k * row_bytes,
+                                                                                           kAuxDefault));
+            r[k][0] = v.x;
+            r[k][RAWW - 1] = v.y;
+        };
 #pragma unroll
         for (int k = 0; k < 8; ++k) {
-            const bool ok = ch_ok && t < ntiles && row0 + k < row_end;
-            const size_t off = ok ? (size_t)(row0 + k) * D + lch : 0;
-            uint32_t tmp[2];
-            if (loads_x) load_pair<XT>(x + off, ok, tmp);
-            else load_pair<GT>(dg + off, ok, tmp);
-#pragma unroll
-            for (int z = 0; z < RAWW; ++z) r[k][z] = tmp[z];
+            if constexpr (kSameWidth) {
+                if constexpr (sizeof(XT) == 2) narrow(k);
+                else wide(k);
+            } else if ((sizeof(XT) == 2) == loads_x) {   // the two roles differ in width: a wave-uniform branch
+                narrow(k);
+            } else {
+                wide(k);
+            }
         }
     };
     float colsum[2] = {0.0f, 0.0f};
@@ -890,36 +914,41 @@ __global__ __launch_bounds__(kGateThreads, 1) void gate_proj_bwd_weights_kernel(
 #pragma unroll
         for (int k = 0; k < 8; ++k) {
             uint32_t tmp[2] = {r[k][0], RAWW > 1 ? r[k][RAWW - 1] : 0u};
-            d[k] = loads_x ? pair_as_bf16<XT>(tmp) : pair_as_bf16<GT>(tmp);
+            if constexpr (sizeof(XT) == sizeof(GT)) d[k] = pair_as_bf16<XT>(tmp);
+            else d[k] = loads_x ? pair_as_bf16<XT>(tmp) : pair_as_bf16<GT>(tmp);
         }
-        if (!loads_x) {
+        // column sums of the gradient tile, for the bias gradient (the x loaders add up x's
+        // columns too, which nobody reads: cheaper than a branch in the tile loop)
 #pragma unroll
-            for (int k = 0; k < 8; ++k) {
-                colsum[0] += bf16_lo(d[k]);
-                colsum[1] += bf16_hi(d[k]);
-            }
+        for (int k = 0; k < 8; ++k) {
+            colsum[0] += bf16_lo(d[k]);
+            colsum[1] += bf16_hi(d[k]);
         }
         // channel 2 c2 takes the low halves, channel 2 c2 + 1 the high halves; rows in order
         u32x4 lo, hi;
-        lo.x = (d[0] & 0xffffu) | (d[1] << 16);
-        lo.y = (d[2] & 0xffffu) | (d[3] << 16);
-        lo.z = (d[4] & 0xffffu) | (d[5] << 16);
-        lo.w = (d[6] & 0xffffu) | (d[7] << 16);
-        hi.x = (d[0] >> 16) | (d[1] & 0xffff0000u);
-        hi.y = (d[2] >> 16) | (d[3] & 0xffff0000u);
-        hi.z = (d[4] >> 16) | (d[5] & 0xffff0000u);
-        hi.w = (d[6] >> 16) | (d[7] & 0xffff0000u);
+        lo.x = __builtin_amdgcn_perm(d[1], d[0], 0x05040100u);
+        lo.y = __builtin_amdgcn_perm(d[3], d[2], 0x05040100u);
+        lo.z = __builtin_amdgcn_perm(d[5], d[4], 0x05040100u);
+        lo.w = __builtin_amdgcn_perm(d[7], d[6], 0x05040100u);
+        hi.x = __builtin_amdgcn_perm(d[1], d[0], 0x07060302u);
+        hi.y = __builtin_amdgcn_perm(d[3], d[2], 0x07060302u);
+        hi.z = __builtin_amdgcn_perm(d[5], d[4], 0x07060302u);
+        hi.w = __builtin_amdgcn_perm(d[7], d[6], 0x07060302u);
         unsigned char* p = &sT[buf][loads_x ? 0 : 1][q * kChunkBytes + (2 * c2) * 16];
         *reinterpret_cast<u32x4*>(p) = lo;
         *reinterpret_cast<u32x4*>(p + 16) = hi;
     };
 
     // ---- compute role: TI x TJ output tiles of block `blk`
-    const int blk = w / WPB;                       // block within the group (idle if >= G)
+    const int blk_raw = w / WPB;                   // block within the group (idle if >= G)
     const int wi = w % WPB;
     const int i0 = (wi / (NT / TJ)) * TI, j0 = (wi % (NT / TJ)) * TJ;
-    const int h = group * G + blk;
-    const bool computes = blk < G && h < nb;
+    const int h = group * G + blk_raw;
+    const bool computes = blk_raw < G && h < nb;
+    // waves without a block of their own run the same instruction stream on block 0 (their sums
+    // are dropped), so that the tile loop has no branch and the matrix products of a tile can be
+    // interleaved with the staging of the next one
+    const int blk = computes ? blk_raw : 0;
     const int col = lane & 31;
     const int a_off = (lane >> 5) * kChunkBytes + (blk * BW + i0 * 32 + col) * 16;
     const int b_off = (lane >> 5) * kChunkBytes + (blk * BW + j0 * 32 + col) * 16;
@@ -929,38 +958,42 @@ __global__ __launch_bounds__(kGateThreads, 1) void gate_proj_bwd_weights_kernel(
 #pragma unroll
         for (int b = 0; b < TJ; ++b) acc[a][b] = f32x16{};
 
-    load_rows(0, ra);
-    load_rows(1, rb);
-    stage_rows(0, ra);
-    load_rows(2, ra);
+#pragma unroll
+    for (int k = 0; k < kSets; ++k) load_rows(k, rs[k]);
+    stage_rows(0, rs[0]);
+    load_rows(kSets, rs[0]);
     __syncthreads();
 
     auto step = [&](int t, int cur, uint32_t (&rnext)[8][RAWW]) {
-        if (computes) {
+        {
+            bf16x8 fa[2][TI], fb[2][TJ];
 #pragma unroll
             for (int ks = 0; ks < 2; ++ks) {
-                bf16x8 fa[TI], fb[TJ];
 #pragma unroll
                 for (int a = 0; a < TI; ++a)
-                    fa[a] = *reinterpret_cast<const bf16x8*>(&sT[cur][0][2 * ks * kChunkBytes + a_off + a * 32 * 16]);
+                    fa[ks][a] = *reinterpret_cast<const bf16x8*>(&sT[cur][0][2 * ks * kChunkBytes + a_off + a * 32 * 16]);
 #pragma unroll
                 for (int b = 0; b < TJ; ++b)
-                    fb[b] = *reinterpret_cast<const bf16x8*>(&sT[cur][1][2 * ks * kChunkBytes + b_off + b * 32 * 16]);
+                    fb[ks][b] = *reinterpret_cast<const bf16x8*>(&sT[cur][1][2 * ks * kChunkBytes + b_off + b * 32 * 16]);
+            }
+#pragma unroll
+            for (int ks = 0; ks < 2; ++ks)
 #pragma unroll
                 for (int a = 0; a < TI; ++a)
 #pragma unroll
                     for (int b = 0; b < TJ; ++b)
-                        acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[a], fb[b], acc[a][b], 0, 0, 0);
-            }
+                        acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[ks][a], fb[ks][b], acc[a][b], 0, 0, 0);
         }
+        // tile t + 1 into the other LDS stage, tile t + 1 + kSets into the registers it leaves
         stage_rows(cur ^ 1, rnext);
-        load_rows(t + 3, rnext);
+        load_rows(t + 1 + kSets, rnext);
         __syncthreads();
     };
-    for (int t = 0; t < ntiles; t += 2) {
-        step(t, 0, rb);
-        if (t + 1 >= ntiles) break;
-        step(t + 1, 1, ra);
+    for (int t = 0; t < ntiles; t += kSets) {
+#pragma unroll
+        for (int k = 0; k < kSets; ++k) {
+            if (t + k < ntiles) step(t + k, k & 1, rs[(k + 1) % kSets]);
+        }
     }
 
     // ---- partial results of this split
@@ -1133,11 +1166,10 @@ int weight_splits(int M, int D) {
 template <typename XT, typename GT, int BW>
 int launch_gate_bwd_weights(const void* x, const void* dg_i, const void* dg_a, float* part_w, float* part_b, int M,
                             int D, int nb, int nsplit, hipStream_t st) {
-    const int rows_per_split = ceil_div(ceil_div(M, nsplit), kTileRows) * kTileRows;
     hipLaunchKernelGGL((gate_proj_bwd_weights_kernel<XT, GT, BW>),
                        dim3((unsigned)nsplit, (unsigned)ceil_div(D, kGroup), 2u), dim3(kGateThreads), 0, st,
                        static_cast<const XT*>(x), static_cast<const GT*>(dg_i), static_cast<const GT*>(dg_a), part_w,
-                       part_b, M, D, nb, rows_per_split);
+                       part_b, M, D, nb);
     return hipGetLastError() == hipSuccess ? HAWK_OK : HAWK_ERR_LAUNCH;
 }
 
@@ -1266,3 +1298,4 @@ int gate_proj_bwd_weights(const void* x, const void* dg_i, const void* dg_a, flo
 }
 
 }  // namespace hawk
+

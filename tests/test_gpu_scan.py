@@ -243,6 +243,19 @@ def test_full_benchmark_shapes_bf16(B, T, D, lo, hi):
     assert torch.equal(h2.float(), h.float() * 2)
 
 
+@pytest.mark.parametrize("B,T,D,dtype", [
+    (8, 2100, 1024, "bf16"),    # 64 chains, last tile cut short
+    (8, 1000, 2560, "bf16"),    # 160 chains (the short backward tiles), few tiles in time
+    (16, 1345, 1280, "bf16"),   # 160 chains, ragged
+    (8, 1500, 1024, "f32"),     # one channel per lane
+    (12, 1111, 960, "f32"),
+])
+def test_launches_of_a_thousand_tiles_and_more(B, T, D, dtype):
+    """Launches with more tiles than the device holds at once (several rounds of workgroups,
+    many chains in flight): full parity against the oracle, all channels."""
+    _run_case(B, T, D, dtype, seed=B + T)
+
+
 def test_scan_launches_replay_correctly_from_a_hip_graph():
     """Forward, backward and the gated pair captured once and replayed several times, with
     eager launches on the same workspace in between; every replay must reproduce the eager
