@@ -87,6 +87,11 @@ struct Row8<bf16_t> {
     __device__ __forceinline__ void load(const bf16_t* p, bool ok) {
         v = ok ? *reinterpret_cast<const u32x4*>(p) : u32x4{0u, 0u, 0u, 0u};
     }
+    // through a buffer resource: bytes outside it read as zeros, without a branch
+    __device__ __forceinline__ void load_buf(rsrc_t r, uint32_t off) { v = buffer_load<u32x4>(r, off, 0u); }
+    __device__ __forceinline__ void load_buf_default(rsrc_t r, uint32_t off) {
+        v = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(r, off, 0u, kAuxDefault));
+    }
     __device__ __forceinline__ u32x4 as_bf16() const { return v; }
     __device__ __forceinline__ void as_f32(f32x4& a, f32x4& b) const {
         a = f32x4{bf16_lo(v.x), bf16_hi(v.x), bf16_lo(v.y), bf16_hi(v.y)};
@@ -100,6 +105,10 @@ struct Row8<float> {
         const f32x4 z = {0.0f, 0.0f, 0.0f, 0.0f};
         lo = ok ? *reinterpret_cast<const f32x4*>(p) : z;
         hi = ok ? *reinterpret_cast<const f32x4*>(p + 4) : z;
+    }
+    __device__ __forceinline__ void load_buf(rsrc_t r, uint32_t off) {
+        lo = buffer_load<f32x4>(r, off, 0u);
+        hi = buffer_load<f32x4>(r, off, 16u);
     }
     __device__ __forceinline__ u32x4 as_bf16() const {
         return u32x4{pack_bf16x2(lo.x, lo.y), pack_bf16x2(lo.z, lo.w), pack_bf16x2(hi.x, hi.y),
@@ -199,11 +208,16 @@ __global__ __launch_bounds__(kGateThreads, 1) void gate_proj_fwd_kernel(
     const int lrow = tid >> 5, lc8 = tid & 31;
     const int lcol = group * kGroup + lc8 * 8;
     const bool col_ok = lcol < D;
+    // (through a buffer resource that covers the rows of the tile which exist: no branch)
+    const uint32_t x_row_bytes = (uint32_t)D * (uint32_t)sizeof(XT);
+    const uint32_t x_off = col_ok ? (uint32_t)(lrow * D + lcol) * (uint32_t)sizeof(XT) : 0x80000000u;
     auto load_tile = [&](int it, Row8<XT>& r) {
-        const int t = worker + it * nworkers;
-        const int row = t * kTileRows + lrow;
-        const bool ok = col_ok && t < ntiles && row < M;
-        r.load(x + (ok ? (size_t)row * D + lcol : 0), ok);
+        const int t = min(worker + it * nworkers, ntiles);   // past the last tile: an empty window
+        const int row0 = min(t * kTileRows, M);
+        if constexpr (sizeof(XT) == 2)
+            r.load_buf_default(make_rsrc(x + (size_t)row0 * D, (uint32_t)min(M - row0, kTileRows) * x_row_bytes), x_off);
+        else
+            r.load_buf(make_rsrc(x + (size_t)row0 * D, (uint32_t)min(M - row0, kTileRows) * x_row_bytes), x_off);
     };
     auto stage_tile = [&](int buf, const Row8<XT>& r) {
         *reinterpret_cast<u32x4*>(sA + buf * kATileBytes + lrow * kARowBytes + lc8 * 16) = r.as_bf16();
@@ -717,13 +731,14 @@ __global__ __launch_bounds__(kGateThreads, 1) void gate_proj_bwd_input_kernel(
     const int lrow = tid >> 5, lc8 = tid & 31;
     const int lcol = group * kGroup + lc8 * 8;
     const bool col_ok = lcol < D;
+    const uint32_t g_row_bytes = (uint32_t)D * (uint32_t)sizeof(GT);
+    const uint32_t g_off = col_ok ? (uint32_t)(lrow * D + lcol) * (uint32_t)sizeof(GT) : 0x80000000u;
     auto load_tile = [&](int it, Row8<GT>& r0, Row8<GT>& r1) {
-        const int t = worker + it * nworkers;
-        const int row = t * kTileRows + lrow;
-        const bool ok = col_ok && t < ntiles && row < M;
-        const size_t off = ok ? (size_t)row * D + lcol : 0;
-        r0.load(dxg + off, ok);
-        r1.load(dag + off, ok);
+        const int t = min(worker + it * nworkers, ntiles);   // past the last tile: an empty window
+        const int row0 = min(t * kTileRows, M);
+        const uint32_t window = (uint32_t)min(M - row0, kTileRows) * g_row_bytes;
+        r0.load_buf(make_rsrc(dxg + (size_t)row0 * D, window), g_off);
+        r1.load_buf(make_rsrc(dag + (size_t)row0 * D, window), g_off);
     };
     auto stage_tile = [&](int buf, const Row8<GT>& r0, const Row8<GT>& r1) {
         unsigned char* p = sA + (2 * buf) * kATileBytes + lrow * kARowBytes + lc8 * 16;
@@ -760,7 +775,12 @@ __global__ __launch_bounds__(kGateThreads, 1) void gate_proj_bwd_input_kernel(
         const int row = (worker + it * nworkers) * kTileRows + lrow;
         const bool out_ok = col_ok && row < M;
         Row8<DT> radd;
-        if constexpr (ADD) radd.load(addend + (out_ok ? (size_t)row * D + lcol : 0), out_ok);
+        if constexpr (ADD) {
+            const int arow0 = min((worker + it * nworkers) * kTileRows, M);
+            const uint32_t a_row_bytes = (uint32_t)D * (uint32_t)sizeof(DT);
+            radd.load_buf(make_rsrc(addend + (size_t)arow0 * D, (uint32_t)min(M - arow0, kTileRows) * a_row_bytes),
+                          col_ok ? (uint32_t)(lrow * D + lcol) * (uint32_t)sizeof(DT) : 0x80000000u);
+        }
         f32x16 acc = {};
         const unsigned char* a_base = sA + (2 * cur) * kATileBytes + a_off;
         constexpr int kBatch = KS < 4 ? KS : 4;
