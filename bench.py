@@ -65,14 +65,16 @@ HBM_PEAK_GBS = 8000.0
 # with the digest of the kernel sources they were measured on.  A record taken on other
 # sources is stale and is not reported.
 TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic.json")
-KERNEL_SOURCES = ("hawk_scan.hip", "hawk_gates.hip", "hawk_conv.hip", "hawk_device.h")
+KERNEL_SOURCES = {"gates": ("hawk_gates.hip", "hawk_device.h")}
+SCAN_KERNEL_SOURCES = ("hawk_scan.hip", "hawk_conv.hip", "hawk_device.h")
 
 
-def kernel_source_digest():
+def kernel_source_digest(workload):
+    """Digest of the sources of the kernels that `workload` times."""
     import hashlib
 
     h = hashlib.sha256()
-    for name in KERNEL_SOURCES:
+    for name in KERNEL_SOURCES.get(workload, SCAN_KERNEL_SOURCES):
         with open(os.path.join(ROOT, "hawk_pytorch_amd", "csrc", name), "rb") as f:
             h.update(f.read())
     return h.hexdigest()[:16]
@@ -86,7 +88,7 @@ def measured_traffic(workload):
             rec = json.load(f).get(workload)
     except (OSError, ValueError):
         return None
-    if not rec or rec.get("kernel_source_digest") != kernel_source_digest():
+    if not rec or rec.get("kernel_source_digest") != kernel_source_digest(workload):
         return None
     return float(rec["fetch_bytes"]) + float(rec["write_bytes"])
 
@@ -108,7 +110,7 @@ def record_traffic(workload, fetch_bytes, write_bytes, note):
         commit = None
     data[workload] = {
         "fetch_bytes": float(fetch_bytes), "write_bytes": float(write_bytes),
-        "kernel_source_digest": kernel_source_digest(), "commit_before": commit,
+        "kernel_source_digest": kernel_source_digest(workload), "commit_before": commit,
         "date": datetime.date.today().isoformat(), "note": note,
     }
     with open(TRAFFIC_FILE, "w") as f:

@@ -65,6 +65,12 @@ SIGNATURES = {
         [_c_void_p] * 2 + [ctypes.c_longlong] + [_c_void_p] * 8 + [ctypes.c_longlong] + [_c_void_p] * 2
         + [_c_int] * 7 + [_c_void_p],
     ),
+    "hawk_decode_core_workspace_bytes": (_c_size_t, [_c_int] * 3),
+    "hawk_decode_core_step_ws": (
+        _c_int,
+        [_c_void_p] * 2 + [ctypes.c_longlong] + [_c_void_p] * 8 + [ctypes.c_longlong] + [_c_void_p] * 2
+        + [_c_int] * 7 + [_c_void_p, _c_size_t, _c_void_p],
+    ),
     "hawk_gate_proj_fwd": (_c_int, [_c_void_p] * 7 + [_c_int] * 6 + [_c_void_p]),
     "hawk_gate_proj_bwd_input": (_c_int, [_c_void_p] * 6 + [_c_int] * 6 + [_c_void_p]),
     "hawk_gate_proj_bwd_weights_workspace_bytes": (_c_size_t, [_c_int] * 3),
@@ -191,11 +197,29 @@ def scan_workspace(dev: torch.device, nbytes: int) -> torch.Tensor:
     return ws
 
 
+_decode_workspaces: dict = {}
+
+
+def decode_workspace(dev: torch.device, nbytes: int) -> torch.Tensor:
+    """Zeroed counters for hawk_decode_core_step_ws, one buffer per (device, stream); every call
+    leaves them zero, so all layers and steps on a stream share it."""
+    if torch.cuda.is_current_stream_capturing():
+        return torch.zeros(max(nbytes, 4), dtype=torch.uint8, device=dev)  # the graph's own, zeroed by a fill kernel
+    key = (_device_index(dev), stream_ptr(dev))
+    with _lock:
+        ws = _decode_workspaces.get(key)
+        if ws is None or ws.numel() < nbytes:
+            ws = torch.zeros(max(nbytes, 4096), dtype=torch.uint8, device=dev)
+            _decode_workspaces[key] = ws
+    return ws
+
+
 def release_workspaces() -> None:
-    """Drop every cached scan workspace (they are re-created on demand)."""
+    """Drop every cached scan and decode workspace (they are re-created on demand)."""
     with _lock:
         _workspaces.clear()
         _captured.clear()
+        _decode_workspaces.clear()
 
 
 def _flag_of(ws: torch.Tensor, dev: torch.device) -> int:

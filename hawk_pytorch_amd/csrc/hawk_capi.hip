@@ -234,10 +234,16 @@ int hawk_decode_core_supported(int D, int num_blocks, int W) {
     return (W >= 1 && W <= 8 && hawk_gate_proj_supported(D, num_blocks)) ? 1 : 0;
 }
 
-int hawk_decode_core_step(void* conv_state, const void* x_new, long long ldx, const float* conv_w,
-                          const float* conv_b, const void* w_i, const float* b_i, const void* w_a, const float* b_a,
-                          const float* a_param, const void* y, long long ldy, void* recc_state, void* out, int B, int D,
-                          int num_blocks, int W, int dtype, int w_dtype, int state_dtype, void* stream) {
+size_t hawk_decode_core_workspace_bytes(int B, int D, int num_blocks) {
+    if (B < 1 || !hawk_gate_proj_supported(D, num_blocks)) return 0;
+    return hawk::decode_core_workspace_bytes(B, D, num_blocks);
+}
+
+int hawk_decode_core_step_ws(void* conv_state, const void* x_new, long long ldx, const float* conv_w,
+                             const float* conv_b, const void* w_i, const float* b_i, const void* w_a, const float* b_a,
+                             const float* a_param, const void* y, long long ldy, void* recc_state, void* out, int B,
+                             int D, int num_blocks, int W, int dtype, int w_dtype, int state_dtype,
+                             void* workspace_device, size_t workspace_bytes, void* stream) {
     if (!x_new || !conv_w || !conv_b || !w_i || !w_a || !a_param || !y || !recc_state || !out ||
         (W > 1 && !conv_state))
         return HAWK_ERR_NULL_POINTER;
@@ -248,8 +254,22 @@ int hawk_decode_core_step(void* conv_state, const void* x_new, long long ldx, co
     if (!aligned16(x_new) || (conv_state && !aligned16(conv_state)) || !aligned16(w_i) || !aligned16(w_a) ||
         !aligned_elem(y, dtype) || !aligned_elem(recc_state, state_dtype) || !aligned_elem(out, dtype))
         return HAWK_ERR_ALIGNMENT;
+    if (workspace_device != nullptr) {
+        if ((reinterpret_cast<uintptr_t>(workspace_device) & 3u) != 0) return HAWK_ERR_ALIGNMENT;
+        if (workspace_bytes < hawk::decode_core_workspace_bytes(B, D, num_blocks)) return HAWK_ERR_WORKSPACE;
+    }
     return hawk::decode_core_step(conv_state, x_new, ldx, conv_w, conv_b, w_i, b_i, w_a, b_a, a_param, y, ldy,
-                                  recc_state, out, B, D, num_blocks, W, w_dtype, state_dtype, as_stream(stream));
+                                  recc_state, out, B, D, num_blocks, W, w_dtype, state_dtype, workspace_device,
+                                  workspace_bytes, as_stream(stream));
+}
+
+int hawk_decode_core_step(void* conv_state, const void* x_new, long long ldx, const float* conv_w,
+                          const float* conv_b, const void* w_i, const float* b_i, const void* w_a, const float* b_a,
+                          const float* a_param, const void* y, long long ldy, void* recc_state, void* out, int B, int D,
+                          int num_blocks, int W, int dtype, int w_dtype, int state_dtype, void* stream) {
+    return hawk_decode_core_step_ws(conv_state, x_new, ldx, conv_w, conv_b, w_i, b_i, w_a, b_a, a_param, y, ldy,
+                                    recc_state, out, B, D, num_blocks, W, dtype, w_dtype, state_dtype, nullptr, 0,
+                                    stream);
 }
 
 int hawk_gate_proj_fwd(const void* x, const void* w_i, const float* b_i, const void* w_a, const float* b_a,

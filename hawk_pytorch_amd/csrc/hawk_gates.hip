@@ -469,8 +469,15 @@ __global__ __launch_bounds__(kSmallWaves* kWave, sizeof(XT) == 2 ? 4 : 2) void g
 // gate's earlier does not shorten it), the conv (2.9 us) and the recurrence (1.6 us).  One
 // workgroup per (32 rows, block) is 80 workgroups there: what the launch saves in starts it
 // loses to running on a third of the device, and its gain is on the host side (one call
-// instead of three plus a copy).  Cutting a block's columns over more workgroups would need the
-// window roll out of the kernel: they would read rows that another of them overwrites.
+// instead of three plus a copy).
+//
+// With a workspace of counters the output columns of a block are cut over NS workgroups
+// (NS = 2 or 4: 64 KiB of weights each at a width of 256 instead of 256 KiB through one L1, and
+// four times the compute units).  Every one of them needs the conv output of all the block's
+// channels, so each computes it from the window, but none rolls the window while reading: a
+// workgroup that has read it (its loads have returned) counts itself in on the (rows, block)
+// counter, and the one that counts in last, when no reader is left, rolls the window at the end
+// of its work and sets the counter back to zero for the next launch.
 // ---------------------------------------------------------------------------------------
 constexpr int kCoreWaves = 8;
 constexpr int kCoreMaxW = 8;
@@ -491,16 +498,18 @@ struct CoreLds {
 // follows behind it
 __device__ __forceinline__ void wave_lds_fence() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
 
-template <typename WT, typename ST, int BW>
+template <typename WT, typename ST, int BW, int NS>
 __global__ __launch_bounds__(kCoreWaves* kWave, 1) void decode_core_kernel(
     bf16_t* __restrict__ conv_state, const bf16_t* __restrict__ x_new, size_t ldx, const float* __restrict__ conv_w,
     const float* __restrict__ conv_b, const WT* __restrict__ w_i, const float* __restrict__ b_i,
     const WT* __restrict__ w_a, const float* __restrict__ b_a, const float* __restrict__ lam,
     const bf16_t* __restrict__ y, size_t ldy, ST* __restrict__ state, bf16_t* __restrict__ out, int M, int D, int W,
-    int ntiles, bool vec_io) {
+    int ntiles, bool vec_io, uint32_t* __restrict__ counters) {
     static_assert(BW % 32 == 0 && BW <= 32 * kCoreWaves, "one wave per 32 output columns of a block");
+    static_assert(NS >= 1 && (BW / NS) % 32 == 0, "whole 32-column slices per workgroup");
     constexpr int KS = BW / 16;
-    constexpr int NT = BW / 32;
+    constexpr int CW = BW / NS;       // output columns of the block that this workgroup produces
+    constexpr int NT = CW / 32;
     constexpr int kRowBytes = CoreLds<BW>::kRowBytes;
     constexpr int TPL = BW >= kWave ? BW / kWave : 1;   // weight tasks per lane and gate
     extern __shared__ __align__(16) unsigned char core_smem[];
@@ -509,9 +518,14 @@ __global__ __launch_bounds__(kCoreWaves* kWave, 1) void decode_core_kernel(
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
     const int w = __builtin_amdgcn_readfirstlane(tid / kWave);
-    const int h = (int)blockIdx.x / ntiles;
-    const int rt = (int)blockIdx.x - h * ntiles;
+    // the NS workgroups of a (rows, block) pair are neighbours in the grid: they start together
+    const int part = (int)blockIdx.x % NS;
+    const int pair = (int)blockIdx.x / NS;
+    const int h = pair / ntiles;
+    const int rt = pair - h * ntiles;
+    const int c_first = part * CW;    // first of this workgroup's output columns within the block
     const bool computes = w < NT;
+    __shared__ uint32_t s_arrival;
 
     // This wave's slice of a weight matrix: thread -> (4 input channels, 8 consecutive output
     // columns).  Sixteen lanes take sixteen consecutive channel quads of one column octet (their
@@ -525,7 +539,7 @@ __global__ __launch_bounds__(kCoreWaves* kWave, 1) void decode_core_kernel(
         for (int q = 0; q < TPL; ++q) {
             const int task = lane + q * kWave;
             const int tkq = task % KQN + KQN * (task / (4 * KQN)), tn8 = ((task / KQN) % 4) * 8;
-            if (task < BW) raw[q].load(wsel + ((size_t)h * BW + 4 * tkq) * BW + w * 32 + tn8, BW);
+            if (task < BW) raw[q].load(wsel + ((size_t)h * BW + 4 * tkq) * BW + c_first + w * 32 + tn8, BW);
             else raw[q].clear();
         }
     };
@@ -576,11 +590,13 @@ __global__ __launch_bounds__(kCoreWaves* kWave, 1) void decode_core_kernel(
 #pragma unroll
                 for (int v = 0; v < 8; ++v) acc[v] = fmaf(conv_w[(size_t)H * D + c + v], xv[v], acc[v]);
                 pack(acc, ubits);
+                if constexpr (NS == 1) {   // the only reader of these rows rolls them on the spot
 #pragma unroll
-                for (int j = 0; j < kCoreMaxW - 1; ++j) {
-                    if (j + 1 < H) *reinterpret_cast<u32x4*>(sb + (size_t)j * D) = win[j + 1];
+                    for (int j = 0; j < kCoreMaxW - 1; ++j) {
+                        if (j + 1 < H) *reinterpret_cast<u32x4*>(sb + (size_t)j * D) = win[j + 1];
+                    }
+                    if (H > 0) *reinterpret_cast<u32x4*>(sb + (size_t)(H - 1) * D) = newest;
                 }
-                if (H > 0) *reinterpret_cast<u32x4*>(sb + (size_t)(H - 1) * D) = newest;
             }
             *reinterpret_cast<u32x4*>(sU + rl * kRowBytes + ch * 16) = ubits;
         }
@@ -598,6 +614,12 @@ __global__ __launch_bounds__(kCoreWaves* kWave, 1) void decode_core_kernel(
     wave_lds_fence();
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
+    if constexpr (NS > 1) {
+        // every thread's window loads have returned (their values went to LDS before the
+        // barrier): this workgroup no longer reads the window
+        if (tid == (kCoreWaves - 1) * kWave && W > 1)   // a wave without matrix products to do
+            s_arrival = __hip_atomic_fetch_add(counters + pair, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
 
     f32x16 acc_i = {}, acc_a = {};
     if (computes) {
@@ -627,13 +649,13 @@ __global__ __launch_bounds__(kCoreWaves* kWave, 1) void decode_core_kernel(
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
     if (computes) {
-        const int c_out = h * BW + w * 32 + col;
+        const int c_out = h * BW + c_first + w * 32 + col;
         const float bias_i = b_i != nullptr ? b_i[c_out] : 0.0f;
         const float bias_a = b_a != nullptr ? b_a[c_out] : 0.0f;
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
             const int rl = 4 * (lane >> 5) + 8 * (r / 4) + (r % 4);
-            unsigned char* o = sO + rl * kORowBytes + (w * 32 + col) * 2;
+            unsigned char* o = sO + rl * kORowBytes + (c_first + w * 32 + col) * 2;
             *reinterpret_cast<uint16_t*>(o) = to_bf16_bits(acc_i[r] + bias_i);
             *reinterpret_cast<uint16_t*>(o + BW * 2) = to_bf16_bits(acc_a[r] + bias_a);
         }
@@ -645,9 +667,9 @@ __global__ __launch_bounds__(kCoreWaves* kWave, 1) void decode_core_kernel(
     // ---- 4. recurrence and output gate
     {
         typedef typename Raw<ST, 8>::type sraw8_t;
-        constexpr int CH = BW / 8;
+        constexpr int CH = CW / 8;
         for (int task = tid; task < kTileRows * CH; task += kCoreWaves * kWave) {
-            const int rl = task / CH, ch = task - rl * CH;
+            const int rl = task / CH, ch = c_first / 8 + (task - rl * CH);
             const int row = rt * kTileRows + rl;
             if (row >= M) continue;
             const int c = h * BW + ch * 8;
@@ -693,6 +715,34 @@ __global__ __launch_bounds__(kCoreWaves* kWave, 1) void decode_core_kernel(
                     *reinterpret_cast<uint16_t*>(op + v) = to_bf16_bits(go[v]);
                 }
             }
+        }
+    }
+
+    // ---- 5. the window roll, by the workgroup that counted in last (s_arrival was written
+    //         before the barriers of steps 3 and 4 and is read after them)
+    if constexpr (NS > 1) {
+        if (W > 1 && s_arrival == (uint32_t)(NS - 1)) {
+            constexpr int CH = BW / 8;
+            const int H = W - 1;
+            for (int task = tid; task < kTileRows * CH; task += kCoreWaves * kWave) {
+                const int rl = task / CH, ch = task - rl * CH;
+                const int row = rt * kTileRows + rl;
+                if (row >= M) continue;
+                const int c = h * BW + ch * 8;
+                bf16_t* sb = conv_state + (size_t)row * H * D + c;
+                u32x4 win[kCoreMaxW - 1];
+#pragma unroll
+                for (int j = 1; j < kCoreMaxW - 1; ++j) {
+                    if (j < H) win[j] = *reinterpret_cast<const u32x4*>(sb + (size_t)j * D);
+                }
+                const u32x4 newest = *reinterpret_cast<const u32x4*>(x_new + (size_t)row * ldx + c);
+#pragma unroll
+                for (int j = 0; j < kCoreMaxW - 1; ++j) {
+                    if (j + 1 < H) *reinterpret_cast<u32x4*>(sb + (size_t)j * D) = win[j + 1];
+                }
+                *reinterpret_cast<u32x4*>(sb + (size_t)(H - 1) * D) = newest;
+            }
+            if (tid == 0) __hip_atomic_store(counters + pair, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
     }
 }
@@ -1205,15 +1255,32 @@ int gate_bwd_weights_bw(const void* x, const void* dg_i, const void* dg_a, float
     }
 }
 
-template <typename WT, typename ST, int BW>
-int launch_decode_core(void* conv_state, const void* x_new, long long ldx, const float* conv_w, const float* conv_b,
-                       const void* w_i, const float* b_i, const void* w_a, const float* b_a, const float* lam,
-                       const void* y, long long ldy, void* state, void* out, int B, int D, int nb, int W,
-                       hipStream_t st) {
+// Workgroups that share a block's output columns, when the caller brought counters for them.
+// Each of them repeats the block's conv, so the cut pays only where fetching the weights is the
+// larger part, at a block width of 256 (256 KiB per block; at 128 the cut was measured slower:
+// 9.5 against 8.1 us at 256 rows), and only while the launch fits the device in one round:
+// at 256 rows and 10 blocks two workgroups per block take 14.9 us against 18.7 for one and 21.8
+// for four (320 workgroups); at 32 rows four take 10.3 against 17.6 us.
+#ifndef HAWK_CORE_MAX_GRID
+#define HAWK_CORE_MAX_GRID 256
+#endif
+constexpr int kCoreMaxGrid = HAWK_CORE_MAX_GRID;
+inline int decode_core_parts(int pairs, int bw, bool have_counters) {
+    if (!have_counters || bw < 256) return 1;
+    if ((long long)pairs * 4 <= kCoreMaxGrid) return 4;
+    if ((long long)pairs * 2 <= kCoreMaxGrid) return 2;
+    return 1;
+}
+
+template <typename WT, typename ST, int BW, int NS>
+int launch_decode_core_ns(void* conv_state, const void* x_new, long long ldx, const float* conv_w, const float* conv_b,
+                          const void* w_i, const float* b_i, const void* w_a, const float* b_a, const float* lam,
+                          const void* y, long long ldy, void* state, void* out, int B, int D, int nb, int W,
+                          uint32_t* counters, hipStream_t st) {
     const int ntiles = ceil_div(B, kTileRows);
-    const long long grid = (long long)nb * ntiles;
+    const long long grid = (long long)nb * ntiles * NS;
     if (grid > 0x7fffffffLL) return HAWK_ERR_BAD_SHAPE;
-    constexpr auto kernel = decode_core_kernel<WT, ST, BW>;
+    constexpr auto kernel = decode_core_kernel<WT, ST, BW, NS>;
     constexpr size_t smem = CoreLds<BW>::kBytes + BW * sizeof(float);   // + softplus(Lambda) of the block
     // 16-byte accesses to y, recc_state and out when their rows allow it
     const bool vec_io = (ldy % 8) == 0 && (reinterpret_cast<uintptr_t>(y) & 15u) == 0 &&
@@ -1223,19 +1290,40 @@ int launch_decode_core(void* conv_state, const void* x_new, long long ldx, const
                        static_cast<bf16_t*>(conv_state), static_cast<const bf16_t*>(x_new), (size_t)ldx, conv_w,
                        conv_b, static_cast<const WT*>(w_i), b_i, static_cast<const WT*>(w_a), b_a, lam,
                        static_cast<const bf16_t*>(y), (size_t)ldy, static_cast<ST*>(state), static_cast<bf16_t*>(out),
-                       B, D, W, ntiles, vec_io);
+                       B, D, W, ntiles, vec_io, counters);
     return hipGetLastError() == hipSuccess ? HAWK_OK : HAWK_ERR_LAUNCH;
+}
+
+template <typename WT, typename ST, int BW>
+int launch_decode_core(void* conv_state, const void* x_new, long long ldx, const float* conv_w, const float* conv_b,
+                       const void* w_i, const float* b_i, const void* w_a, const float* b_a, const float* lam,
+                       const void* y, long long ldy, void* state, void* out, int B, int D, int nb, int W,
+                       uint32_t* counters, hipStream_t st) {
+    const int parts = decode_core_parts(nb * ceil_div(B, kTileRows), BW, counters != nullptr);
+    if constexpr (BW >= 128) {
+        if (parts == 4)
+            return launch_decode_core_ns<WT, ST, BW, 4>(conv_state, x_new, ldx, conv_w, conv_b, w_i, b_i, w_a, b_a, lam, y,
+                                                        ldy, state, out, B, D, nb, W, counters, st);
+    }
+    if constexpr (BW >= 64) {
+        if (parts == 2)
+            return launch_decode_core_ns<WT, ST, BW, 2>(conv_state, x_new, ldx, conv_w, conv_b, w_i, b_i, w_a, b_a, lam, y,
+                                                        ldy, state, out, B, D, nb, W, counters, st);
+    }
+    return launch_decode_core_ns<WT, ST, BW, 1>(conv_state, x_new, ldx, conv_w, conv_b, w_i, b_i, w_a, b_a, lam, y, ldy,
+                                                state, out, B, D, nb, W, nullptr, st);
 }
 
 template <typename WT, typename ST>
 int decode_core_bw(void* conv_state, const void* x_new, long long ldx, const float* conv_w, const float* conv_b,
                    const void* w_i, const float* b_i, const void* w_a, const float* b_a, const float* lam,
-                   const void* y, long long ldy, void* state, void* out, int B, int D, int nb, int W, hipStream_t st) {
+                   const void* y, long long ldy, void* state, void* out, int B, int D, int nb, int W, uint32_t* counters,
+                   hipStream_t st) {
     switch (D / nb) {
-        case 32: return launch_decode_core<WT, ST, 32>(conv_state, x_new, ldx, conv_w, conv_b, w_i, b_i, w_a, b_a, lam, y, ldy, state, out, B, D, nb, W, st);
-        case 64: return launch_decode_core<WT, ST, 64>(conv_state, x_new, ldx, conv_w, conv_b, w_i, b_i, w_a, b_a, lam, y, ldy, state, out, B, D, nb, W, st);
-        case 128: return launch_decode_core<WT, ST, 128>(conv_state, x_new, ldx, conv_w, conv_b, w_i, b_i, w_a, b_a, lam, y, ldy, state, out, B, D, nb, W, st);
-        case 256: return launch_decode_core<WT, ST, 256>(conv_state, x_new, ldx, conv_w, conv_b, w_i, b_i, w_a, b_a, lam, y, ldy, state, out, B, D, nb, W, st);
+        case 32: return launch_decode_core<WT, ST, 32>(conv_state, x_new, ldx, conv_w, conv_b, w_i, b_i, w_a, b_a, lam, y, ldy, state, out, B, D, nb, W, counters, st);
+        case 64: return launch_decode_core<WT, ST, 64>(conv_state, x_new, ldx, conv_w, conv_b, w_i, b_i, w_a, b_a, lam, y, ldy, state, out, B, D, nb, W, counters, st);
+        case 128: return launch_decode_core<WT, ST, 128>(conv_state, x_new, ldx, conv_w, conv_b, w_i, b_i, w_a, b_a, lam, y, ldy, state, out, B, D, nb, W, counters, st);
+        case 256: return launch_decode_core<WT, ST, 256>(conv_state, x_new, ldx, conv_w, conv_b, w_i, b_i, w_a, b_a, lam, y, ldy, state, out, B, D, nb, W, counters, st);
         default: return HAWK_ERR_BAD_SHAPE;
     }
 }
@@ -1244,18 +1332,27 @@ int decode_core_bw(void* conv_state, const void* x_new, long long ldx, const flo
 
 bool gate_proj_block_width_supported(int bw) { return bw == 32 || bw == 64 || bw == 128 || bw == 256; }
 
+size_t decode_core_workspace_bytes(int B, int D, int nb) {
+    (void)D;
+    return (size_t)nb * ceil_div(B, kTileRows) * sizeof(uint32_t);
+}
+
 int decode_core_step(void* conv_state, const void* x_new, long long ldx, const float* conv_w, const float* conv_b,
                      const void* w_i, const float* b_i, const void* w_a, const float* b_a, const float* lam,
                      const void* y, long long ldy, void* state, void* out, int B, int D, int nb, int W, int w_dtype,
-                     int state_dtype, hipStream_t st) {
+                     int state_dtype, void* workspace, size_t workspace_bytes, hipStream_t st) {
+    // counters for cutting a block's columns over several workgroups, if the caller brought enough
+    uint32_t* counters = (workspace != nullptr && workspace_bytes >= decode_core_workspace_bytes(B, D, nb))
+                             ? static_cast<uint32_t*>(workspace)
+                             : nullptr;
     if (w_dtype == HAWK_DTYPE_BF16) {
         if (state_dtype == HAWK_DTYPE_BF16)
-            return decode_core_bw<bf16_t, bf16_t>(conv_state, x_new, ldx, conv_w, conv_b, w_i, b_i, w_a, b_a, lam, y, ldy, state, out, B, D, nb, W, st);
-        return decode_core_bw<bf16_t, float>(conv_state, x_new, ldx, conv_w, conv_b, w_i, b_i, w_a, b_a, lam, y, ldy, state, out, B, D, nb, W, st);
+            return decode_core_bw<bf16_t, bf16_t>(conv_state, x_new, ldx, conv_w, conv_b, w_i, b_i, w_a, b_a, lam, y, ldy, state, out, B, D, nb, W, counters, st);
+        return decode_core_bw<bf16_t, float>(conv_state, x_new, ldx, conv_w, conv_b, w_i, b_i, w_a, b_a, lam, y, ldy, state, out, B, D, nb, W, counters, st);
     }
     if (state_dtype == HAWK_DTYPE_BF16)
-        return decode_core_bw<float, bf16_t>(conv_state, x_new, ldx, conv_w, conv_b, w_i, b_i, w_a, b_a, lam, y, ldy, state, out, B, D, nb, W, st);
-    return decode_core_bw<float, float>(conv_state, x_new, ldx, conv_w, conv_b, w_i, b_i, w_a, b_a, lam, y, ldy, state, out, B, D, nb, W, st);
+        return decode_core_bw<float, bf16_t>(conv_state, x_new, ldx, conv_w, conv_b, w_i, b_i, w_a, b_a, lam, y, ldy, state, out, B, D, nb, W, counters, st);
+    return decode_core_bw<float, float>(conv_state, x_new, ldx, conv_w, conv_b, w_i, b_i, w_a, b_a, lam, y, ldy, state, out, B, D, nb, W, counters, st);
 }
 
 int gate_proj_fwd(const void* x, const void* w_i, const float* b_i, const void* w_a, const float* b_a, void* out_i,

@@ -60,7 +60,10 @@ int gate_proj_bwd_input(const void* dxg, const void* dag, const void* w_i, const
 int decode_core_step(void* conv_state, const void* x_new, long long ldx, const float* conv_w, const float* conv_b,
                      const void* w_i, const float* b_i, const void* w_a, const float* b_a, const float* lam,
                      const void* y, long long ldy, void* state, void* out, int B, int D, int nb, int W, int w_dtype,
-                     int state_dtype, hipStream_t st);
+                     int state_dtype, void* workspace, size_t workspace_bytes, hipStream_t st);
+// counters (one 32-bit word per 32 rows and block, zero between launches) that let a launch cut a
+// block's output columns over several workgroups
+size_t decode_core_workspace_bytes(int B, int D, int nb);
 size_t gate_proj_bwd_weights_workspace_bytes(int M, int D, int nb);
 int gate_proj_bwd_weights(const void* x, const void* dg_i, const void* dg_a, float* dw_i, float* db_i, float* dw_a,
                           float* db_a, int M, int D, int nb, int x_dtype, int g_dtype, void* ws, size_t ws_bytes,

@@ -307,14 +307,19 @@ def decode_core_step(conv_state, x_new, conv: "Conv1D", input_gate: "BlockDiagon
     b_a = _lib.dense16(a_gate.b.detach().float().reshape(D))
     lam = _lib.dense16(a_param.detach().float())
     out = torch.empty((B, D), dtype=torch.bfloat16, device=dev)
+    lib = _lib.load()
     with torch.cuda.device(dev):
-        status = _lib.load().hawk_decode_core_step(
+        # counters that let several workgroups share a block's output columns
+        nws = lib.hawk_decode_core_workspace_bytes(B, D, input_gate.num_blocks)
+        ws = _lib.decode_workspace(dev, nws)
+        status = lib.hawk_decode_core_step_ws(
             conv_state.data_ptr(), xn.data_ptr(), ldx, w32.data_ptr(), b32.data_ptr(), w_i.data_ptr(),
             b_i.data_ptr(), w_a.data_ptr(), b_a.data_ptr(), lam.data_ptr(), y2.data_ptr(), ldy,
             recc_state.data_ptr(), out.data_ptr(), B, D, input_gate.num_blocks, W, _lib.HAWK_DTYPE_BF16,
-            _lib.dtype_code(w_i.dtype), _lib.dtype_code(recc_state.dtype), _lib.stream_ptr(dev),
+            _lib.dtype_code(w_i.dtype), _lib.dtype_code(recc_state.dtype), ws.data_ptr(), ws.numel(),
+            _lib.stream_ptr(dev),
         )
-    _lib.check("hawk_decode_core_step", status)
+    _lib.check("hawk_decode_core_step_ws", status)
     return out.reshape(shape)
 
 

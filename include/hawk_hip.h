@@ -253,6 +253,23 @@ int hawk_decode_core_step(void* conv_state, const void* x_new, long long ldx, co
                           void* recc_state, void* out, int B, int D, int num_blocks, int W,
                           int dtype, int w_dtype, int state_dtype, void* stream);
 
+/* The same step with a workspace: hawk_decode_core_workspace_bytes(B, D, num_blocks) bytes of
+ * device memory (4-byte aligned) that hold zeros before the first call (hipMemsetAsync, or
+ * hawk_scan_workspace_init) and are left holding zeros by every call, so one buffer serves all
+ * layers and steps issued in order on one stream; concurrent streams need one each.  With it the
+ * output columns of a block are produced by up to four workgroups instead of one (a block's
+ * 2 x bw x bw weights then pass through four L1 caches, not one, and a batch of 256 rows with
+ * 10 blocks occupies 320 workgroups instead of 80); the workgroup that is last to have read a
+ * conv window rolls it.  Results are bit-identical to hawk_decode_core_step.  A NULL workspace
+ * makes the call hawk_decode_core_step.  Same upstream lines as above. */
+size_t hawk_decode_core_workspace_bytes(int B, int D, int num_blocks);
+int hawk_decode_core_step_ws(void* conv_state, const void* x_new, long long ldx, const float* conv_w,
+                             const float* conv_b, const void* w_i, const float* b_i, const void* w_a,
+                             const float* b_a, const float* a_param, const void* y, long long ldy,
+                             void* recc_state, void* out, int B, int D, int num_blocks, int W,
+                             int dtype, int w_dtype, int state_dtype, void* workspace_device,
+                             size_t workspace_bytes, void* stream);
+
 /* Both gate logits of M = B*T tokens in one pass over x:
  *   x_rg_lru[m, h*bw+j] = b_i[h*bw+j] + sum_i x[m, h*bw+i] w_i[h, i, j]     (same for a_rg_lru)
  * Replaces the two BlockDiagonalLinear calls of hawk/hawk.py:181-182 (einsum + bias,

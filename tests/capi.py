@@ -216,19 +216,31 @@ def gate_proj_fwd(x, w_i, b_i, w_a, b_a, out_dtype=None):
     return oi, oa
 
 
-def decode_core_step(conv_state, x_new, conv_w, conv_b, w_i, b_i, w_a, b_a, lam, y, state):
+def decode_core_step(conv_state, x_new, conv_w, conv_b, w_i, b_i, w_a, b_a, lam, y, state, ws=None):
     """x_new, y: [B,D] bf16 views with unit channel stride (rows may be further apart than D);
-    conv_state [B,W-1,D] bf16 and state [B,D] are updated in place.  Returns out [B,D] bf16."""
+    conv_state [B,W-1,D] bf16 and state [B,D] are updated in place.  Returns out [B,D] bf16.
+    ws: zeroed counters (uint8 tensor) for the entry point that cuts a block over workgroups."""
     B, D = x_new.shape
     W = conv_w.shape[0]
     out = torch.empty((B, D), dtype=torch.bfloat16, device="cuda")
-    rc = _lib.load().hawk_decode_core_step(
+    args = [
         _lib.ptr(conv_state), x_new.data_ptr(), x_new.stride(0) if B > 1 else D, conv_w.data_ptr(), conv_b.data_ptr(),
         w_i.data_ptr(), _lib.ptr(b_i), w_a.data_ptr(), _lib.ptr(b_a), lam.data_ptr(), y.data_ptr(),
         y.stride(0) if B > 1 else D, state.data_ptr(), out.data_ptr(), B, D, w_i.shape[0], W,
-        _lib.dtype_code(x_new.dtype), _lib.dtype_code(w_i.dtype), _lib.dtype_code(state.dtype), _stream())
-    _lib.check("hawk_decode_core_step", rc)
+        _lib.dtype_code(x_new.dtype), _lib.dtype_code(w_i.dtype), _lib.dtype_code(state.dtype)]
+    if ws is None:
+        rc = _lib.load().hawk_decode_core_step(*args, _stream())
+        _lib.check("hawk_decode_core_step", rc)
+    else:
+        rc = _lib.load().hawk_decode_core_step_ws(*args, ws.data_ptr(), ws.numel(), _stream())
+        _lib.check("hawk_decode_core_step_ws", rc)
     return out
+
+
+def decode_core_workspace(B, D, nb):
+    n = _lib.load().hawk_decode_core_workspace_bytes(B, D, nb)
+    assert n > 0
+    return torch.zeros(n, dtype=torch.uint8, device="cuda")
 
 
 def gate_proj_bwd_input(dxg, dag, w_i, w_a, dx_dtype=None, addend=None, in_place=False):

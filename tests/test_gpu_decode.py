@@ -199,3 +199,30 @@ def test_decode_core_step_with_operands_that_forbid_16_byte_accesses(state_dtype
     assert torch.equal(cs, cs_ref)
     assert torch.equal(st_off, st_ref)
     assert torch.equal(out, out_ref)
+
+
+@pytest.mark.parametrize("w_dtype,state_dtype", [("bf16", "bf16"), ("f32", "f32")])
+@pytest.mark.parametrize("B,D,nb,W", [(256, 2560, 10, 4), (1, 2560, 10, 4), (33, 512, 4, 4), (100, 256, 4, 2),
+                                      (70, 256, 2, 8), (3, 128, 2, 1), (64, 1024, 4, 4), (700, 512, 2, 4),
+                                      (40, 256, 8, 4)])
+def test_decode_core_step_with_counters_is_bit_identical_to_the_one_without(B, D, nb, W, w_dtype, state_dtype):
+    """hawk_decode_core_step_ws cuts a block's output columns over up to four workgroups (block
+    widths of 64 and more, launches small enough to gain from it); the workgroup that is last to
+    have read a conv window rolls it.  Window, state and output must equal the single-workgroup
+    launch bit for bit over consecutive tokens on one workspace, which every call must leave
+    holding zeros."""
+    wide, cs, conv_w, conv_b, w_i, b_i, w_a, b_a, lam, st = _core_operands(B, D, nb, W, w_dtype, state_dtype, B + D + W)
+    cs_ref, st_ref = cs.clone(), st.clone()
+    ws = capi.decode_core_workspace(B, D, nb)
+    rng = np.random.default_rng(11)
+    for step in range(4):
+        x_new, y = wide[:, :D], wide[:, D:]
+        out = capi.decode_core_step(cs if W > 1 else None, x_new, conv_w, conv_b, w_i, b_i, w_a, b_a, lam, y, st, ws=ws)
+        out_ref = capi.decode_core_step(cs_ref if W > 1 else None, x_new, conv_w, conv_b, w_i, b_i, w_a, b_a, lam, y,
+                                        st_ref)
+        torch.cuda.synchronize()
+        assert torch.equal(cs, cs_ref), step
+        assert torch.equal(st, st_ref), step
+        assert torch.equal(out, out_ref), step
+        assert int(ws.view(torch.int32).abs().sum()) == 0, step
+        wide = capi.to_dev(rng.standard_normal((B, 2 * D)), "bf16")
