@@ -498,13 +498,17 @@ struct CoreLds {
 // follows behind it
 __device__ __forceinline__ void wave_lds_fence() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
 
-template <typename WT, typename ST, int BW, int NS>
+// WC: the conv window's width when it is known at compile time (4, upstream's), else 0: with a
+// known width the window's loads are straight-line code, all in flight together, instead of a
+// chain of branches each waiting for its own load.
+template <typename WT, typename ST, int BW, int NS, int WC>
 __global__ __launch_bounds__(kCoreWaves* kWave, 1) void decode_core_kernel(
     bf16_t* __restrict__ conv_state, const bf16_t* __restrict__ x_new, size_t ldx, const float* __restrict__ conv_w,
     const float* __restrict__ conv_b, const WT* __restrict__ w_i, const float* __restrict__ b_i,
     const WT* __restrict__ w_a, const float* __restrict__ b_a, const float* __restrict__ lam,
-    const bf16_t* __restrict__ y, size_t ldy, ST* __restrict__ state, bf16_t* __restrict__ out, int M, int D, int W,
-    int ntiles, bool vec_io, uint32_t* __restrict__ counters) {
+    const bf16_t* __restrict__ y, size_t ldy, ST* __restrict__ state, bf16_t* __restrict__ out, int M, int D,
+    int W_runtime, int ntiles, bool vec_io, uint32_t* __restrict__ counters) {
+    const int W = WC > 0 ? WC : W_runtime;
     static_assert(BW % 32 == 0 && BW <= 32 * kCoreWaves, "one wave per 32 output columns of a block");
     static_assert(NS >= 1 && (BW / NS) % 32 == 0, "whole 32-column slices per workgroup");
     constexpr int KS = BW / 16;
@@ -569,26 +573,53 @@ __global__ __launch_bounds__(kCoreWaves* kWave, 1) void decode_core_kernel(
             u32x4 ubits = {0u, 0u, 0u, 0u};
             if (row < M) {
                 bf16_t* sb = conv_state + (size_t)row * H * D + c;
+                // every load of the task is issued before the first of them is used
                 u32x4 win[kCoreMaxW - 1];
+                f32x4 cw[kCoreMaxW][2];
 #pragma unroll
                 for (int j = 0; j < kCoreMaxW - 1; ++j) {
                     if (j < H) win[j] = *reinterpret_cast<const u32x4*>(sb + (size_t)j * D);
                 }
                 const u32x4 newest = *reinterpret_cast<const u32x4*>(x_new + (size_t)row * ldx + c);
+#pragma unroll
+                for (int j = 0; j < kCoreMaxW; ++j) {
+                    if (j <= H) {
+                        cw[j][0] = *reinterpret_cast<const f32x4*>(conv_w + (size_t)j * D + c);
+                        cw[j][1] = *reinterpret_cast<const f32x4*>(conv_w + (size_t)j * D + c + 4);
+                    }
+                }
+                const f32x4 cb0 = *reinterpret_cast<const f32x4*>(conv_b + c);
+                const f32x4 cb1 = *reinterpret_cast<const f32x4*>(conv_b + c + 4);
                 float acc[8], xv[8];
 #pragma unroll
-                for (int v = 0; v < 8; ++v) acc[v] = conv_b[c + v];
+                for (int v = 0; v < 4; ++v) {
+                    acc[v] = cb0[v];
+                    acc[4 + v] = cb1[v];
+                }
 #pragma unroll
                 for (int j = 0; j < kCoreMaxW - 1; ++j) {
                     if (j < H) {
                         unpack(win[j], xv);
 #pragma unroll
-                        for (int v = 0; v < 8; ++v) acc[v] = fmaf(conv_w[(size_t)j * D + c + v], xv[v], acc[v]);
+                        for (int v = 0; v < 8; ++v) acc[v] = fmaf(cw[j][v / 4][v % 4], xv[v], acc[v]);
                     }
                 }
                 unpack(newest, xv);
+                {
+                    f32x4 last0 = cw[0][0], last1 = cw[0][1];   // row H of the weights
 #pragma unroll
-                for (int v = 0; v < 8; ++v) acc[v] = fmaf(conv_w[(size_t)H * D + c + v], xv[v], acc[v]);
+                    for (int j = 1; j < kCoreMaxW; ++j) {
+                        if (j == H) {
+                            last0 = cw[j][0];
+                            last1 = cw[j][1];
+                        }
+                    }
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) {
+                        acc[v] = fmaf(last0[v], xv[v], acc[v]);
+                        acc[4 + v] = fmaf(last1[v], xv[4 + v], acc[4 + v]);
+                    }
+                }
                 pack(acc, ubits);
                 if constexpr (NS == 1) {   // the only reader of these rows rolls them on the spot
 #pragma unroll
@@ -1272,15 +1303,15 @@ inline int decode_core_parts(int pairs, int bw, bool have_counters) {
     return 1;
 }
 
-template <typename WT, typename ST, int BW, int NS>
-int launch_decode_core_ns(void* conv_state, const void* x_new, long long ldx, const float* conv_w, const float* conv_b,
+template <typename WT, typename ST, int BW, int NS, int WC>
+int launch_decode_core_nsw(void* conv_state, const void* x_new, long long ldx, const float* conv_w, const float* conv_b,
                           const void* w_i, const float* b_i, const void* w_a, const float* b_a, const float* lam,
                           const void* y, long long ldy, void* state, void* out, int B, int D, int nb, int W,
                           uint32_t* counters, hipStream_t st) {
     const int ntiles = ceil_div(B, kTileRows);
     const long long grid = (long long)nb * ntiles * NS;
     if (grid > 0x7fffffffLL) return HAWK_ERR_BAD_SHAPE;
-    constexpr auto kernel = decode_core_kernel<WT, ST, BW, NS>;
+    constexpr auto kernel = decode_core_kernel<WT, ST, BW, NS, WC>;
     constexpr size_t smem = CoreLds<BW>::kBytes + BW * sizeof(float);   // + softplus(Lambda) of the block
     // 16-byte accesses to y, recc_state and out when their rows allow it
     const bool vec_io = (ldy % 8) == 0 && (reinterpret_cast<uintptr_t>(y) & 15u) == 0 &&
@@ -1292,6 +1323,18 @@ int launch_decode_core_ns(void* conv_state, const void* x_new, long long ldx, co
                        static_cast<const bf16_t*>(y), (size_t)ldy, static_cast<ST*>(state), static_cast<bf16_t*>(out),
                        B, D, W, ntiles, vec_io, counters);
     return hipGetLastError() == hipSuccess ? HAWK_OK : HAWK_ERR_LAUNCH;
+}
+
+template <typename WT, typename ST, int BW, int NS>
+int launch_decode_core_ns(void* conv_state, const void* x_new, long long ldx, const float* conv_w, const float* conv_b,
+                          const void* w_i, const float* b_i, const void* w_a, const float* b_a, const float* lam,
+                          const void* y, long long ldy, void* state, void* out, int B, int D, int nb, int W,
+                          uint32_t* counters, hipStream_t st) {
+    if (W == 4)
+        return launch_decode_core_nsw<WT, ST, BW, NS, 4>(conv_state, x_new, ldx, conv_w, conv_b, w_i, b_i, w_a, b_a, lam,
+                                                         y, ldy, state, out, B, D, nb, W, counters, st);
+    return launch_decode_core_nsw<WT, ST, BW, NS, 0>(conv_state, x_new, ldx, conv_w, conv_b, w_i, b_i, w_a, b_a, lam, y,
+                                                     ldy, state, out, B, D, nb, W, counters, st);
 }
 
 template <typename WT, typename ST, int BW>
