@@ -12,10 +12,12 @@ D=4096; ``--workload scan_conv`` adds the temporal conv1d forward and backward;
 y being one half of a [B, T, 2D] projection), 12 + 20 bytes per element;
 ``--workload gates`` runs the fused block-diagonal gate projections (matrix-core kernels:
 forward, input gradient, weight gradients) on 32768 tokens, D = 2560, 10 blocks, bf16;
-``--workload block`` chains the whole recurrent core of one layer at B=8, T=4096, D=2560 (conv,
-both gate projections, scan fused with the output gate, and the backward of all of them)
-through the C ABI, seven launches that move 31 activation-sized tensors (plus two casts of the
-fp32 gate weights to bf16, as the Python host does at this size);
+``--workload block`` chains the whole recurrent core of one layer at B=8, T=4096, D=2560 (conv and
+both gate projections in one kernel, scan fused with the output gate, and the backward of all of
+them) through the C ABI on the [B,T,2D] output of the block's input projection in place, six
+launches that move 30 activation-sized tensors (plus two casts of the fp32 gate weights to bf16,
+as the Python host does at this size); ``--unfused-conv`` runs the conv as a launch of its own on
+a copy of the x half, seven launches and 31 tensors;
 ``--workload model`` runs full training steps (forward, backward, AdamW) of the upstream
 README model (vocabulary 32000, hidden = recurrent = 512, MLP 1024, 8 layers, 16 gate blocks)
 on a 1 x 2048 batch under bf16 autocast, with and without the fused gate / epilogue kernels;
@@ -282,6 +284,7 @@ def run_block(args, lib, dev):
     e = lambda: torch.empty(B, T, D, device=dev, dtype=bf)  # noqa: E731
     u, xg, ag, h, out = e(), e(), e(), e(), e()
     du, dxg, dag, dy, dxin = e(), e(), e(), e(), e()
+    dxy = torch.empty(B, T, 2 * D, device=dev, dtype=bf)   # gradient of xy, both halves written in place
     dlam = torch.empty(D, device=dev)
     dwi, dwa, dbi, dba = torch.empty_like(wi), torch.empty_like(wa), torch.empty_like(bi), torch.empty_like(ba)
     dcw, dcb = torch.empty_like(cw), torch.empty_like(cb)
@@ -294,27 +297,39 @@ def run_block(args, lib, dev):
     wi16, wa16 = torch.empty_like(wi, dtype=bf), torch.empty_like(wa, dtype=bf)
 
     def fwd():
-        _lib.check("conv_fwd", lib.hawk_conv1d_fwd(p(xin), p(cw), p(cb), None, p(u), B, T, D, W, code, code, st))
         # as the Python host does from 8192 rows on: the fp32 gate weights are rounded to bf16 once
         # per step (two small kernels, inside the timed region) instead of by every workgroup
         wi16.copy_(wi)
         wa16.copy_(wa)
-        _lib.check("gate_fwd", lib.hawk_gate_proj_fwd(p(u), p(wi16), p(bi), p(wa16), p(ba), p(xg), p(ag), M, D, nb,
-                                                      code, code, code, st))
+        if args.unfused_conv:
+            _lib.check("conv_fwd", lib.hawk_conv1d_fwd(p(xin), p(cw), p(cb), None, p(u), B, T, D, W, code, code, st))
+            _lib.check("gate_fwd", lib.hawk_gate_proj_fwd(p(u), p(wi16), p(bi), p(wa16), p(ba), p(xg), p(ag), M, D,
+                                                          nb, code, code, code, st))
+        else:
+            # conv and both projections in one kernel, reading the x half of xy in place
+            _lib.check("conv_gate_fwd", lib.hawk_conv_gate_proj_fwd(
+                p(xy), 2 * D, p(cw), p(cb), p(wi16), p(bi), p(wa16), p(ba), p(u), p(xg), p(ag), B, T, D, nb, W,
+                code, st))
         _lib.check("scan_gated_fwd", lib.hawk_rglru_scan_gated_fwd(
             p(u), p(xg), p(ag), p(lam), p(y), 2 * D, p(h), p(out), None, B, T, D, code, code, p(ws), ws.numel(), st))
 
     def bwd():
+        inplace = not args.unfused_conv
         _lib.check("scan_gated_bwd", lib.hawk_rglru_scan_gated_bwd(
-            p(u), p(xg), p(ag), p(lam), p(y), 2 * D, p(h), p(gout), p(du), p(dxg), p(dag), p(dy), D, p(dlam),
+            p(u), p(xg), p(ag), p(lam), p(y), 2 * D, p(h), p(gout), p(du), p(dxg), p(dag),
+            p(dxy) + 2 * D if inplace else p(dy), 2 * D if inplace else D, p(dlam),
             B, T, D, code, code, p(ws), ws.numel(), st))
         # the projections' input gradient accumulates onto the scan's, in place
         _lib.check("gate_bwd_input", lib.hawk_gate_proj_bwd_input(p(dxg), p(dag), p(wi16), p(wa16), p(du), p(du), M,
                                                                   D, nb, code, code, code, st))
         _lib.check("gate_bwd_weights", lib.hawk_gate_proj_bwd_weights(
             p(u), p(dxg), p(dag), p(dwi), p(dbi), p(dwa), p(dba), M, D, nb, code, code, p(gws), gws.numel(), st))
-        _lib.check("conv_bwd", lib.hawk_conv1d_bwd(p(du), p(xin), p(cw), p(dxin), p(dcw), p(dcb), B, T, D, W, code,
-                                                   code, p(cws), cws.numel(), st))
+        if inplace:
+            _lib.check("conv_bwd", lib.hawk_conv1d_bwd_strided(p(du), p(xy), 2 * D, p(cw), p(dxy), 2 * D, p(dcw),
+                                                               p(dcb), B, T, D, W, code, code, p(cws), cws.numel(), st))
+        else:
+            _lib.check("conv_bwd", lib.hawk_conv1d_bwd(p(du), p(xin), p(cw), p(dxin), p(dcw), p(dcb), B, T, D, W,
+                                                       code, code, p(cws), cws.numel(), st))
 
     for _ in range(args.settle_steps + args.warmup):
         fwd(), bwd()
@@ -331,12 +346,13 @@ def run_block(args, lib, dev):
     wall = time.perf_counter() - t0
     flag = ctypes.c_int(0)
     _lib.check("status", lib.hawk_scan_workspace_status(ws.data_ptr(), st, ctypes.byref(flag)))
-    assert flag.value == 0 and bool(torch.isfinite(dxin.float()).all())
+    assert flag.value == 0 and bool(torch.isfinite((dxin if args.unfused_conv else dxy).float()).all())
     fwd_ms = float(np.mean([e_[0].elapsed_time(e_[1]) for e_ in ev]))
     bwd_ms = float(np.mean([e_[1].elapsed_time(e_[2]) for e_ in ev]))
     ms_per_step = wall * 1e3 / args.steps
-    # tensors moved: conv 2, gates 3, gated scan 6 | gated scan 10, gate dx 4, gate dw 3, conv 3
-    fwd_bytes, bwd_bytes = 11 * 2 * N, 20 * 2 * N
+    # tensors moved: conv 2, gates 3 (conv + gates in one kernel: 4), gated scan 6 | gated scan 10,
+    # gate dx 4, gate dw 3, conv 3
+    fwd_bytes, bwd_bytes = (11 if args.unfused_conv else 10) * 2 * N, 20 * 2 * N
     step_gbs = (fwd_bytes + bwd_bytes) / (ms_per_step * 1e-3) / 1e9
     print(json.dumps({
         "metric": "Hawk recurrent core (conv, gate projections, gated scan) fwd+bwd tokens/s, 1 GPU",
@@ -424,6 +440,7 @@ def run_model(args, lib, dev):
         return (time.perf_counter() - t0) * 1e3 / args.steps, float(static_loss.detach())
 
     fused_ms, fused_loss = time_steps()
+    nodes_ms, nodes_loss = time_steps(fused_block_core=False)
     plain_ms, plain_loss = time_steps(fused_gates=False, fused_epilogue=False)
     graph_ms, graph_loss = time_graph_steps()
     print(json.dumps({
@@ -434,10 +451,12 @@ def run_model(args, lib, dev):
         "data": f"synthetic, seed {args.seed}: random-init weights, token ids uniform in [1, {vocab})",
         "config": {"workload": "model: README Hawk (V=32000, H=R=512, I=1024, L=8, 16 blocks, conv 4), "
                                "forward + backward + AdamW, eager launches", "B": B, "T": T},
+        "ms_per_step_with_conv_and_core_as_separate_nodes": nodes_ms,
         "ms_per_step_without_fused_gates_and_epilogue": plain_ms,
         "ms_per_step_as_hip_graph": graph_ms,
         "tokens_per_s_as_hip_graph": B * T / (graph_ms * 1e-3),
-        "loss_after_last_step": {"fused": fused_loss, "unfused": plain_loss, "hip_graph": graph_loss},
+        "loss_after_last_step": {"fused": fused_loss, "separate_nodes": nodes_loss, "unfused": plain_loss,
+                                 "hip_graph": graph_loss},
         "roofline": None,
     }))
 
@@ -757,6 +776,10 @@ def main():
     ap.add_argument("--settle-steps", type=int, default=100,
                     help="further untimed steps run before the warm-up in the kernel workloads (scan*, long, gates, "
                          "block): kernel durations settle about 50 steps (20 ms) after the GPU leaves idle")
+    ap.add_argument("--unfused-conv", action="store_true",
+                    help="workload block: conv and gate projections as two launches on a copy of the x half of the "
+                         "input projection, gradients into separate tensors, instead of one launch on the "
+                         "projection's output in place and one gradient tensor")
     ap.add_argument("--workload", choices=sorted(WORKLOADS) + ["block", "decode", "gates", "model"], default="scan")
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--no-cpu-baseline", action="store_true")

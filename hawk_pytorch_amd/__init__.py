@@ -21,6 +21,7 @@ from .scan_fused import (
     GatedDiagonalRecurrence,
     fused_linear_scan,
     fused_linear_scan_gated,
+    recurrent_block_core,
     recurrent_core,
     sequential_scan_backward,
     sequential_scan_forward,
@@ -43,6 +44,7 @@ __all__ = [
     "decode_core_step",
     "fused_linear_scan",
     "gate_projections",
+    "recurrent_block_core",
     "recurrent_core",
     "release_workspaces",
     "fused_linear_scan_gated",

@@ -56,6 +56,14 @@ SIGNATURES = {
     "hawk_conv1d_fwd": (_c_int, [_c_void_p] * 5 + [_c_int] * 6 + [_c_void_p]),
     "hawk_conv1d_bwd_workspace_bytes": (_c_size_t, [_c_int] * 4),
     "hawk_conv1d_bwd": (_c_int, [_c_void_p] * 6 + [_c_int] * 6 + [_c_void_p, _c_size_t, _c_void_p]),
+    "hawk_conv1d_fwd_strided": (
+        _c_int, [_c_void_p, ctypes.c_longlong] + [_c_void_p] * 4 + [ctypes.c_longlong] + [_c_int] * 6 + [_c_void_p]
+    ),
+    "hawk_conv1d_bwd_strided": (
+        _c_int,
+        [_c_void_p] * 2 + [ctypes.c_longlong] + [_c_void_p] * 2 + [ctypes.c_longlong] + [_c_void_p] * 2
+        + [_c_int] * 6 + [_c_void_p, _c_size_t, _c_void_p],
+    ),
     "hawk_conv1d_step": (_c_int, [_c_void_p] * 5 + [_c_int] * 5 + [_c_void_p]),
     "hawk_rglru_step": (_c_int, [_c_void_p] * 6 + [_c_int] * 4 + [_c_void_p]),
     "hawk_gate_proj_supported": (_c_int, [_c_int, _c_int]),
@@ -72,6 +80,9 @@ SIGNATURES = {
         + [_c_int] * 7 + [_c_void_p, _c_size_t, _c_void_p],
     ),
     "hawk_gate_proj_fwd": (_c_int, [_c_void_p] * 7 + [_c_int] * 6 + [_c_void_p]),
+    "hawk_conv_gate_proj_fwd": (
+        _c_int, [_c_void_p, ctypes.c_longlong] + [_c_void_p] * 9 + [_c_int] * 6 + [_c_void_p]
+    ),
     "hawk_gate_proj_bwd_input": (_c_int, [_c_void_p] * 6 + [_c_int] * 6 + [_c_void_p]),
     "hawk_gate_proj_bwd_weights_workspace_bytes": (_c_size_t, [_c_int] * 3),
     "hawk_gate_proj_bwd_weights": (_c_int, [_c_void_p] * 7 + [_c_int] * 5 + [_c_void_p, _c_size_t, _c_void_p]),

@@ -165,14 +165,23 @@ int hawk_rglru_scan_gated_bwd(const void* x, const void* x_rg_lru, const void* a
                                 as_stream(stream));
 }
 
-int hawk_conv1d_fwd(const void* x, const float* w, const float* bias, const void* state, void* y, int B, int T,
-                    int D, int W, int x_dtype, int y_dtype, void* stream) {
+int hawk_conv1d_fwd_strided(const void* x, long long x_row_stride, const float* w, const float* bias,
+                            const void* state, void* y, long long y_row_stride, int B, int T, int D, int W,
+                            int x_dtype, int y_dtype, void* stream) {
     if (!x || !w || !bias || !y) return HAWK_ERR_NULL_POINTER;
     if (!dtype_ok(x_dtype) || !dtype_ok(y_dtype)) return HAWK_ERR_BAD_DTYPE;
     if (B < 1 || T < 1 || D < 1 || W < 1 || W > 8 || B > kMaxGridY) return HAWK_ERR_BAD_SHAPE;
     if (W != 4 && T > kMaxGridY) return HAWK_ERR_BAD_SHAPE;
+    if (x_row_stride < D || y_row_stride < D || x_row_stride > kMaxRowStride || y_row_stride > kMaxRowStride)
+        return HAWK_ERR_BAD_SHAPE;
     if (!aligned16(x) || !aligned16(y) || (state && !aligned16(state))) return HAWK_ERR_ALIGNMENT;
-    return hawk::conv1d_fwd(x, w, bias, state, y, B, T, D, W, x_dtype, y_dtype, as_stream(stream));
+    return hawk::conv1d_fwd(x, x_row_stride, w, bias, state, y, y_row_stride, B, T, D, W, x_dtype, y_dtype,
+                            as_stream(stream));
+}
+
+int hawk_conv1d_fwd(const void* x, const float* w, const float* bias, const void* state, void* y, int B, int T,
+                    int D, int W, int x_dtype, int y_dtype, void* stream) {
+    return hawk_conv1d_fwd_strided(x, D, w, bias, state, y, D, B, T, D, W, x_dtype, y_dtype, stream);
 }
 
 size_t hawk_conv1d_bwd_workspace_bytes(int B, int T, int D, int W) {
@@ -180,16 +189,25 @@ size_t hawk_conv1d_bwd_workspace_bytes(int B, int T, int D, int W) {
     return hawk::conv1d_bwd_workspace_bytes(B, T, D, W);
 }
 
-int hawk_conv1d_bwd(const void* grad_y, const void* x, const float* w, void* dx, float* dw, float* db, int B, int T,
-                    int D, int W, int x_dtype, int gy_dtype, void* workspace_device, size_t workspace_bytes,
-                    void* stream) {
+int hawk_conv1d_bwd_strided(const void* grad_y, const void* x, long long x_row_stride, const float* w, void* dx,
+                            long long dx_row_stride, float* dw, float* db, int B, int T, int D, int W, int x_dtype,
+                            int gy_dtype, void* workspace_device, size_t workspace_bytes, void* stream) {
     if (!grad_y || !x || !w || !dx || !dw || !db) return HAWK_ERR_NULL_POINTER;
     if (!dtype_ok(x_dtype) || !dtype_ok(gy_dtype)) return HAWK_ERR_BAD_DTYPE;
     if (B < 1 || T < 1 || D < 1 || W < 1 || W > 8 || B > kMaxGridY) return HAWK_ERR_BAD_SHAPE;
+    if (x_row_stride < D || dx_row_stride < D || x_row_stride > kMaxRowStride || dx_row_stride > kMaxRowStride)
+        return HAWK_ERR_BAD_SHAPE;
     if (!aligned16(grad_y) || !aligned16(x) || !aligned16(dx)) return HAWK_ERR_ALIGNMENT;
     if (workspace_device == nullptr) return HAWK_ERR_WORKSPACE;
-    return hawk::conv1d_bwd(grad_y, x, w, dx, dw, db, B, T, D, W, x_dtype, gy_dtype, workspace_device,
-                            workspace_bytes, as_stream(stream));
+    return hawk::conv1d_bwd(grad_y, x, x_row_stride, w, dx, dx_row_stride, dw, db, B, T, D, W, x_dtype, gy_dtype,
+                            workspace_device, workspace_bytes, as_stream(stream));
+}
+
+int hawk_conv1d_bwd(const void* grad_y, const void* x, const float* w, void* dx, float* dw, float* db, int B, int T,
+                    int D, int W, int x_dtype, int gy_dtype, void* workspace_device, size_t workspace_bytes,
+                    void* stream) {
+    return hawk_conv1d_bwd_strided(grad_y, x, D, w, dx, D, dw, db, B, T, D, W, x_dtype, gy_dtype, workspace_device,
+                                   workspace_bytes, stream);
 }
 
 int hawk_conv1d_step(void* conv_state, const void* x_new, const float* w, const float* bias, void* y, int B, int D,
@@ -282,6 +300,23 @@ int hawk_gate_proj_fwd(const void* x, const void* w_i, const float* b_i, const v
         return HAWK_ERR_ALIGNMENT;
     return hawk::gate_proj_fwd(x, w_i, b_i, w_a, b_a, x_rg_lru, a_rg_lru, M, D, num_blocks, x_dtype, w_dtype,
                                out_dtype, as_stream(stream));
+}
+
+int hawk_conv_gate_proj_fwd(const void* x, long long x_row_stride, const float* conv_w, const float* conv_b,
+                            const void* w_i, const float* b_i, const void* w_a, const float* b_a, void* u,
+                            void* x_rg_lru, void* a_rg_lru, int B, int T, int D, int num_blocks, int temporal_width,
+                            int w_dtype, void* stream) {
+    if (!x || !conv_w || !conv_b || !w_i || !w_a || !u || !x_rg_lru || !a_rg_lru) return HAWK_ERR_NULL_POINTER;
+    if (!dtype_ok(w_dtype)) return HAWK_ERR_BAD_DTYPE;
+    // one wrap of the position per 32-row tile, 32-bit byte offsets over a tile and its history
+    if (B < 1 || T < 32 || temporal_width != 4 || !hawk_gate_proj_supported(D, num_blocks) ||
+        (long long)B * T > 0x7fffffffLL || x_row_stride < D || x_row_stride > kMaxRowStride || x_row_stride % 8 != 0)
+        return HAWK_ERR_BAD_SHAPE;
+    if (!aligned16(x) || !aligned16(u) || !aligned16(x_rg_lru) || !aligned16(a_rg_lru) || !aligned16(w_i) ||
+        !aligned16(w_a))
+        return HAWK_ERR_ALIGNMENT;
+    return hawk::conv_gate_proj_fwd(x, x_row_stride, conv_w, conv_b, w_i, b_i, w_a, b_a, u, x_rg_lru, a_rg_lru, B, T,
+                                    D, num_blocks, w_dtype, as_stream(stream));
 }
 
 int hawk_gate_proj_bwd_input(const void* d_x_rg_lru, const void* d_a_rg_lru, const void* w_i, const void* w_a,

@@ -28,7 +28,7 @@ inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 template <typename XT, typename YT, int V, int W, int RT>
 __global__ __launch_bounds__(kConvWaves * kWave) void conv1d_fwd_kernel(
     const XT* __restrict__ x, const float* __restrict__ w, const float* __restrict__ bias,
-    const XT* __restrict__ state, YT* __restrict__ y, int T, int D, int nct) {
+    const XT* __restrict__ state, YT* __restrict__ y, int T, int D, int nct, size_t ldx, size_t ldy) {
     typedef typename Raw<XT, V>::type xraw_t;
     typedef typename Raw<YT, V>::type yraw_t;
     constexpr int H = W - 1;
@@ -42,13 +42,13 @@ __global__ __launch_bounds__(kConvWaves * kWave) void conv1d_fwd_kernel(
     const int t0 = (rg * kConvWaves + wv) * RT;
     if (c0 >= D || t0 >= T) return;
 
-    const XT* xb = x + (size_t)b * T * D + c0;
+    const XT* xb = x + (size_t)b * T * ldx + c0;
     xraw_t raw[RT + H];
 #pragma unroll
     for (int j = 0; j < RT + H; ++j) {
         const int t = t0 - H + j;
         if (t >= 0) {
-            raw[j] = (t < T) ? load_raw<XT, V>(xb + (size_t)t * D) : raw_zero<xraw_t>();
+            raw[j] = (t < T) ? load_raw<XT, V>(xb + (size_t)t * ldx) : raw_zero<xraw_t>();
         } else if (state != nullptr) {
             raw[j] = load_raw<XT, V>(state + ((size_t)b * H + (H + t)) * D + c0);
         } else {
@@ -66,7 +66,7 @@ __global__ __launch_bounds__(kConvWaves * kWave) void conv1d_fwd_kernel(
 #pragma unroll
     for (int k = 0; k < H; ++k) unpack(raw[k], win[k]);
 
-    YT* yb = y + (size_t)b * T * D + c0;
+    YT* yb = y + (size_t)b * T * ldy + c0;
 #pragma unroll
     for (int j = 0; j < RT; ++j) {
         unpack(raw[H + j], win[H]);
@@ -81,7 +81,7 @@ __global__ __launch_bounds__(kConvWaves * kWave) void conv1d_fwd_kernel(
         if (t0 + j < T) {
             yraw_t r;
             pack(out, r);
-            store_raw<YT, V>(yb + (size_t)(t0 + j) * D, r);
+            store_raw<YT, V>(yb + (size_t)(t0 + j) * ldy, r);
         }
 #pragma unroll
         for (int k = 0; k < H; ++k) {
@@ -96,7 +96,7 @@ __global__ __launch_bounds__(kConvWaves * kWave) void conv1d_fwd_kernel(
 template <typename XT, typename YT, int V>
 __global__ __launch_bounds__(256) void conv1d_fwd_anyw_kernel(
     const XT* __restrict__ x, const float* __restrict__ w, const float* __restrict__ bias,
-    const XT* __restrict__ state, YT* __restrict__ y, int T, int D, int W, int nvec) {
+    const XT* __restrict__ state, YT* __restrict__ y, int T, int D, int W, int nvec, size_t ldx, size_t ldy) {
     typedef typename Raw<YT, V>::type yraw_t;
     const int vc = blockIdx.x * blockDim.x + threadIdx.x;
     const int t = blockIdx.y;
@@ -111,7 +111,7 @@ __global__ __launch_bounds__(256) void conv1d_fwd_anyw_kernel(
         const int tt = t - s;
         float xv[V];
         if (tt >= 0) {
-            unpack(load_raw<XT, V>(x + ((size_t)b * T + tt) * D + c0), xv);
+            unpack(load_raw<XT, V>(x + ((size_t)b * T + tt) * ldx + c0), xv);
         } else if (state != nullptr) {
             unpack(load_raw<XT, V>(state + ((size_t)b * H + (H + tt)) * D + c0), xv);
         } else {
@@ -122,7 +122,7 @@ __global__ __launch_bounds__(256) void conv1d_fwd_anyw_kernel(
     }
     yraw_t r;
     pack(acc, r);
-    store_raw<YT, V>(y + ((size_t)b * T + t) * D + c0, r);
+    store_raw<YT, V>(y + ((size_t)b * T + t) * ldy + c0, r);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -134,7 +134,7 @@ __global__ __launch_bounds__(256) void conv1d_fwd_anyw_kernel(
 template <typename XT, typename GT, int V, int W, int RT>
 __global__ __launch_bounds__(kConvWaves * kWave) void conv1d_bwd_kernel(
     const GT* __restrict__ gy, const XT* __restrict__ x, const float* __restrict__ w,
-    XT* __restrict__ dx, float* __restrict__ part, int T, int D, int nct, int chunks) {
+    XT* __restrict__ dx, float* __restrict__ part, int T, int D, int nct, int chunks, size_t ldx, size_t lddx) {
     typedef typename Raw<XT, V>::type xraw_t;
     typedef typename Raw<GT, V>::type graw_t;
     constexpr int H = W - 1;
@@ -166,8 +166,8 @@ __global__ __launch_bounds__(kConvWaves * kWave) void conv1d_bwd_kernel(
     }
 
     const GT* gb = gy + (size_t)b * T * D + c0;
-    const XT* xb = x + (size_t)b * T * D + c0;
-    XT* dxb = dx + (size_t)b * T * D + c0;
+    const XT* xb = x + (size_t)b * T * ldx + c0;
+    XT* dxb = dx + (size_t)b * T * lddx + c0;
 
     for (int ch = 0; ch < chunks; ++ch) {
         const int t0 = ((rg * kConvWaves + wv) * chunks + ch) * RT;
@@ -179,7 +179,7 @@ __global__ __launch_bounds__(kConvWaves * kWave) void conv1d_bwd_kernel(
             const int tg = t0 + j;
             graw[j] = (tg < T) ? load_raw<GT, V>(gb + (size_t)tg * D) : raw_zero<graw_t>();
             const int tx = t0 - H + j;
-            xraw[j] = (tx >= 0 && tx < T) ? load_raw<XT, V>(xb + (size_t)tx * D) : raw_zero<xraw_t>();
+            xraw[j] = (tx >= 0 && tx < T) ? load_raw<XT, V>(xb + (size_t)tx * ldx) : raw_zero<xraw_t>();
         }
         float gwin[W][V], xwin[W][V];
 #pragma unroll
@@ -207,7 +207,7 @@ __global__ __launch_bounds__(kConvWaves * kWave) void conv1d_bwd_kernel(
             if (t0 + j < T) {
                 xraw_t r;
                 pack(out, r);
-                store_raw<XT, V>(dxb + (size_t)(t0 + j) * D, r);
+                store_raw<XT, V>(dxb + (size_t)(t0 + j) * lddx, r);
             }
 #pragma unroll
             for (int k = 0; k < H; ++k) {
@@ -246,7 +246,7 @@ __global__ __launch_bounds__(kConvWaves * kWave) void conv1d_bwd_kernel(
 template <typename XT, typename GT>
 __global__ __launch_bounds__(256) void conv1d_bwd_anyw_kernel(
     const GT* __restrict__ gy, const XT* __restrict__ x, const float* __restrict__ w,
-    XT* __restrict__ dx, float* __restrict__ part, int T, int D, int W, int rows_per_group) {
+    XT* __restrict__ dx, float* __restrict__ part, int T, int D, int W, int rows_per_group, size_t ldx, size_t lddx) {
     const int c = blockIdx.x * blockDim.x + threadIdx.x;
     const int rg = blockIdx.y;
     const int b = blockIdx.z;
@@ -270,7 +270,7 @@ __global__ __launch_bounds__(256) void conv1d_bwd_anyw_kernel(
                 }
                 if (t - s >= 0) {
                     float xv[1];
-                    unpack(load_raw<XT, 1>(x + ((size_t)b * T + t - s) * D + c), xv);
+                    unpack(load_raw<XT, 1>(x + ((size_t)b * T + t - s) * ldx + c), xv);
                     dwk[s] = fmaf(g0[0], xv[0], dwk[s]);  // slot s holds dw[W-1-s]
                 }
             }
@@ -279,7 +279,7 @@ __global__ __launch_bounds__(256) void conv1d_bwd_anyw_kernel(
         float o[1] = {acc};
         typename Raw<XT, 1>::type r;
         pack(o, r);
-        store_raw<XT, 1>(dx + ((size_t)b * T + t) * D + c, r);
+        store_raw<XT, 1>(dx + ((size_t)b * T + t) * lddx + c, r);
     }
     float* prow = part + ((size_t)rg * gridDim.z + b) * (size_t)(W + 1) * D;
 #pragma unroll
@@ -322,9 +322,10 @@ __global__ __launch_bounds__(1024) void colsum_kernel(const float* __restrict__ 
     }
 }
 
-int pick_v4(int D) {
-    if (D % 4 == 0) return 4;
-    if (D % 2 == 0) return 2;
+// Channels per lane: every row of every tensor must start on a multiple of it.
+int pick_v4(int D, size_t ld_a, size_t ld_b) {
+    if (D % 4 == 0 && ld_a % 4 == 0 && ld_b % 4 == 0) return 4;
+    if (D % 2 == 0 && ld_a % 2 == 0 && ld_b % 2 == 0) return 2;
     return 1;
 }
 
@@ -336,24 +337,24 @@ int bwd_rows_per_group(int T) {
 
 template <typename XT, typename YT>
 int fwd_dispatch(const void* x, const float* w, const float* bias, const void* state, void* y, int B, int T, int D,
-                 int W, hipStream_t st) {
+                 int W, size_t ldx, size_t ldy, hipStream_t st) {
     const XT* xp = static_cast<const XT*>(x);
     const XT* sp = static_cast<const XT*>(state);
     YT* yp = static_cast<YT*>(y);
-    const int V = pick_v4(D);
+    const int V = pick_v4(D, ldx, ldy);
     if (W == 4) {
         const int nct = ceil_div(D, kWave * V);
         const int nrg = ceil_div(T, kConvWaves * kConvRT);
         const dim3 grid((unsigned)(nct * nrg), (unsigned)B), block(kConvWaves * kWave);
-        if (V == 4) hipLaunchKernelGGL((conv1d_fwd_kernel<XT, YT, 4, 4, kConvRT>), grid, block, 0, st, xp, w, bias, sp, yp, T, D, nct);
-        else if (V == 2) hipLaunchKernelGGL((conv1d_fwd_kernel<XT, YT, 2, 4, kConvRT>), grid, block, 0, st, xp, w, bias, sp, yp, T, D, nct);
-        else hipLaunchKernelGGL((conv1d_fwd_kernel<XT, YT, 1, 4, kConvRT>), grid, block, 0, st, xp, w, bias, sp, yp, T, D, nct);
+        if (V == 4) hipLaunchKernelGGL((conv1d_fwd_kernel<XT, YT, 4, 4, kConvRT>), grid, block, 0, st, xp, w, bias, sp, yp, T, D, nct, ldx, ldy);
+        else if (V == 2) hipLaunchKernelGGL((conv1d_fwd_kernel<XT, YT, 2, 4, kConvRT>), grid, block, 0, st, xp, w, bias, sp, yp, T, D, nct, ldx, ldy);
+        else hipLaunchKernelGGL((conv1d_fwd_kernel<XT, YT, 1, 4, kConvRT>), grid, block, 0, st, xp, w, bias, sp, yp, T, D, nct, ldx, ldy);
     } else {
         const int nvec = D / V;
         const dim3 grid((unsigned)ceil_div(nvec, 256), (unsigned)T, (unsigned)B), block(256);
-        if (V == 4) hipLaunchKernelGGL((conv1d_fwd_anyw_kernel<XT, YT, 4>), grid, block, 0, st, xp, w, bias, sp, yp, T, D, W, nvec);
-        else if (V == 2) hipLaunchKernelGGL((conv1d_fwd_anyw_kernel<XT, YT, 2>), grid, block, 0, st, xp, w, bias, sp, yp, T, D, W, nvec);
-        else hipLaunchKernelGGL((conv1d_fwd_anyw_kernel<XT, YT, 1>), grid, block, 0, st, xp, w, bias, sp, yp, T, D, W, nvec);
+        if (V == 4) hipLaunchKernelGGL((conv1d_fwd_anyw_kernel<XT, YT, 4>), grid, block, 0, st, xp, w, bias, sp, yp, T, D, W, nvec, ldx, ldy);
+        else if (V == 2) hipLaunchKernelGGL((conv1d_fwd_anyw_kernel<XT, YT, 2>), grid, block, 0, st, xp, w, bias, sp, yp, T, D, W, nvec, ldx, ldy);
+        else hipLaunchKernelGGL((conv1d_fwd_anyw_kernel<XT, YT, 1>), grid, block, 0, st, xp, w, bias, sp, yp, T, D, W, nvec, ldx, ldy);
     }
     return hipGetLastError() == hipSuccess ? HAWK_OK : HAWK_ERR_LAUNCH;
 }
@@ -376,21 +377,21 @@ BwdPlan bwd_plan(int T, int W) {
 
 template <typename XT, typename GT>
 int bwd_dispatch(const void* gy, const void* x, const float* w, void* dx, float* dw, float* db, int B, int T, int D,
-                 int W, float* part, hipStream_t st) {
+                 int W, size_t ldx, size_t lddx, float* part, hipStream_t st) {
     const GT* gp = static_cast<const GT*>(gy);
     const XT* xp = static_cast<const XT*>(x);
     XT* dxp = static_cast<XT*>(dx);
     const BwdPlan p = bwd_plan(T, W);
     if (W == 4) {
-        const int V = pick_v4(D);
+        const int V = pick_v4(D, ldx, lddx);
         const int nct = ceil_div(D, kWave * V);
         const dim3 grid((unsigned)(nct * p.ngroups), (unsigned)B), block(kConvWaves * kWave);
-        if (V == 4) hipLaunchKernelGGL((conv1d_bwd_kernel<XT, GT, 4, 4, kConvRT>), grid, block, 0, st, gp, xp, w, dxp, part, T, D, nct, p.chunks);
-        else if (V == 2) hipLaunchKernelGGL((conv1d_bwd_kernel<XT, GT, 2, 4, kConvRT>), grid, block, 0, st, gp, xp, w, dxp, part, T, D, nct, p.chunks);
-        else hipLaunchKernelGGL((conv1d_bwd_kernel<XT, GT, 1, 4, kConvRT>), grid, block, 0, st, gp, xp, w, dxp, part, T, D, nct, p.chunks);
+        if (V == 4) hipLaunchKernelGGL((conv1d_bwd_kernel<XT, GT, 4, 4, kConvRT>), grid, block, 0, st, gp, xp, w, dxp, part, T, D, nct, p.chunks, ldx, lddx);
+        else if (V == 2) hipLaunchKernelGGL((conv1d_bwd_kernel<XT, GT, 2, 4, kConvRT>), grid, block, 0, st, gp, xp, w, dxp, part, T, D, nct, p.chunks, ldx, lddx);
+        else hipLaunchKernelGGL((conv1d_bwd_kernel<XT, GT, 1, 4, kConvRT>), grid, block, 0, st, gp, xp, w, dxp, part, T, D, nct, p.chunks, ldx, lddx);
     } else {
         const dim3 grid((unsigned)ceil_div(D, 256), (unsigned)p.ngroups, (unsigned)B), block(256);
-        hipLaunchKernelGGL((conv1d_bwd_anyw_kernel<XT, GT>), grid, block, 0, st, gp, xp, w, dxp, part, T, D, W, p.rows_per_group);
+        hipLaunchKernelGGL((conv1d_bwd_anyw_kernel<XT, GT>), grid, block, 0, st, gp, xp, w, dxp, part, T, D, W, p.rows_per_group, ldx, lddx);
     }
     if (hipGetLastError() != hipSuccess) return HAWK_ERR_LAUNCH;
     const int cols = (W + 1) * D;
@@ -401,14 +402,15 @@ int bwd_dispatch(const void* gy, const void* x, const float* w, void* dx, float*
 
 }  // namespace
 
-int conv1d_fwd(const void* x, const float* w, const float* bias, const void* state, void* y, int B, int T, int D,
-               int W, int x_dtype, int y_dtype, hipStream_t st) {
+int conv1d_fwd(const void* x, long long ldx, const float* w, const float* bias, const void* state, void* y,
+               long long ldy, int B, int T, int D, int W, int x_dtype, int y_dtype, hipStream_t st) {
+    const size_t lx = (size_t)ldx, ly = (size_t)ldy;
     if (x_dtype == HAWK_DTYPE_BF16) {
-        if (y_dtype == HAWK_DTYPE_BF16) return fwd_dispatch<bf16_t, bf16_t>(x, w, bias, state, y, B, T, D, W, st);
-        return fwd_dispatch<bf16_t, float>(x, w, bias, state, y, B, T, D, W, st);
+        if (y_dtype == HAWK_DTYPE_BF16) return fwd_dispatch<bf16_t, bf16_t>(x, w, bias, state, y, B, T, D, W, lx, ly, st);
+        return fwd_dispatch<bf16_t, float>(x, w, bias, state, y, B, T, D, W, lx, ly, st);
     }
-    if (y_dtype == HAWK_DTYPE_BF16) return fwd_dispatch<float, bf16_t>(x, w, bias, state, y, B, T, D, W, st);
-    return fwd_dispatch<float, float>(x, w, bias, state, y, B, T, D, W, st);
+    if (y_dtype == HAWK_DTYPE_BF16) return fwd_dispatch<float, bf16_t>(x, w, bias, state, y, B, T, D, W, lx, ly, st);
+    return fwd_dispatch<float, float>(x, w, bias, state, y, B, T, D, W, lx, ly, st);
 }
 
 size_t conv1d_bwd_workspace_bytes(int B, int T, int D, int W) {
@@ -416,16 +418,19 @@ size_t conv1d_bwd_workspace_bytes(int B, int T, int D, int W) {
     return align_up((size_t)p.ngroups * B * (size_t)(W + 1) * D * sizeof(float), 256);
 }
 
-int conv1d_bwd(const void* gy, const void* x, const float* w, void* dx, float* dw, float* db, int B, int T, int D,
-               int W, int x_dtype, int gy_dtype, void* ws, size_t ws_bytes, hipStream_t st) {
+int conv1d_bwd(const void* gy, const void* x, long long ldx, const float* w, void* dx, long long lddx, float* dw,
+               float* db, int B, int T, int D, int W, int x_dtype, int gy_dtype, void* ws, size_t ws_bytes,
+               hipStream_t st) {
     if (ws == nullptr || ws_bytes < conv1d_bwd_workspace_bytes(B, T, D, W)) return HAWK_ERR_WORKSPACE;
     float* part = static_cast<float*>(ws);
+    const size_t lx = (size_t)ldx, ld = (size_t)lddx;
     if (x_dtype == HAWK_DTYPE_BF16) {
-        if (gy_dtype == HAWK_DTYPE_BF16) return bwd_dispatch<bf16_t, bf16_t>(gy, x, w, dx, dw, db, B, T, D, W, part, st);
-        return bwd_dispatch<bf16_t, float>(gy, x, w, dx, dw, db, B, T, D, W, part, st);
+        if (gy_dtype == HAWK_DTYPE_BF16)
+            return bwd_dispatch<bf16_t, bf16_t>(gy, x, w, dx, dw, db, B, T, D, W, lx, ld, part, st);
+        return bwd_dispatch<bf16_t, float>(gy, x, w, dx, dw, db, B, T, D, W, lx, ld, part, st);
     }
-    if (gy_dtype == HAWK_DTYPE_BF16) return bwd_dispatch<float, bf16_t>(gy, x, w, dx, dw, db, B, T, D, W, part, st);
-    return bwd_dispatch<float, float>(gy, x, w, dx, dw, db, B, T, D, W, part, st);
+    if (gy_dtype == HAWK_DTYPE_BF16) return bwd_dispatch<float, bf16_t>(gy, x, w, dx, dw, db, B, T, D, W, lx, ld, part, st);
+    return bwd_dispatch<float, float>(gy, x, w, dx, dw, db, B, T, D, W, lx, ld, part, st);
 }
 
 }  // namespace hawk

@@ -177,18 +177,42 @@ struct WeightStage {
     static constexpr int kBytes = 2 * kGroup * kRowBytes;
 };
 
-template <typename XT, typename WT, typename OT, int BW>
+// With CONV the kernel's input is the temporal conv's input (hawk/hawk.py:172-176 upstream:
+// conv, then both gates) and the kernel applies the width-4 causal depthwise conv itself: a
+// raw tile lands in LDS with the three rows in front of it, every thread forms one row piece of
+// the conv output from four raw rows (fp32, taps oldest first, the arithmetic of
+// conv1d_fwd_kernel), writes it into the MFMA A tile and to memory, where the scan reads it.
+// The conv output is then never read back by this kernel: one pass over a tensor less.
+struct ConvFront {
+    const float* w;   // [4, D], tap 3 multiplies the row itself
+    const float* b;   // [D]
+    bf16_t* u;        // conv output, dense [M, D]
+    int T;            // rows per sequence: rows of one sequence never see another's
+    long long ldx;    // row stride of x in elements
+};
+constexpr int kConvTaps = 4;
+constexpr int kRTileBytes = (kTileRows + kConvTaps - 1) * kARowBytes;   // a raw tile and its history rows
+template <typename OT>
+constexpr size_t gate_fwd_lds_bytes(bool conv) {
+    return 2 * kATileBytes + (size_t)kTileRows * (2 * kGroup * sizeof(OT) + 16) +
+           (conv ? 2 * (size_t)kRTileBytes + (kConvTaps + 1) * kGroup * sizeof(float) : 0);
+}
+
+template <typename XT, typename WT, typename OT, int BW, bool CONV>
 __global__ __launch_bounds__(kGateThreads, 1) void gate_proj_fwd_kernel(
     const XT* __restrict__ x, const WT* __restrict__ w_i, const float* __restrict__ b_i,
     const WT* __restrict__ w_a, const float* __restrict__ b_a, OT* __restrict__ out_i, OT* __restrict__ out_a,
-    int M, int D, int nb, int ntiles) {
+    int M, int D, int nb, int ntiles, ConvFront cf) {
     static_assert(BW == 32 || BW == 64 || BW == 128 || BW == 256, "block width");
+    static_assert(!CONV || sizeof(XT) == 2, "the fused conv runs on bf16 activations");
     constexpr int KS = BW / 16;                                     // MFMA k-steps per output tile
     constexpr int G = kGroup / BW;                                  // whole blocks per workgroup
     constexpr int kORowBytes = 2 * kGroup * (int)sizeof(OT) + 16;   // both gates' columns of one row + pad
     extern __shared__ __align__(16) unsigned char smem[];
     unsigned char* sA = smem;                     // two activation tiles
     unsigned char* sO = smem + 2 * kATileBytes;   // one result tile
+    unsigned char* sR = sO + kTileRows * kORowBytes;                      // CONV: two raw tiles
+    float* sCW = reinterpret_cast<float*>(sR + 2 * kRTileBytes);          // CONV: taps and bias of the group
 
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
@@ -222,13 +246,83 @@ __global__ __launch_bounds__(kGateThreads, 1) void gate_proj_fwd_kernel(
     auto stage_tile = [&](int buf, const Row8<XT>& r) {
         *reinterpret_cast<u32x4*>(sA + buf * kATileBytes + lrow * kARowBytes + lc8 * 16) = r.as_bf16();
     };
+    // CONV: a raw tile is its 32 rows and the three rows in front of them (threads of the first
+    // three rows fetch one history piece each; every other thread's second load is out of range
+    // and costs no memory access).  Rows in front of the tensor do not exist and are masked later.
+    const uint32_t ldx_bytes = CONV ? (uint32_t)cf.ldx * 2u : 0u;
+    auto load_raw_tile = [&](int it, auto& r, auto& hist) {
+        const int t = min(worker + it * nworkers, ntiles);
+        const int row0 = min(t * kTileRows, M);
+        const int hb = row0 >= kConvTaps - 1 ? kConvTaps - 1 : 0;
+        const int nrows = min(M - row0, kTileRows) + hb;
+        const rsrc_t rs = make_rsrc(x + (size_t)(row0 - hb) * (size_t)cf.ldx,
+                                    nrows > 0 ? (uint32_t)(nrows - 1) * ldx_bytes + (uint32_t)D * 2u : 0u);
+        const uint32_t col_bytes = (uint32_t)lcol * 2u;
+        r.load_buf_default(rs, col_ok ? (uint32_t)(hb + lrow) * ldx_bytes + col_bytes : 0x80000000u);
+        hist.load_buf_default(rs, (col_ok && lrow < hb) ? (uint32_t)lrow * ldx_bytes + col_bytes : 0x80000000u);
+    };
+    auto stage_raw_tile = [&](int buf, const auto& r, const auto& hist) {
+        unsigned char* dst = sR + buf * kRTileBytes + lrow * kARowBytes + lc8 * 16;
+        *reinterpret_cast<u32x4*>(dst + (kConvTaps - 1) * kARowBytes) = r.as_bf16();
+        if (lrow < kConvTaps - 1) *reinterpret_cast<u32x4*>(dst) = hist.as_bf16();
+    };
+    // conv of tile j from raw buffer `buf` into A buffer `buf`, and out to memory
+    auto conv_tile = [&](int j, int buf) {
+        const int tt = worker + j * nworkers;
+        if (tt >= ntiles) return;
+        const int row0 = tt * kTileRows;
+        int t = row0 % cf.T + lrow;   // position in the sequence (T >= 32: at most one wrap)
+        if (t >= cf.T) t -= cf.T;
+        const unsigned char* src = sR + buf * kRTileBytes + lrow * kARowBytes + lc8 * 16;
+        const float* cw = sCW + lc8 * 8;
+        float acc[8];
+        {
+            const f32x4 b0 = *reinterpret_cast<const f32x4*>(cw + kConvTaps * kGroup);
+            const f32x4 b1 = *reinterpret_cast<const f32x4*>(cw + kConvTaps * kGroup + 4);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) acc[e] = b0[e], acc[4 + e] = b1[e];
+        }
+#pragma unroll
+        for (int k = 0; k < kConvTaps; ++k) {
+            u32x4 v = *reinterpret_cast<const u32x4*>(src + k * kARowBytes);   // row t - (3 - k)
+            if (t < kConvTaps - 1 - k) v = u32x4{0u, 0u, 0u, 0u};             // before the sequence starts
+            const f32x4 w0 = *reinterpret_cast<const f32x4*>(cw + k * kGroup);
+            const f32x4 w1 = *reinterpret_cast<const f32x4*>(cw + k * kGroup + 4);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const float lo = (e & 1) ? bf16_hi(v[e / 2]) : bf16_lo(v[e / 2]);
+                const float hi = (e & 1) ? bf16_hi(v[2 + e / 2]) : bf16_lo(v[2 + e / 2]);
+                acc[e] = fmaf(w0[e], lo, acc[e]);
+                acc[4 + e] = fmaf(w1[e], hi, acc[4 + e]);
+            }
+        }
+        const u32x4 o = {pack_bf16x2(acc[0], acc[1]), pack_bf16x2(acc[2], acc[3]), pack_bf16x2(acc[4], acc[5]),
+                         pack_bf16x2(acc[6], acc[7])};
+        *reinterpret_cast<u32x4*>(sA + buf * kATileBytes + lrow * kARowBytes + lc8 * 16) = o;
+        const int row = row0 + lrow;
+        if (row < M && col_ok)
+            __builtin_nontemporal_store(o, reinterpret_cast<u32x4*>(cf.u + (size_t)row * D + lcol));
+    };
 
     // Two register sets alternate as landing places for the prefetched tiles (tile it+1 is
     // staged into LDS during iteration it, and its registers are reloaded with tile it+3), and
-    // the loop is unrolled by two so that buffers and registers are fixed per half.
-    Row8<XT> ra, rb;
-    load_tile(0, ra);
-    load_tile(1, rb);
+    // the loop is unrolled by two so that buffers and registers are fixed per half.  With CONV a
+    // tile is staged raw one iteration earlier (tile it+2 during iteration it, its registers
+    // reloaded with tile it+4) and convolved into the A buffer during iteration it+1's stores.
+    Row8<XT> ra, rb, ha, hb_;
+    if constexpr (CONV) {
+        load_raw_tile(0, ra, ha);
+        load_raw_tile(1, rb, hb_);
+        if (tid < kGroup) {
+            const int cch = group * kGroup + tid;
+#pragma unroll
+            for (int k = 0; k < kConvTaps; ++k) sCW[k * kGroup + tid] = cch < D ? cf.w[(size_t)k * D + cch] : 0.0f;
+            sCW[kConvTaps * kGroup + tid] = cch < D ? cf.b[cch] : 0.0f;
+        }
+    } else {
+        load_tile(0, ra);
+        load_tile(1, rb);
+    }
     __builtin_amdgcn_sched_barrier(0);  // the first tiles travel while the weights are fetched
 
     // ---- the weights.  A lane's B operand is 8 consecutive input channels of one output
@@ -280,14 +374,23 @@ __global__ __launch_bounds__(kGateThreads, 1) void gate_proj_fwd_kernel(
         __syncthreads();
     }
 
-    stage_tile(0, ra);
-    load_tile(2, ra);
+    if constexpr (CONV) {
+        stage_raw_tile(0, ra, ha);
+        load_raw_tile(2, ra, ha);
+        stage_raw_tile(1, rb, hb_);
+        load_raw_tile(3, rb, hb_);
+        __syncthreads();
+        conv_tile(0, 0);
+    } else {
+        stage_tile(0, ra);
+        load_tile(2, ra);
+    }
     __syncthreads();
 
     const int a_off = col * kARowBytes + (blk * BW + khalf) * 2;
     unsigned char* o_base = sO + (4 * (lane >> 5)) * kORowBytes + (g * kGroup + 32 * c + col) * (int)sizeof(OT);
 
-    auto step = [&](int it, int cur, Row8<XT>& rnext) {
+    auto step = [&](int it, int cur, Row8<XT>& rnext, Row8<XT>& hnext) {
         // 32 x 32 output tile of this wave: A operands from LDS, B operands resident.  The A
         // operands are fetched four k-steps at a time: the weights leave no room for more.
         f32x16 acc = {};
@@ -309,9 +412,15 @@ __global__ __launch_bounds__(kGateThreads, 1) void gate_proj_fwd_kernel(
             const int m = 8 * (r / 4) + (r % 4);
             store_out(o_base + m * kORowBytes, acc[r] + bias, static_cast<OT*>(nullptr));
         }
-        // tile it+1 into the other buffer, tile it+3 into the registers it leaves
-        stage_tile(cur ^ 1, rnext);
-        load_tile(it + 3, rnext);
+        if constexpr (CONV) {
+            // raw tile it+2 into the raw buffer tile it has left, tile it+4 into its registers
+            stage_raw_tile(cur, rnext, hnext);
+            load_raw_tile(it + 4, rnext, hnext);
+        } else {
+            // tile it+1 into the other buffer, tile it+3 into the registers it leaves
+            stage_tile(cur ^ 1, rnext);
+            load_tile(it + 3, rnext);
+        }
         __syncthreads();
         // a gate's row of the group is 32 (bf16) or 64 (fp32) pieces of 16 bytes; consecutive
         // threads take consecutive pieces, so that every store instruction writes whole rows
@@ -331,13 +440,14 @@ __global__ __launch_bounds__(kGateThreads, 1) void gate_proj_fwd_kernel(
                 __builtin_nontemporal_store(va, reinterpret_cast<u32x4*>(out_a + (size_t)row * D + ocol));
             }
         }
+        if constexpr (CONV) conv_tile(it + 1, cur ^ 1);
         __syncthreads();
     };
 
     for (int it = 0; worker + it * nworkers < ntiles; it += 2) {
-        step(it, 0, rb);
+        if constexpr (CONV) step(it, 0, ra, ha); else step(it, 0, rb, hb_);
         if (worker + (it + 1) * nworkers >= ntiles) break;
-        step(it + 1, 1, ra);
+        if constexpr (CONV) step(it + 1, 1, rb, hb_); else step(it + 1, 1, ra, ha);
     }
 }
 
@@ -1183,14 +1293,49 @@ int launch_gate_fwd(const void* x, const void* w_i, const float* b_i, const void
     int nworkers = kNumCU / ngroups;
     if (nworkers < 1) nworkers = 1;
     if (nworkers > ntiles) nworkers = ntiles;
-    size_t smem = 2 * kATileBytes + (size_t)kTileRows * (2 * kGroup * sizeof(OT) + 16);
+    size_t smem = gate_fwd_lds_bytes<OT>(false);
     if (smem < (size_t)WeightStage<BW>::kBytes) smem = WeightStage<BW>::kBytes;
-    constexpr auto kernel = gate_proj_fwd_kernel<XT, WT, OT, BW>;
+    constexpr auto kernel = gate_proj_fwd_kernel<XT, WT, OT, BW, false>;
     if (!allow_dynamic_lds<kernel>(smem)) return HAWK_ERR_LAUNCH;
     hipLaunchKernelGGL(kernel, dim3((unsigned)nworkers, (unsigned)ngroups), dim3(kGateThreads), smem, st,
                        static_cast<const XT*>(x), static_cast<const WT*>(w_i), b_i, static_cast<const WT*>(w_a), b_a,
-                       static_cast<OT*>(out_i), static_cast<OT*>(out_a), M, D, nb, ntiles);
+                       static_cast<OT*>(out_i), static_cast<OT*>(out_a), M, D, nb, ntiles, ConvFront{});
     return hipGetLastError() == hipSuccess ? HAWK_OK : HAWK_ERR_LAUNCH;
+}
+
+// The forward with the temporal conv in front (bf16 activations; the weight-transposition scratch
+// of the prologue must stay clear of the conv taps at the end of the LDS block).
+template <typename WT, int BW>
+int launch_conv_gate_fwd(const void* x, long long ldx, const float* conv_w, const float* conv_b, const void* w_i,
+                         const float* b_i, const void* w_a, const float* b_a, void* u, void* out_i, void* out_a,
+                         int M, int T, int D, int nb, hipStream_t st) {
+    const int ngroups = ceil_div(D, kGroup);
+    const int ntiles = ceil_div(M, kTileRows);
+    int nworkers = kNumCU / ngroups;
+    if (nworkers < 1) nworkers = 1;
+    if (nworkers > ntiles) nworkers = ntiles;
+    constexpr size_t smem = gate_fwd_lds_bytes<bf16_t>(true);
+    static_assert((size_t)WeightStage<BW>::kBytes <= smem - (kConvTaps + 1) * kGroup * sizeof(float), "LDS layout");
+    constexpr auto kernel = gate_proj_fwd_kernel<bf16_t, WT, bf16_t, BW, true>;
+    if (!allow_dynamic_lds<kernel>(smem)) return HAWK_ERR_LAUNCH;
+    const ConvFront cf = {conv_w, conv_b, static_cast<bf16_t*>(u), T, ldx};
+    hipLaunchKernelGGL(kernel, dim3((unsigned)nworkers, (unsigned)ngroups), dim3(kGateThreads), smem, st,
+                       static_cast<const bf16_t*>(x), static_cast<const WT*>(w_i), b_i, static_cast<const WT*>(w_a),
+                       b_a, static_cast<bf16_t*>(out_i), static_cast<bf16_t*>(out_a), M, D, nb, ntiles, cf);
+    return hipGetLastError() == hipSuccess ? HAWK_OK : HAWK_ERR_LAUNCH;
+}
+
+template <typename WT>
+int conv_gate_fwd_bw(const void* x, long long ldx, const float* conv_w, const float* conv_b, const void* w_i,
+                     const float* b_i, const void* w_a, const float* b_a, void* u, void* out_i, void* out_a, int M,
+                     int T, int D, int nb, int bw, hipStream_t st) {
+    switch (bw) {
+        case 32: return launch_conv_gate_fwd<WT, 32>(x, ldx, conv_w, conv_b, w_i, b_i, w_a, b_a, u, out_i, out_a, M, T, D, nb, st);
+        case 64: return launch_conv_gate_fwd<WT, 64>(x, ldx, conv_w, conv_b, w_i, b_i, w_a, b_a, u, out_i, out_a, M, T, D, nb, st);
+        case 128: return launch_conv_gate_fwd<WT, 128>(x, ldx, conv_w, conv_b, w_i, b_i, w_a, b_a, u, out_i, out_a, M, T, D, nb, st);
+        case 256: return launch_conv_gate_fwd<WT, 256>(x, ldx, conv_w, conv_b, w_i, b_i, w_a, b_a, u, out_i, out_a, M, T, D, nb, st);
+        default: return HAWK_ERR_BAD_SHAPE;
+    }
 }
 
 template <typename XT, typename WT, typename OT>
@@ -1409,6 +1554,15 @@ int gate_proj_fwd(const void* x, const void* w_i, const float* b_i, const void* 
     if (w_dtype == HAWK_DTYPE_BF16)
         return gate_fwd_out<float, bf16_t>(x, w_i, b_i, w_a, b_a, out_i, out_a, M, D, nb, bw, out_dtype, st);
     return gate_fwd_out<float, float>(x, w_i, b_i, w_a, b_a, out_i, out_a, M, D, nb, bw, out_dtype, st);
+}
+
+int conv_gate_proj_fwd(const void* x, long long ldx, const float* conv_w, const float* conv_b, const void* w_i,
+                       const float* b_i, const void* w_a, const float* b_a, void* u, void* out_i, void* out_a, int B,
+                       int T, int D, int nb, int w_dtype, hipStream_t st) {
+    const int bw = D / nb, M = B * T;
+    if (w_dtype == HAWK_DTYPE_BF16)
+        return conv_gate_fwd_bw<bf16_t>(x, ldx, conv_w, conv_b, w_i, b_i, w_a, b_a, u, out_i, out_a, M, T, D, nb, bw, st);
+    return conv_gate_fwd_bw<float>(x, ldx, conv_w, conv_b, w_i, b_i, w_a, b_a, u, out_i, out_a, M, T, D, nb, bw, st);
 }
 
 int gate_proj_bwd_input(const void* dxg, const void* dag, const void* w_i, const void* w_a, const void* addend,

@@ -34,11 +34,13 @@ int scan_gated_bwd(const void* x, const void* xg, const void* ag, const float* l
                    hipStream_t st);
 
 // hawk_conv.hip
-int conv1d_fwd(const void* x, const float* w, const float* bias, const void* state, void* y, int B, int T, int D,
-               int W, int x_dtype, int y_dtype, hipStream_t st);
+// ldx, ldy, lddx: row strides in elements (>= D); batch rows lie T rows apart
+int conv1d_fwd(const void* x, long long ldx, const float* w, const float* bias, const void* state, void* y,
+               long long ldy, int B, int T, int D, int W, int x_dtype, int y_dtype, hipStream_t st);
 size_t conv1d_bwd_workspace_bytes(int B, int T, int D, int W);
-int conv1d_bwd(const void* gy, const void* x, const float* w, void* dx, float* dw, float* db, int B, int T, int D,
-               int W, int x_dtype, int gy_dtype, void* ws, size_t ws_bytes, hipStream_t st);
+int conv1d_bwd(const void* gy, const void* x, long long ldx, const float* w, void* dx, long long lddx, float* dw,
+               float* db, int B, int T, int D, int W, int x_dtype, int gy_dtype, void* ws, size_t ws_bytes,
+               hipStream_t st);
 
 // hawk_step.hip
 int conv1d_step(void* conv_state, const void* x_new, const float* w, const float* bias, void* y, int B, int D,
@@ -53,6 +55,11 @@ int rglru_step_gated(const void* x, const void* xg, const void* ag, const float*
 bool gate_proj_block_width_supported(int bw);
 int gate_proj_fwd(const void* x, const void* w_i, const float* b_i, const void* w_a, const float* b_a, void* out_i,
                   void* out_a, int M, int D, int nb, int x_dtype, int w_dtype, int out_dtype, hipStream_t st);
+// temporal conv (width 4, bf16 in and out, x rows ldx elements apart) and both projections of
+// its output in one kernel; u receives the conv output
+int conv_gate_proj_fwd(const void* x, long long ldx, const float* conv_w, const float* conv_b, const void* w_i,
+                       const float* b_i, const void* w_a, const float* b_a, void* u, void* out_i, void* out_a, int B,
+                       int T, int D, int nb, int w_dtype, hipStream_t st);
 int gate_proj_bwd_input(const void* dxg, const void* dag, const void* w_i, const void* w_a, const void* addend,
                         void* dx, int M, int D, int nb, int g_dtype, int w_dtype, int dx_dtype, hipStream_t st);
 // conv window roll + conv, both projections, state update and output gate of one decode step

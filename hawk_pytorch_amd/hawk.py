@@ -41,7 +41,13 @@ from .external import (
     temporal_conv1d,
     temporal_conv1d_step,
 )
-from .scan_fused import fused_linear_scan, fused_linear_scan_gated, recurrent_core
+from .scan_fused import (
+    block_core_layout_ok,
+    fused_linear_scan,
+    fused_linear_scan_gated,
+    recurrent_block_core,
+    recurrent_core,
+)
 
 
 @dataclass
@@ -63,6 +69,10 @@ class HawkConfig:
     # not an upstream field: with both of the above, a decode step's conv, projections, state
     # update and output gate as one launch (hawk/hawk.py:137-151, :169-182, :196-198)
     fused_decode_core: bool = True
+    # not an upstream field: with fused_epilogue and fused_gates, a sequence's conv, projections,
+    # scan and output gate as one autograd node that reads both halves of the input projection
+    # in place and returns that projection's gradient as one tensor (hawk/hawk.py:163-186)
+    fused_block_core: bool = True
 
     def __post_init__(self):
         if self.post_norm:
@@ -132,7 +142,8 @@ class Hawk(nn.Module):
 
     def forward(self, x: torch.Tensor, layer_past: Optional[RNNCache]) -> Tuple[torch.Tensor, Optional[RNNCache]]:
         warm = self.use_cache and layer_past is not None and layer_past.current_cache_size > 0
-        branch, gate_branch = self.input_xy(x).chunk(2, dim=-1)
+        xy = self.input_xy(x)
+        branch, gate_branch = xy.chunk(2, dim=-1)
 
         if warm:
             # One new token per batch row.  (Upstream accepts more and silently keeps only the
@@ -177,6 +188,14 @@ class Hawk(nn.Module):
                 layer_past.seed_conv_state(branch)
             cache = layer_past if self.use_cache else None
             if self.config.fused_gates and gate_projections_supported(branch, self.rg_lru_input_gate):
+                if (self.config.fused_epilogue and self.config.fused_block_core and block_core_layout_ok(xy)):
+                    # conv, projections, scan and output gate as one autograd node on xy itself
+                    gated, h_last = recurrent_block_core(xy, self.conv1d, self.rg_lru_input_gate,
+                                                         self.rg_lru_a_gate, self.rg_lru_a_param,
+                                                         return_last_state=True)
+                    if self.use_cache:
+                        layer_past.update_cache(h_last)
+                    return self.resid_proj(gated), cache
                 # bf16 end to end: upstream's gate einsums (under autocast) and its scan
                 # (cast_inputs, hawk/scan_fused.py:428) round the conv output to bf16 anyway
                 u = temporal_conv1d(branch, self.conv1d.w, self.conv1d.b, torch.bfloat16)

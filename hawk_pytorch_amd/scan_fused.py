@@ -468,3 +468,188 @@ def recurrent_core(u, input_gate, a_gate, a_param, y, return_last_state: bool = 
     out, h_last = RecurrentCore.apply(u, input_gate.w, input_gate.b, a_gate.w, a_gate.b, a_param, y,
                                       return_last_state)
     return (out, h_last) if return_last_state else out
+
+
+# ---------------------------------------------------------------------------------------
+# The same node with the temporal conv in front, fed by the block's input projection itself
+# (hawk/hawk.py:163-186: chunk, Conv1D, both gates, scan, output gate).  xy is the [B,T,2D]
+# output of that projection: the conv reads its first half and the output gate its second half
+# in place (upstream's chunk gives views, but its Conv1D and scan copy them), the conv and both
+# gate projections are one kernel, and the backward writes the two halves of the gradient of
+# xy side by side into one tensor, where autograd would concatenate two.  One custom op per
+# direction, so the host issues two calls per layer.
+# ---------------------------------------------------------------------------------------
+_FUSED_CONV_MIN_T = 32   # hawk_conv_gate_proj_fwd needs T >= 32 and a temporal width of 4
+
+
+def block_core_layout_ok(xy: torch.Tensor) -> bool:
+    """xy [B,T,2D] bf16 on the GPU with unit channel stride and evenly spaced rows a multiple of
+    8 elements apart: what the kernels read in place.  (Plain Python on shapes and strides, so a
+    tracing compiler sees through it.)"""
+    if xy.dim() != 3 or xy.dtype != torch.bfloat16 or xy.device.type != "cuda" or xy.shape[-1] % 16 != 0:
+        return False
+    ld = _row_stride(xy)
+    return ld is not None and ld % 8 == 0
+
+
+def _launch_block_core_fwd(xy, conv_w, conv_b, w_i, b_i, w_a, b_a, lam, want_h: bool, want_last: bool):
+    from .external import _gate_workspace  # noqa: F401  (deferred: external imports nothing from here)
+
+    dev = _lib.require_cuda(xy, conv_w, conv_b, w_i, b_i, w_a, b_a, lam)
+    if xy.data_ptr() % 16 != 0:
+        xy = xy.clone(memory_format=torch.contiguous_format)
+    B, T, D2 = xy.shape
+    D = D2 // 2
+    ld = _row_stride(xy)
+    W = conv_w.shape[0]
+    nb = w_i.shape[0]
+    conv_w, conv_b, w_i, w_a, b_i, b_a, lam = (_lib.dense16(t) for t in (conv_w, conv_b, w_i, w_a, b_i, b_a, lam))
+    bf, code = torch.bfloat16, _lib.HAWK_DTYPE_BF16
+    u, xg, ag, out = (torch.empty((B, T, D), dtype=bf, device=dev) for _ in range(4))
+    h = torch.empty((B, T, D) if want_h else (0,), dtype=bf, device=dev)
+    h_last = torch.empty((B, 1, D) if want_last else (0,), dtype=bf, device=dev)
+    lib = _lib.load()
+    ws = _lib.scan_workspace(dev, lib.hawk_scan_workspace_bytes(B, T, D, code))
+    y_ptr = xy.data_ptr() + D * xy.element_size()
+    with torch.cuda.device(dev):
+        st = _lib.stream_ptr(dev)
+        if W == 4 and T >= _FUSED_CONV_MIN_T:
+            _lib.check("hawk_conv_gate_proj_fwd", lib.hawk_conv_gate_proj_fwd(
+                xy.data_ptr(), ld, conv_w.data_ptr(), conv_b.data_ptr(), w_i.data_ptr(), b_i.data_ptr(),
+                w_a.data_ptr(), b_a.data_ptr(), u.data_ptr(), xg.data_ptr(), ag.data_ptr(), B, T, D, nb, W,
+                _lib.dtype_code(w_i.dtype), st))
+        else:
+            _lib.check("hawk_conv1d_fwd_strided", lib.hawk_conv1d_fwd_strided(
+                xy.data_ptr(), ld, conv_w.data_ptr(), conv_b.data_ptr(), None, u.data_ptr(), D, B, T, D, W, code,
+                code, st))
+            _lib.check("hawk_gate_proj_fwd", lib.hawk_gate_proj_fwd(
+                u.data_ptr(), w_i.data_ptr(), b_i.data_ptr(), w_a.data_ptr(), b_a.data_ptr(), xg.data_ptr(),
+                ag.data_ptr(), B * T, D, nb, code, _lib.dtype_code(w_i.dtype), code, st))
+        _lib.check("hawk_rglru_scan_gated_fwd", lib.hawk_rglru_scan_gated_fwd(
+            u.data_ptr(), xg.data_ptr(), ag.data_ptr(), lam.data_ptr(), y_ptr, ld,
+            h.data_ptr() if want_h else None, out.data_ptr(), h_last.data_ptr() if want_last else None,
+            B, T, D, code, code, ws.data_ptr(), ws.numel(), st))
+    return out, u, xg, ag, h, h_last
+
+
+def _launch_block_core_bwd(xy, u, xg, ag, h, conv_w, w_i, w_a, lam, grad_out):
+    from .external import _gate_workspace
+
+    dev = _lib.require_cuda(xy, u, xg, ag, h, conv_w, w_i, w_a, lam, grad_out)
+    if xy.data_ptr() % 16 != 0:
+        xy = xy.clone(memory_format=torch.contiguous_format)
+    B, T, D2 = xy.shape
+    D = D2 // 2
+    ld = _row_stride(xy)
+    W = conv_w.shape[0]
+    nb, bw, _ = w_i.shape
+    M = B * T
+    conv_w, w_i, w_a, lam, grad_out = (_lib.dense16(t) for t in (conv_w, w_i, w_a, lam, grad_out))
+    bf, code, f32 = torch.bfloat16, _lib.HAWK_DTYPE_BF16, torch.float32
+    lib = _lib.load()
+    d_xy = torch.empty((B, T, D2), dtype=bf, device=dev)
+    du, dxg, dag = (torch.empty((B, T, D), dtype=bf, device=dev) for _ in range(3))
+    dlam = torch.empty(D, dtype=f32, device=dev)
+    dw_i, dw_a = (torch.empty((nb, bw, bw), dtype=f32, device=dev) for _ in range(2))
+    db_i, db_a, dcb = (torch.empty(D, dtype=f32, device=dev) for _ in range(3))
+    dcw = torch.empty((W, D), dtype=f32, device=dev)
+    ws = _lib.scan_workspace(dev, lib.hawk_scan_workspace_bytes(B, T, D, code))
+    gws = _gate_workspace(dev, lib.hawk_gate_proj_bwd_weights_workspace_bytes(M, D, nb))
+    cws = torch.empty(lib.hawk_conv1d_bwd_workspace_bytes(B, T, D, W), dtype=torch.uint8, device=dev)
+    y_ptr = xy.data_ptr() + D * xy.element_size()
+    dy_ptr = d_xy.data_ptr() + D * d_xy.element_size()
+    wcode = _lib.dtype_code(w_i.dtype)
+    with torch.cuda.device(dev):
+        st = _lib.stream_ptr(dev)
+        _lib.check("hawk_rglru_scan_gated_bwd", lib.hawk_rglru_scan_gated_bwd(
+            u.data_ptr(), xg.data_ptr(), ag.data_ptr(), lam.data_ptr(), y_ptr, ld, h.data_ptr(),
+            grad_out.data_ptr(), du.data_ptr(), dxg.data_ptr(), dag.data_ptr(), dy_ptr, D2, dlam.data_ptr(),
+            B, T, D, code, code, ws.data_ptr(), ws.numel(), st))
+        # the projections' input gradient accumulates onto the scan's, in place
+        _lib.check("hawk_gate_proj_bwd_input", lib.hawk_gate_proj_bwd_input(
+            dxg.data_ptr(), dag.data_ptr(), w_i.data_ptr(), w_a.data_ptr(), du.data_ptr(), du.data_ptr(), M, D, nb,
+            code, wcode, code, st))
+        _lib.check("hawk_gate_proj_bwd_weights", lib.hawk_gate_proj_bwd_weights(
+            u.data_ptr(), dxg.data_ptr(), dag.data_ptr(), dw_i.data_ptr(), db_i.data_ptr(), dw_a.data_ptr(),
+            db_a.data_ptr(), M, D, nb, code, code, gws.data_ptr(), gws.numel(), st))
+        _lib.check("hawk_conv1d_bwd_strided", lib.hawk_conv1d_bwd_strided(
+            du.data_ptr(), xy.data_ptr(), ld, conv_w.data_ptr(), d_xy.data_ptr(), D2, dcw.data_ptr(),
+            dcb.data_ptr(), B, T, D, W, code, code, cws.data_ptr(), cws.numel(), st))
+    return d_xy, dcw, dcb, dw_i, db_i, dw_a, db_a, dlam
+
+
+@torch.library.custom_op("hawk_amd::block_core_fwd", mutates_args=(), device_types="cuda")
+def _block_core_fwd_op(
+    xy: torch.Tensor, conv_w: torch.Tensor, conv_b: torch.Tensor, w_i: torch.Tensor, b_i: torch.Tensor,
+    w_a: torch.Tensor, b_a: torch.Tensor, a_param: torch.Tensor, want_h: bool, want_last: bool,
+) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+    return _launch_block_core_fwd(xy, conv_w, conv_b, w_i, b_i, w_a, b_a, a_param, want_h, want_last)
+
+
+@_block_core_fwd_op.register_fake
+def _(xy, conv_w, conv_b, w_i, b_i, w_a, b_a, a_param, want_h, want_last):
+    B, T, D2 = xy.shape
+    D = D2 // 2
+    e = lambda *s: torch.empty(s, dtype=torch.bfloat16, device=xy.device)  # noqa: E731
+    return (e(B, T, D), e(B, T, D), e(B, T, D), e(B, T, D), e(B, T, D) if want_h else e(0),
+            e(B, 1, D) if want_last else e(0))
+
+
+@torch.library.custom_op("hawk_amd::block_core_bwd", mutates_args=(), device_types="cuda")
+def _block_core_bwd_op(
+    xy: torch.Tensor, u: torch.Tensor, xg: torch.Tensor, ag: torch.Tensor, h: torch.Tensor, conv_w: torch.Tensor,
+    w_i: torch.Tensor, w_a: torch.Tensor, a_param: torch.Tensor, grad_out: torch.Tensor,
+) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor,
+           torch.Tensor]:
+    return _launch_block_core_bwd(xy, u, xg, ag, h, conv_w, w_i, w_a, a_param, grad_out)
+
+
+@_block_core_bwd_op.register_fake
+def _(xy, u, xg, ag, h, conv_w, w_i, w_a, a_param, grad_out):
+    nb, bw, _ = w_i.shape
+    D = nb * bw
+    f = lambda *s: torch.empty(s, dtype=torch.float32, device=xy.device)  # noqa: E731
+    return (torch.empty(xy.shape, dtype=torch.bfloat16, device=xy.device), f(conv_w.shape[0], D), f(D),
+            f(nb, bw, bw), f(D), f(nb, bw, bw), f(D), f(D))
+
+
+class BlockCore(Function):
+    @staticmethod
+    def forward(ctx, xy, conv_w, conv_b, w_i, b_i, w_a, b_a, a_param, want_last):
+        from .external import kernel_weights
+
+        assert block_core_layout_ok(xy), "xy must be a [B,T,2D] bf16 tensor the kernels can read in place"
+        B, T, D2 = xy.shape
+        assert a_param.shape == (D2 // 2,), "Error: a_param does not match the channel count"
+        ctx.dtypes = tuple(t.dtype for t in (conv_w, conv_b, w_i, b_i, w_a, b_a, a_param))
+        lam = a_param.float().contiguous()
+        cw = conv_w.float().contiguous()
+        w_i16, w_a16 = kernel_weights(w_i, w_a, B * T)
+        want_h = any(ctx.needs_input_grad[:8])
+        out, u, xg, ag, h, h_last = _block_core_fwd_op(
+            xy, cw, conv_b.float().contiguous(), w_i16, b_i.float().reshape(-1), w_a16, b_a.float().reshape(-1),
+            lam, want_h, bool(want_last))
+        if want_h:
+            ctx.save_for_backward(xy, u, xg, ag, h, cw, w_i16, w_a16, lam)
+        ctx.mark_non_differentiable(h_last)
+        return out, h_last
+
+    @staticmethod
+    def backward(ctx, grad_out, _grad_last):  # type: ignore[override]
+        xy, u, xg, ag, h, cw, w_i, w_a, lam = ctx.saved_tensors
+        go = grad_out if grad_out.dtype == torch.bfloat16 else grad_out.to(torch.bfloat16)
+        go = go if go.is_contiguous() else go.contiguous()
+        d_xy, dcw, dcb, dw_i, db_i, dw_a, db_a, dlam = _block_core_bwd_op(xy, u, xg, ag, h, cw, w_i, w_a, lam, go)
+        nb, bw, _ = w_i.shape
+        t = ctx.dtypes
+        return (d_xy, dcw.to(t[0]), dcb.to(t[1]), dw_i.to(t[2]), db_i.reshape(nb, bw).to(t[3]), dw_a.to(t[4]),
+                db_a.reshape(nb, bw).to(t[5]), dlam.to(t[6]), None)
+
+
+def recurrent_block_core(xy, conv, input_gate, a_gate, a_param, return_last_state: bool = False):
+    """``gelu(y) * scan(u, input_gate(u), a_gate(u), a_param)`` with ``u = conv(x)`` and
+    ``x, y = xy.chunk(2, -1)``, for a bf16 ``xy`` that ``block_core_layout_ok`` accepts and gate
+    modules the fused projection kernels serve (``external.gate_projections_supported``)."""
+    out, h_last = BlockCore.apply(xy, conv.w, conv.b, input_gate.w, input_gate.b, a_gate.w, a_gate.b, a_param,
+                                  return_last_state)
+    return (out, h_last) if return_last_state else out

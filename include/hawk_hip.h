@@ -176,6 +176,14 @@ int hawk_conv1d_fwd(const void* x, const float* w, const float* bias, const void
                     void* y, int B, int T, int D, int W, int x_dtype, int y_dtype,
                     void* stream);
 
+/* The same with rows of x and y further apart than D elements (x_row_stride, y_row_stride >= D,
+ * in elements; batch rows lie T rows apart): the x half of the block's [B,T,2D] input
+ * projection (hawk/hawk.py:163-164, a chunk of one tensor) is read in place instead of
+ * being copied out first.  `state` stays dense.  Same upstream lines as hawk_conv1d_fwd. */
+int hawk_conv1d_fwd_strided(const void* x, long long x_row_stride, const float* w, const float* bias,
+                            const void* state, void* y, long long y_row_stride, int B, int T, int D,
+                            int W, int x_dtype, int y_dtype, void* stream);
+
 /* Size of the scratch buffer hawk_conv1d_bwd needs for its dw/db partial sums. */
 size_t hawk_conv1d_bwd_workspace_bytes(int B, int T, int D, int W);
 
@@ -185,6 +193,15 @@ size_t hawk_conv1d_bwd_workspace_bytes(int B, int T, int D, int W);
 int hawk_conv1d_bwd(const void* grad_y, const void* x, const float* w, void* dx, float* dw,
                     float* db, int B, int T, int D, int W, int x_dtype, int gy_dtype,
                     void* workspace_device, size_t workspace_bytes, void* stream);
+
+/* The same with rows of x and dx further apart than D elements: x is read from, and dx written
+ * into, the x half of a [B,T,2D] tensor in place (the gradient of the input projection's
+ * output is then one tensor that this call and hawk_rglru_scan_gated_bwd fill side by side,
+ * where autograd would concatenate two).  grad_y is dense. */
+int hawk_conv1d_bwd_strided(const void* grad_y, const void* x, long long x_row_stride, const float* w,
+                            void* dx, long long dx_row_stride, float* dw, float* db, int B, int T, int D,
+                            int W, int x_dtype, int gy_dtype, void* workspace_device,
+                            size_t workspace_bytes, void* stream);
 
 /* ---------------------------------------------------------------------------------------
  * Decode steps (one new token per batch row).
@@ -282,6 +299,22 @@ int hawk_decode_core_step_ws(void* conv_state, const void* x_new, long long ldx,
 int hawk_gate_proj_fwd(const void* x, const void* w_i, const float* b_i, const void* w_a,
                        const float* b_a, void* x_rg_lru, void* a_rg_lru, int M, int D,
                        int num_blocks, int x_dtype, int w_dtype, int out_dtype, void* stream);
+
+/* The temporal conv and both gate projections of its output in one pass over the conv's input:
+ *   u[b, t, c]  = conv_b[c] + sum_k conv_w[k, c] x[b, t - (3 - k), c]   (rows before t = 0 are zero)
+ *   x_rg_lru, a_rg_lru = hawk_gate_proj_fwd(u)
+ * Replaces Conv1D.forward followed by the two BlockDiagonalLinear calls (hawk/hawk.py:172-182,
+ * hawk/external.py:49-95, :224-233) for a sequence without conv history: the same arithmetic in
+ * the same order as hawk_conv1d_fwd (bf16 output) followed by hawk_gate_proj_fwd, bit for bit,
+ * without reading u back.  x [B,T,D] bf16, rows x_row_stride >= D elements apart (a multiple
+ * of 8: the x half of the block's input projection is read in place); u, x_rg_lru, a_rg_lru
+ * [B,T,D] bf16, dense; conv_w [4,D], conv_b [D] fp32; gate weights and biases as in
+ * hawk_gate_proj_fwd.  temporal_width must be 4 and T >= 32 (HAWK_ERR_BAD_SHAPE otherwise; use
+ * the two separate calls then). */
+int hawk_conv_gate_proj_fwd(const void* x, long long x_row_stride, const float* conv_w,
+                            const float* conv_b, const void* w_i, const float* b_i, const void* w_a,
+                            const float* b_a, void* u, void* x_rg_lru, void* a_rg_lru, int B, int T,
+                            int D, int num_blocks, int temporal_width, int w_dtype, void* stream);
 
 /* Gradient of the two projections with respect to x, in one pass over both logit gradients:
  *   dx[m, h*bw+i] = sum_j d_x_rg_lru[m, h*bw+j] w_i[h, i, j] + sum_j d_a_rg_lru[m, h*bw+j] w_a[h, i, j]

@@ -126,6 +126,34 @@ def conv_bwd(gy, x, w):
     return dx, dw, db
 
 
+def conv_fwd_strided(x, w, b, y, state=None):
+    """x, y: [B,T,D] views with unit channel stride and evenly spaced rows; y is written in place."""
+    B, T, D = x.shape
+    assert x.stride(2) == 1 and y.stride(2) == 1 and x.stride(0) == T * x.stride(1) and y.stride(0) == T * y.stride(1)
+    rc = _lib.load().hawk_conv1d_fwd_strided(
+        x.data_ptr(), x.stride(1), w.data_ptr(), b.data_ptr(), None if state is None else state.data_ptr(),
+        y.data_ptr(), y.stride(1), B, T, D, w.shape[0], _lib.dtype_code(x.dtype), _lib.dtype_code(y.dtype), _stream())
+    _lib.check("hawk_conv1d_fwd_strided", rc)
+    return y
+
+
+def conv_bwd_strided(gy, x, w, dx):
+    """x, dx: [B,T,D] views with evenly spaced rows (dx is written in place); gy dense."""
+    B, T, D = x.shape
+    W = w.shape[0]
+    lib = _lib.load()
+    assert x.stride(2) == 1 and dx.stride(2) == 1 and x.stride(0) == T * x.stride(1) and dx.stride(0) == T * dx.stride(1)
+    dw = torch.empty((W, D), dtype=torch.float32, device="cuda")
+    db = torch.empty((D,), dtype=torch.float32, device="cuda")
+    n = lib.hawk_conv1d_bwd_workspace_bytes(B, T, D, W)
+    ws = torch.empty(n, dtype=torch.uint8, device="cuda")
+    rc = lib.hawk_conv1d_bwd_strided(
+        gy.data_ptr(), x.data_ptr(), x.stride(1), w.data_ptr(), dx.data_ptr(), dx.stride(1), dw.data_ptr(),
+        db.data_ptr(), B, T, D, W, _lib.dtype_code(x.dtype), _lib.dtype_code(gy.dtype), ws.data_ptr(), n, _stream())
+    _lib.check("hawk_conv1d_bwd_strided", rc)
+    return dw, db
+
+
 def conv_step(state, x_new, w, b, y_dtype=None):
     B, D = x_new.shape
     W = w.shape[0]
@@ -214,6 +242,21 @@ def gate_proj_fwd(x, w_i, b_i, w_a, b_a, out_dtype=None):
         M, D, nb, _lib.dtype_code(x.dtype), _lib.dtype_code(w_i.dtype), _lib.dtype_code(out_dtype), _stream())
     _lib.check("hawk_gate_proj_fwd", rc)
     return oi, oa
+
+
+def conv_gate_proj_fwd(x, conv_w, conv_b, w_i, b_i, w_a, b_a):
+    """x [B,T,D] bf16 with unit channel stride and dense batch/time (rows may be further apart
+    than D); returns the conv output and both logits, dense [B,T,D] bf16."""
+    B, T, D = x.shape
+    assert x.stride(2) == 1 and x.stride(0) == T * x.stride(1)
+    nb = w_i.shape[0]
+    u, oi, oa = (torch.empty((B, T, D), dtype=torch.bfloat16, device="cuda") for _ in range(3))
+    rc = _lib.load().hawk_conv_gate_proj_fwd(
+        x.data_ptr(), x.stride(1), conv_w.data_ptr(), conv_b.data_ptr(), w_i.data_ptr(), _lib.ptr(b_i),
+        w_a.data_ptr(), _lib.ptr(b_a), u.data_ptr(), oi.data_ptr(), oa.data_ptr(), B, T, D, nb, conv_w.shape[0],
+        _lib.dtype_code(w_i.dtype), _stream())
+    _lib.check("hawk_conv_gate_proj_fwd", rc)
+    return u, oi, oa
 
 
 def decode_core_step(conv_state, x_new, conv_w, conv_b, w_i, b_i, w_a, b_a, lam, y, state, ws=None):

@@ -89,3 +89,39 @@ def test_benchmark_shape_bf16():
     assert max_rel(capi.to_np(db), db_all.cpu().numpy()) < 1e-4
     dw_last = (gy.double() * x.double()).sum(dim=(0, 1))  # tap on the current row is w[W-1]
     assert max_rel(capi.to_np(dw[W - 1]), dw_last.cpu().numpy()) < 1e-4
+
+
+# ---------------------------------------------------------------------------------------
+# Rows further apart than D: one half of a [B,T,2D] tensor read and written in place.
+# ---------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+@pytest.mark.parametrize("B,T,D,W,pad", [(2, 70, 128, 4, 128), (3, 33, 260, 4, 4), (1, 200, 100, 4, 2),
+                                         (2, 50, 63, 4, 1), (2, 40, 96, 3, 96), (1, 17, 64, 8, 8)])
+def test_strided_rows_give_the_bits_of_the_dense_call(B, T, D, W, pad, dtype):
+    rng = np.random.default_rng(B * 100 + T)
+    wide = capi.to_dev(rng.standard_normal((B, T, D + pad)), dtype)
+    x = wide[..., :D]
+    gy = capi.to_dev(rng.standard_normal((B, T, D)), dtype)
+    w, b = capi.to_dev(rng.standard_normal((W, D)) * 0.5, "f32"), capi.to_dev(rng.standard_normal(D) * 0.1, "f32")
+    y_ref = capi.conv_fwd(x.contiguous(), w, b)
+    dx_ref, dw_ref, db_ref = capi.conv_bwd(gy, x.contiguous(), w)
+    # outputs into the first D columns of a wider tensor whose other columns must stay as they are
+    out_wide = torch.full((B, T, D + pad), 7.0, dtype=x.dtype, device="cuda")
+    capi.conv_fwd_strided(x, w, b, out_wide[..., :D])
+    dx_wide = torch.full((B, T, D + pad), 7.0, dtype=x.dtype, device="cuda")
+    dw, db = capi.conv_bwd_strided(gy, x, w, dx_wide[..., :D])
+    torch.cuda.synchronize()
+    assert torch.equal(out_wide[..., :D], y_ref) and bool((out_wide[..., D:] == 7.0).all())
+    assert torch.equal(dx_wide[..., :D], dx_ref) and bool((dx_wide[..., D:] == 7.0).all())
+    assert torch.equal(dw, dw_ref) and torch.equal(db, db_ref)
+
+
+def test_strided_rows_refuse_a_stride_below_the_channel_count():
+    from hawk_pytorch_amd import _lib
+
+    x = torch.zeros(1, 8, 64, device="cuda")
+    w, b = torch.zeros(4, 64, device="cuda"), torch.zeros(64, device="cuda")
+    lib = _lib.load()
+    rc = lib.hawk_conv1d_fwd_strided(x.data_ptr(), 32, w.data_ptr(), b.data_ptr(), None, x.data_ptr(), 64, 1, 8, 64, 4,
+                                     1, 1, None)
+    assert rc == _lib.HAWK_ERR_BAD_SHAPE

@@ -225,3 +225,53 @@ def test_input_gradient_adds_the_addend_also_in_place():
     buf = add.clone()
     same = capi.gate_proj_bwd_input(gi, ga, wi, wa, torch.bfloat16, addend=buf, in_place=True)
     assert same.data_ptr() == buf.data_ptr() and torch.equal(buf, got)
+
+
+# ---------------------------------------------------------------------------------------
+# The forward with the temporal conv in front: same bits as the two separate calls.
+# ---------------------------------------------------------------------------------------
+def _conv_gate_case(B, T, D, nb, w_dtype, strided, seed):
+    rng = np.random.default_rng(seed)
+    bw = D // nb
+    xy = capi.to_dev(rng.standard_normal((B, T, 2 * D if strided else D)), "bf16")
+    x = xy[..., :D]
+    cw = capi.to_dev(rng.standard_normal((4, D)) * 0.5, "f32")
+    cb = capi.to_dev(rng.standard_normal(D) * 0.1, "f32")
+    wi = capi.to_dev(rng.standard_normal((nb, bw, bw)) / np.sqrt(bw), w_dtype)
+    wa = capi.to_dev(rng.standard_normal((nb, bw, bw)) / np.sqrt(bw), w_dtype)
+    bi, ba = capi.to_dev(rng.standard_normal(D), "f32"), capi.to_dev(rng.standard_normal(D), "f32")
+    u, oi, oa = capi.conv_gate_proj_fwd(x, cw, cb, wi, bi, wa, ba)
+    u_ref = capi.conv_fwd(x.contiguous(), cw, cb, y_dtype=torch.bfloat16)
+    oi_ref, oa_ref = capi.gate_proj_fwd(u_ref.reshape(B * T, D), wi, bi, wa, ba, torch.bfloat16)
+    torch.cuda.synchronize()
+    assert torch.equal(u, u_ref), ("conv output", B, T, D, nb)
+    assert torch.equal(oi.reshape(B * T, D), oi_ref), ("x_rg_lru", B, T, D, nb)
+    assert torch.equal(oa.reshape(B * T, D), oa_ref), ("a_rg_lru", B, T, D, nb)
+    # and the conv itself against the oracle (the separate kernel has its own tests; this pins
+    # the masking of rows before each sequence's first one)
+    ref = oracle.conv1d_fwd(capi.to_np(x).astype(np.float64), capi.to_np(cw).astype(np.float64),
+                            capi.to_np(cb).astype(np.float64))
+    assert max_rel(capi.to_np(u), ref) < 2e-2
+
+
+@pytest.mark.parametrize("B,T,D,nb", [(1, 32, 256, 1), (2, 33, 256, 1), (3, 100, 512, 4), (2, 77, 2560, 10),
+                                      (5, 45, 96, 3), (1, 4096, 512, 16), (4, 64, 768, 3), (7, 37, 384, 3)])
+@pytest.mark.parametrize("strided", [False, True])
+def test_conv_in_front_gives_the_bits_of_the_two_calls(B, T, D, nb, strided):
+    _conv_gate_case(B, T, D, nb, "bf16", strided, seed=B * 1000 + T)
+
+
+def test_conv_in_front_with_fp32_weights_and_many_tiles_per_workgroup():
+    _conv_gate_case(8, 1111, 2560, 10, "f32", True, seed=11)
+    _conv_gate_case(2, 4096 + 5, 1024, 4, "f32", False, seed=12)
+
+
+def test_conv_in_front_refuses_what_it_does_not_serve():
+    x = torch.zeros(1, 16, 256, dtype=torch.bfloat16, device="cuda")
+    cw, cb = torch.zeros(4, 256, device="cuda"), torch.zeros(256, device="cuda")
+    w = torch.zeros(1, 256, 256, dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(Exception, match="status 2"):
+        capi.conv_gate_proj_fwd(x, cw, cb, w, None, w, None)                      # T < 32
+    x = torch.zeros(1, 64, 256, dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(Exception, match="status 2"):
+        capi.conv_gate_proj_fwd(x, torch.zeros(3, 256, device="cuda"), cb, w, None, w, None)   # width 3

@@ -652,6 +652,64 @@ def test_recurrent_core_matches_its_parts():
     assert torch.equal(got[0], want[0])  # the forward is the very same pair of kernels
 
 
+@pytest.mark.parametrize("B,T,D,nb,W", [(2, 300, 512, 4, 4), (3, 77, 256, 1, 4), (2, 20, 512, 16, 4), (2, 64, 384, 3, 3)])
+def test_block_core_matches_its_parts_bit_for_bit(B, T, D, nb, W):
+    """conv + projections + scan + gate as one autograd node on the input projection's output
+    (both halves read in place, its gradient written as one tensor) against conv and
+    recurrent_core as separate nodes on chunked views: the same kernels on the same values."""
+    torch.manual_seed(13)
+    gi = hk.BlockDiagonalLinear(D, nb).cuda()
+    ga = hk.BlockDiagonalLinear(D, nb).cuda()
+    conv = hk.Conv1D(width=D, temporal_width=W).cuda()
+    with torch.no_grad():
+        gi.b.normal_()
+        ga.b.normal_()
+        conv.b.normal_(std=0.1)
+    lam = torch.nn.Parameter(torch.tensor(make_scan_inputs(1, 1, D, seed=1)[3], device="cuda", dtype=torch.float32))
+    xy = torch.randn(B, T, 2 * D, device="cuda").to(torch.bfloat16).requires_grad_(True)
+    go = torch.randn(B, T, D, device="cuda").to(torch.bfloat16)
+    params = (xy, lam, gi.w, gi.b, ga.w, ga.b, conv.w, conv.b)
+
+    def run(fn):
+        for p in params:
+            p.grad = None
+        with torch.autocast(device_type="cuda", dtype=torch.bfloat16):
+            out, last = fn()
+        out.backward(go)
+        return (out.detach(), last.detach(), *(p.grad.detach().clone() for p in params))
+
+    def parts():
+        x, y = xy.chunk(2, dim=-1)
+        u = hk.temporal_conv1d(x, conv.w, conv.b, torch.bfloat16)
+        return hk.recurrent_core(u, gi, ga, lam, y, return_last_state=True)
+
+    got = run(lambda: hk.recurrent_block_core(xy, conv, gi, ga, lam, return_last_state=True))
+    want = run(parts)
+    names = ("out", "h_last", "d_xy", "dLambda", "dw_i", "db_i", "dw_a", "db_a", "dconv_w", "dconv_b")
+    for name, a, b in zip(names, got, want):
+        assert a.shape == b.shape and a.dtype == b.dtype, name
+        assert torch.equal(a, b), (name, max_rel(capi.to_np(a), capi.to_np(b)))
+
+
+def test_model_uses_the_block_core_and_agrees_with_the_separate_nodes():
+    cfg = dict(vocab_size=512, hidden_size=256, intermediate_size=512, num_hidden_layers=2, recurrent_size=256,
+               num_blocks=4)
+    torch.manual_seed(3)
+    model = hk.HawkModel(hk.HawkConfig(**cfg)).cuda()
+    other = hk.HawkModel(hk.HawkConfig(fused_block_core=False, **cfg)).cuda()
+    other.load_state_dict(model.state_dict())
+    ids = torch.randint(1, 512, (2, 96), device="cuda")
+    losses = []
+    for m in (model, other):
+        with torch.autocast(device_type="cuda", dtype=torch.bfloat16):
+            loss = m(ids, ids)
+        loss.backward()
+        losses.append(loss.item())
+    assert losses[0] == losses[1]
+    for (n, p), (_, q) in zip(model.named_parameters(), other.named_parameters()):
+        assert max_rel(capi.to_np(p.grad), capi.to_np(q.grad)) < 1e-3, n
+
+
 def test_rounding_fp32_gate_weights_once_per_forward_changes_no_bit():
     """From 8192 rows on the host hands the projection kernels bf16 copies of fp32 weights
     instead of letting every workgroup round them: outputs and all gradients must be the same."""

@@ -296,6 +296,37 @@ def test_argument_validation_of_the_gated_and_projection_entry_points():
     assert lib.hawk_gate_proj_bwd_weights_workspace_bytes(32768, 2560, 7) == 0
 
 
+def test_argument_validation_of_the_conv_front_and_the_strided_conv():
+    lib = _lib.load()
+    E = _lib
+    p = 4096  # never dereferenced: every call below is refused before a launch
+    ok = [p, 512, p, p, p, None, p, None, p, p, p, 2, 64, 256, 1, 4, 0, None]
+    bad = list(ok); bad[12] = 31          # T < 32
+    assert lib.hawk_conv_gate_proj_fwd(*bad) == E.HAWK_ERR_BAD_SHAPE
+    bad = list(ok); bad[15] = 3           # temporal width other than 4
+    assert lib.hawk_conv_gate_proj_fwd(*bad) == E.HAWK_ERR_BAD_SHAPE
+    bad = list(ok); bad[1] = 255          # rows closer together than D
+    assert lib.hawk_conv_gate_proj_fwd(*bad) == E.HAWK_ERR_BAD_SHAPE
+    bad = list(ok); bad[1] = 260          # row stride not a multiple of 8
+    assert lib.hawk_conv_gate_proj_fwd(*bad) == E.HAWK_ERR_BAD_SHAPE
+    bad = list(ok); bad[14] = 3           # block width 256 / 3
+    assert lib.hawk_conv_gate_proj_fwd(*bad) == E.HAWK_ERR_BAD_SHAPE
+    bad = list(ok); bad[8] = None         # no conv output
+    assert lib.hawk_conv_gate_proj_fwd(*bad) == E.HAWK_ERR_NULL_POINTER
+    bad = list(ok); bad[0] = p + 2
+    assert lib.hawk_conv_gate_proj_fwd(*bad) == E.HAWK_ERR_ALIGNMENT
+    bad = list(ok); bad[16] = 5
+    assert lib.hawk_conv_gate_proj_fwd(*bad) == E.HAWK_ERR_BAD_DTYPE
+    # strided conv: strides below D or above 2^24 elements
+    assert lib.hawk_conv1d_fwd_strided(p, 63, p, p, None, p, 64, 1, 8, 64, 4, 0, 0, None) == E.HAWK_ERR_BAD_SHAPE
+    assert lib.hawk_conv1d_fwd_strided(p, 64, p, p, None, p, (1 << 24) + 1, 1, 8, 64, 4, 0, 0, None) \
+        == E.HAWK_ERR_BAD_SHAPE
+    assert lib.hawk_conv1d_bwd_strided(p, p, 64, p, p, 32, p, p, 1, 8, 64, 4, 0, 0, p, 1 << 20, None) \
+        == E.HAWK_ERR_BAD_SHAPE
+    assert lib.hawk_conv1d_bwd_strided(p, p, 64, p, p, 128, p, p, 1, 8, 64, 4, 0, 0, None, 0, None) \
+        == E.HAWK_ERR_WORKSPACE
+
+
 def test_argument_validation_of_the_fused_decode_step():
     lib = _lib.load()
     buf = (ctypes.c_char * 4096)()
