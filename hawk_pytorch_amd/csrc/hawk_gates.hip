@@ -275,29 +275,25 @@ __global__ __launch_bounds__(kGateThreads, 1) void gate_proj_fwd_kernel(
         if (t >= cf.T) t -= cf.T;
         const unsigned char* src = sR + buf * kRTileBytes + lrow * kARowBytes + lc8 * 16;
         const float* cw = sCW + lc8 * 8;
-        float acc[8];
-        {
-            const f32x4 b0 = *reinterpret_cast<const f32x4*>(cw + kConvTaps * kGroup);
-            const f32x4 b1 = *reinterpret_cast<const f32x4*>(cw + kConvTaps * kGroup + 4);
+        // four channels at a time: the weights of the matrix products leave few registers
+        u32x4 o;
 #pragma unroll
-            for (int e = 0; e < 4; ++e) acc[e] = b0[e], acc[4 + e] = b1[e];
-        }
+        for (int hf = 0; hf < 2; ++hf) {
+            const f32x4 b4 = *reinterpret_cast<const f32x4*>(cw + kConvTaps * kGroup + 4 * hf);
+            float acc[4] = {b4[0], b4[1], b4[2], b4[3]};
 #pragma unroll
-        for (int k = 0; k < kConvTaps; ++k) {
-            u32x4 v = *reinterpret_cast<const u32x4*>(src + k * kARowBytes);   // row t - (3 - k)
-            if (t < kConvTaps - 1 - k) v = u32x4{0u, 0u, 0u, 0u};             // before the sequence starts
-            const f32x4 w0 = *reinterpret_cast<const f32x4*>(cw + k * kGroup);
-            const f32x4 w1 = *reinterpret_cast<const f32x4*>(cw + k * kGroup + 4);
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const float lo = (e & 1) ? bf16_hi(v[e / 2]) : bf16_lo(v[e / 2]);
-                const float hi = (e & 1) ? bf16_hi(v[2 + e / 2]) : bf16_lo(v[2 + e / 2]);
-                acc[e] = fmaf(w0[e], lo, acc[e]);
-                acc[4 + e] = fmaf(w1[e], hi, acc[4 + e]);
+            for (int k = 0; k < kConvTaps; ++k) {
+                u32x2 v = *reinterpret_cast<const u32x2*>(src + k * kARowBytes + 8 * hf);   // row t - (3 - k)
+                if (t < kConvTaps - 1 - k) v = u32x2{0u, 0u};                               // before the sequence starts
+                const f32x4 w4 = *reinterpret_cast<const f32x4*>(cw + k * kGroup + 4 * hf);
+                acc[0] = fmaf(w4[0], bf16_lo(v.x), acc[0]);
+                acc[1] = fmaf(w4[1], bf16_hi(v.x), acc[1]);
+                acc[2] = fmaf(w4[2], bf16_lo(v.y), acc[2]);
+                acc[3] = fmaf(w4[3], bf16_hi(v.y), acc[3]);
             }
+            o[2 * hf] = pack_bf16x2(acc[0], acc[1]);
+            o[2 * hf + 1] = pack_bf16x2(acc[2], acc[3]);
         }
-        const u32x4 o = {pack_bf16x2(acc[0], acc[1]), pack_bf16x2(acc[2], acc[3]), pack_bf16x2(acc[4], acc[5]),
-                         pack_bf16x2(acc[6], acc[7])};
         *reinterpret_cast<u32x4*>(sA + buf * kATileBytes + lrow * kARowBytes + lc8 * 16) = o;
         const int row = row0 + lrow;
         if (row < M && col_ok)
@@ -440,6 +436,8 @@ __global__ __launch_bounds__(kGateThreads, 1) void gate_proj_fwd_kernel(
                 __builtin_nontemporal_store(va, reinterpret_cast<u32x4*>(out_a + (size_t)row * D + ocol));
             }
         }
+        // (issued behind the matrix products instead, the conv spills and the kernel takes 194 us
+        // against 150 us at 32768 rows of 2560 channels)
         if constexpr (CONV) conv_tile(it + 1, cur ^ 1);
         __syncthreads();
     };
