@@ -29,9 +29,10 @@ The kernel workloads (scan*, long, gates, block) run ``--settle-steps`` untimed 
 before the ``--warmup`` ones: for about 50 steps (20 ms) after the GPU leaves idle the same kernels
 run up to 12 % slower than they do from then on.
 
-The default workload's line also carries, under "also", records for the long-context and the
-scan + conv configurations, timed after the headline region in the same process (``--no-also``
-leaves them out).
+The default workload's line also carries, under "also", records for the long-context, the
+scan + conv and the gated-scan configurations, the gate projections, the recurrent core of one
+layer and the decode step, timed after the headline region in the same process with a quarter of the steps
+(``--no-also`` leaves them out).
 
 Prints one JSON line:
   value        tokens/s = B*T / (wall time per step), whole job on one GPU
@@ -262,7 +263,7 @@ def run_gates(args, lib, dev):
                            "TFLOPs": flops[i] / (ms[i] * 1e-3) / 1e12}
                     for i, name in enumerate(("fwd", "bwd_input", "bwd_weights"))},
     }
-    print(json.dumps(out))
+    return out
 
 
 def run_block(args, lib, dev):
@@ -355,7 +356,7 @@ def run_block(args, lib, dev):
     # gate dx 4, gate dw 3, conv 3
     fwd_bytes, bwd_bytes = (11 if args.unfused_conv else 10) * 2 * N, 20 * 2 * N
     step_gbs = (fwd_bytes + bwd_bytes) / (ms_per_step * 1e-3) / 1e9
-    print(json.dumps({
+    return {
         "metric": "Hawk recurrent core (conv, gate projections, gated scan) fwd+bwd tokens/s, 1 GPU",
         "value": B * T / (ms_per_step * 1e-3), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "settle_steps": args.settle_steps, "ms_per_step": ms_per_step,
@@ -369,7 +370,7 @@ def run_block(args, lib, dev):
                      "algorithmic_bytes_per_launch": fwd_bytes + bwd_bytes},
         "fwd": {"ms": fwd_ms, "GBs": fwd_bytes / (fwd_ms * 1e-3) / 1e9},
         "bwd": {"ms": bwd_ms, "GBs": bwd_bytes / (bwd_ms * 1e-3) / 1e9},
-    }))
+    }
 
 
 def run_model(args, lib, dev):
@@ -444,7 +445,7 @@ def run_model(args, lib, dev):
     nodes_ms, nodes_loss = time_steps(fused_block_core=False)
     plain_ms, plain_loss = time_steps(fused_gates=False, fused_epilogue=False)
     graph_ms, graph_loss = time_graph_steps()
-    print(json.dumps({
+    return {
         "metric": "Hawk training step tokens/s (README model, batch 1 x 2048, bf16 autocast), 1 GPU",
         "value": B * T / (fused_ms * 1e-3), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": fused_ms, "higher_is_better": True, "scaling": "weak",
@@ -459,7 +460,7 @@ def run_model(args, lib, dev):
         "loss_after_last_step": {"fused": fused_loss, "separate_nodes": nodes_loss, "unfused": plain_loss,
                                  "hip_graph": graph_loss},
         "roofline": None,
-    }))
+    }
 
 
 def run_decode(args, lib, dev):
@@ -592,7 +593,7 @@ def run_decode(args, lib, dev):
             "algorithmic_bytes_per_launch": hot_bytes,
         },
     }
-    print(json.dumps(out_json))
+    return out_json
 
 
 def run_scan(args, lib, dev, name, steps, warmup, settle, calibration_copy=False):
@@ -812,17 +813,9 @@ def main():
     lib = _lib.load()
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    if args.workload == "decode":
-        run_decode(args, lib, dev)
-        return
-    if args.workload == "gates":
-        run_gates(args, lib, dev)
-        return
-    if args.workload == "model":
-        run_model(args, lib, dev)
-        return
-    if args.workload == "block":
-        run_block(args, lib, dev)
+    others = {"decode": run_decode, "gates": run_gates, "model": run_model, "block": run_block}
+    if args.workload in others:
+        print(json.dumps(others[args.workload](args, lib, dev)))
         return
     out = run_scan(args, lib, dev, args.workload, args.steps, args.warmup, args.settle_steps, args.calibration_copy)
     cpu_args = out.pop("_cpu_args")
@@ -830,12 +823,21 @@ def main():
         # the other scan configurations of the benchmark definition, timed after the headline
         # region in the same process (fewer steps; the GPU is already at its steady clocks)
         also = {}
-        for other in ("long", "scan_conv"):
+        few = argparse.Namespace(**vars(args))
+        few.steps, few.settle_steps, few.calibration_copy = max(20, args.steps // 4), max(10, args.settle_steps // 4), False
+        for other in ("long", "scan_conv", "scan_gated"):
             torch.cuda.empty_cache()
-            rec = run_scan(args, lib, dev, other, max(20, args.steps // 4), args.warmup, max(10, args.settle_steps // 4))
+            rec = run_scan(args, lib, dev, other, few.steps, args.warmup, few.settle_steps)
             rec.pop("_cpu_args")
             also[other] = {k: rec[k] for k in ("config", "value", "unit", "ms_per_step", "steps", "warmup",
                                                "settle_steps", "roofline", "fwd", "step_hbm")}
+        # the matrix-core gate projections and the recurrent core of one layer at the same shape, and
+        # one-token decode steps of the 26-layer model at batch 256
+        for other, fn in (("gates", run_gates), ("block", run_block), ("decode", run_decode)):
+            torch.cuda.empty_cache()
+            rec = fn(few, lib, dev)
+            also[other] = {k: rec[k] for k in rec if k not in ("metric", "n_gpus", "higher_is_better", "scaling",
+                                                              "vs_baseline", "dtype", "data")}
         out["also"] = also
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(*cpu_args, args.seed)
