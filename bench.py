@@ -200,15 +200,27 @@ def run_gates(args, lib, dev):
     ws = torch.empty(nws, dtype=torch.uint8, device=dev)
     stream = torch.cuda.current_stream(dev).cuda_stream
 
+    # As the Python host does from 8192 rows on, the fp32 weights are rounded to bf16 once per step
+    # (two small kernels, inside the step but outside the three brackets) instead of by every
+    # workgroup of both kernels that read them; --fp32-gate-weights hands the kernels the fp32 ones.
+    wi16, wa16 = torch.empty_like(wi, dtype=bf), torch.empty_like(wa, dtype=bf)
+    cast = not args.fp32_gate_weights
+    kwi, kwa, wcode = (wi16, wa16, code) if cast else (wi, wa, f32)
+
+    def round_weights():
+        if cast:
+            wi16.copy_(wi)
+            wa16.copy_(wa)
+
     def fwd():
         _lib.check("gate_proj_fwd", lib.hawk_gate_proj_fwd(
-            x.data_ptr(), wi.data_ptr(), bi.data_ptr(), wa.data_ptr(), ba.data_ptr(), oi.data_ptr(), oa.data_ptr(),
-            M, D, nb, code, f32, code, stream))
+            x.data_ptr(), kwi.data_ptr(), bi.data_ptr(), kwa.data_ptr(), ba.data_ptr(), oi.data_ptr(), oa.data_ptr(),
+            M, D, nb, code, wcode, code, stream))
 
     def bwd_input():
         _lib.check("gate_proj_bwd_input", lib.hawk_gate_proj_bwd_input(
-            gi.data_ptr(), ga.data_ptr(), wi.data_ptr(), wa.data_ptr(), None, dx.data_ptr(), M, D, nb, code, f32, code,
-            stream))
+            gi.data_ptr(), ga.data_ptr(), kwi.data_ptr(), kwa.data_ptr(), None, dx.data_ptr(), M, D, nb, code, wcode,
+            code, stream))
 
     def bwd_weights():
         _lib.check("gate_proj_bwd_weights", lib.hawk_gate_proj_bwd_weights(
@@ -220,11 +232,12 @@ def run_gates(args, lib, dev):
             oi.copy_(x)
         torch.cuda.synchronize()
     for _ in range(args.settle_steps + args.warmup):
-        fwd(), bwd_input(), bwd_weights()
+        round_weights(), fwd(), bwd_input(), bwd_weights()
     torch.cuda.synchronize()
     ev = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(args.steps)]
     t0 = time.perf_counter()
     for k in range(args.steps):
+        round_weights()
         ev[k][0].record()
         fwd()
         ev[k][1].record()
@@ -251,7 +264,9 @@ def run_gates(args, lib, dev):
         "dtype": "bf16 operands, f32 accumulation",
         "data": f"synthetic, seed {args.seed}: activations and gradients ~ N(0,1), weights ~ N(0, 1/bw)",
         "config": {"workload": f"gates: both block-diagonal gate projections fwd + input grad + weight grads, "
-                               f"M={M}, D={D}, {nb} blocks of {bw}, bf16", "M": M, "D": D, "num_blocks": nb},
+                               f"M={M}, D={D}, {nb} blocks of {bw}, bf16, fp32 weights "
+                               + ("rounded to bf16 once per step" if cast else "rounded by every workgroup"),
+                   "M": M, "D": D, "num_blocks": nb},
         "roofline": {
             "bound": "hbm",
             "kernel": "gate_proj_bwd_weights_kernel (+ gate_proj_reduce_kernel, same launch call)",
@@ -778,6 +793,9 @@ def main():
     ap.add_argument("--settle-steps", type=int, default=100,
                     help="further untimed steps run before the warm-up in the kernel workloads (scan*, long, gates, "
                          "block): kernel durations settle about 50 steps (20 ms) after the GPU leaves idle")
+    ap.add_argument("--fp32-gate-weights", action="store_true",
+                    help="workload gates: hand the projection kernels the fp32 weights instead of rounding them "
+                         "to bf16 once per step")
     ap.add_argument("--unfused-conv", action="store_true",
                     help="workload block: conv and gate projections as two launches on a copy of the x half of the "
                          "input projection, gradients into separate tensors, instead of one launch on the "
