@@ -584,8 +584,10 @@ __global__ __launch_bounds__(kSmallWaves* kWave, sizeof(XT) == 2 ? 4 : 2) void g
 // four times the compute units).  Every one of them needs the conv output of all the block's
 // channels, so each computes it from the window, but none rolls the window while reading: a
 // workgroup that has read it (its loads have returned) counts itself in on the (rows, block)
-// counter, and the one that counts in last, when no reader is left, rolls the window at the end
-// of its work and sets the counter back to zero for the next launch.
+// counter, and in the one that counts in last, when no reader is left, the waves that have no
+// matrix products to do roll the window while the others multiply, and set the counter back to
+// zero for the next launch.  (Rolling at the end of the workgroup's work instead put the rows'
+// round trip on the critical path.)
 // ---------------------------------------------------------------------------------------
 constexpr int kCoreWaves = 8;
 constexpr int kCoreMaxW = 8;
@@ -619,6 +621,7 @@ __global__ __launch_bounds__(kCoreWaves* kWave, 1) void decode_core_kernel(
     const int W = WC > 0 ? WC : W_runtime;
     static_assert(BW % 32 == 0 && BW <= 32 * kCoreWaves, "one wave per 32 output columns of a block");
     static_assert(NS >= 1 && (BW / NS) % 32 == 0, "whole 32-column slices per workgroup");
+    static_assert(NS == 1 || BW / NS / 32 < kCoreWaves, "a cut workgroup needs a wave without matrix products");
     constexpr int KS = BW / 16;
     constexpr int CW = BW / NS;       // output columns of the block that this workgroup produces
     constexpr int NT = CW / 32;
@@ -637,7 +640,9 @@ __global__ __launch_bounds__(kCoreWaves* kWave, 1) void decode_core_kernel(
     const int rt = pair - h * ntiles;
     const int c_first = part * CW;    // first of this workgroup's output columns within the block
     const bool computes = w < NT;
-    __shared__ uint32_t s_arrival;
+    __shared__ uint32_t s_arrival;           // this workgroup's place among the NS of its pair
+    constexpr uint32_t kNotArrived = 0xffffffffu;
+    if (NS > 1 && tid == 0) s_arrival = kNotArrived;   // visible after the barrier that ends the conv
 
     // This wave's slice of a weight matrix: thread -> (4 input channels, 8 consecutive output
     // columns).  Sixteen lanes take sixteen consecutive channel quads of one column octet (their
@@ -669,6 +674,35 @@ __global__ __launch_bounds__(kCoreWaves* kWave, 1) void decode_core_kernel(
         }
     };
     if (computes) fetch_weights(w_i);
+
+    // Everything the later steps read from memory and whose address is known now is asked for
+    // now, so that the kernel pays one memory round trip and not one per step: the recurrence's
+    // y and state rows (step 4), the biases of this wave's columns (step 3) and Lambda (step 2).
+    // (Not with fp32 weights: their raw rows fill the register file, and these would spill.)
+    constexpr bool kEarly = sizeof(WT) == 2;
+    typedef typename Raw<ST, 8>::type sraw8_t;
+    constexpr int kRecCH = CW / 8;
+    constexpr int kRecPerThread = (kTileRows * kRecCH + kCoreWaves * kWave - 1) / (kCoreWaves * kWave);
+    u32x4 early_y[kRecPerThread];
+    sraw8_t early_s[kRecPerThread];
+    if (kEarly && vec_io) {
+#pragma unroll
+        for (int q = 0; q < kRecPerThread; ++q) {
+            const int task = min(tid + q * kCoreWaves * kWave, kTileRows * kRecCH - 1);
+            const int rl = task / kRecCH, ch = c_first / 8 + (task - rl * kRecCH);
+            const int row = min(rt * kTileRows + rl, M - 1);
+            const int c = h * BW + ch * 8;
+            early_y[q] = load_raw<bf16_t, 8>(y + (size_t)row * ldy + c);
+            early_s[q] = load_raw<ST, 8>(state + (size_t)row * D + c);
+        }
+    }
+    float early_bias_i = 0.0f, early_bias_a = 0.0f;
+    if (computes) {
+        const int c_out = h * BW + c_first + w * 32 + (lane & 31);
+        if (b_i != nullptr) early_bias_i = b_i[c_out];
+        if (b_a != nullptr) early_bias_a = b_a[c_out];
+    }
+    const float early_lam = tid < BW ? lam[h * BW + tid] : 0.0f;
 
     // ---- 1. conv window roll + conv: 16-byte chunks of 8 channels
     {
@@ -745,7 +779,7 @@ __global__ __launch_bounds__(kCoreWaves* kWave, 1) void decode_core_kernel(
     const int col = lane & 31, khalf = 8 * (lane >> 5);
     // softplus(Lambda) of the block's channels, once per workgroup
     float* sSp = reinterpret_cast<float*>(core_smem + CoreLds<BW>::kBytes);
-    if (tid < BW) sSp[tid] = softplus_precise(lam[h * BW + tid]);
+    if (tid < BW) sSp[tid] = softplus_precise(early_lam);
     if (computes) {
         stage_weights();
         fetch_weights(w_a);
@@ -754,10 +788,61 @@ __global__ __launch_bounds__(kCoreWaves* kWave, 1) void decode_core_kernel(
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
     if constexpr (NS > 1) {
-        // every thread's window loads have returned (their values went to LDS before the
-        // barrier): this workgroup no longer reads the window
-        if (tid == (kCoreWaves - 1) * kWave && W > 1)   // a wave without matrix products to do
-            s_arrival = __hip_atomic_fetch_add(counters + pair, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        // Every thread's window loads have returned (their values went to LDS before the
+        // barrier): this workgroup no longer reads the window.  The waves without matrix products
+        // count it in, and in the workgroup that counts in last, when no reader is left anywhere,
+        // they roll the window while the other waves multiply.  They ask for the rows before they
+        // know the count, so that the loads travel together with the counter's round trip.
+        if (!computes && W > 1) {
+            constexpr int CH = BW / 8;
+            constexpr int kIdle = (kCoreWaves - NT) * kWave;
+            const int H = W - 1;
+            const int itid = tid - NT * kWave;
+            if (itid == 0) {
+                const uint32_t a = __hip_atomic_fetch_add(counters + pair, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_store(&s_arrival, a, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            }
+            // all of a thread's rows are asked for at once (one round trip, not one per task)
+            constexpr int kPerThread = (kTileRows * CH + kIdle - 1) / kIdle;
+            u32x4 win[kPerThread][kCoreMaxW - 1], newest[kPerThread];
+#pragma unroll
+            for (int q = 0; q < kPerThread; ++q) {
+                const int task = min(itid + q * kIdle, kTileRows * CH - 1);
+                const int rl = task / CH, ch = task - rl * CH;
+                const int row = min(rt * kTileRows + rl, M - 1);
+                const int c = h * BW + ch * 8;
+                const bf16_t* sb = conv_state + (size_t)row * H * D + c;
+#pragma unroll
+                for (int j = 1; j < kCoreMaxW - 1; ++j) {
+                    if (j < H) win[q][j] = *reinterpret_cast<const u32x4*>(sb + (size_t)j * D);
+                }
+                newest[q] = *reinterpret_cast<const u32x4*>(x_new + (size_t)row * ldx + c);
+            }
+            uint32_t arrived = kNotArrived;
+            while (arrived == kNotArrived) {
+                arrived = __hip_atomic_load(&s_arrival, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                if (arrived == kNotArrived) __builtin_amdgcn_s_sleep(1);
+            }
+            if (arrived == (uint32_t)(NS - 1)) {
+#pragma unroll
+                for (int q = 0; q < kPerThread; ++q) {
+                    const int task = itid + q * kIdle;
+                    const int rl = task / CH, ch = task - rl * CH;
+                    const int row = rt * kTileRows + rl;
+                    if (task < kTileRows * CH && row < M) {
+                        bf16_t* sb = conv_state + (size_t)row * H * D + h * BW + ch * 8;
+#pragma unroll
+                        for (int j = 0; j < kCoreMaxW - 1; ++j) {
+                            if (j + 1 < H) *reinterpret_cast<u32x4*>(sb + (size_t)j * D) = win[q][j + 1];
+                        }
+                        *reinterpret_cast<u32x4*>(sb + (size_t)(H - 1) * D) = newest[q];
+                    }
+                }
+            }
+            // every part has counted in: the counter can go back to zero for the next launch
+            if (itid == 0 && arrived == (uint32_t)(NS - 1))
+                __hip_atomic_store(counters + pair, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
     }
 
     f32x16 acc_i = {}, acc_a = {};
@@ -788,9 +873,7 @@ __global__ __launch_bounds__(kCoreWaves* kWave, 1) void decode_core_kernel(
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
     if (computes) {
-        const int c_out = h * BW + c_first + w * 32 + col;
-        const float bias_i = b_i != nullptr ? b_i[c_out] : 0.0f;
-        const float bias_a = b_a != nullptr ? b_a[c_out] : 0.0f;
+        const float bias_i = early_bias_i, bias_a = early_bias_a;
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
             const int rl = 4 * (lane >> 5) + 8 * (r / 4) + (r % 4);
@@ -805,9 +888,11 @@ __global__ __launch_bounds__(kCoreWaves* kWave, 1) void decode_core_kernel(
 
     // ---- 4. recurrence and output gate
     {
-        typedef typename Raw<ST, 8>::type sraw8_t;
         constexpr int CH = CW / 8;
-        for (int task = tid; task < kTileRows * CH; task += kCoreWaves * kWave) {
+#pragma unroll
+        for (int q = 0; q < kRecPerThread; ++q) {
+            const int task = tid + q * kCoreWaves * kWave;
+            if (task >= kTileRows * CH) break;
             const int rl = task / CH, ch = c_first / 8 + (task - rl * CH);
             const int row = rt * kTileRows + rl;
             if (row >= M) continue;
@@ -819,7 +904,10 @@ __global__ __launch_bounds__(kCoreWaves* kWave, 1) void decode_core_kernel(
             const bf16_t* yp = y + (size_t)row * ldy + c;
             ST* sp = state + (size_t)row * D + c;
             bf16_t* op = out + (size_t)row * D + c;
-            if (vec_io) {
+            if (kEarly && vec_io) {
+                unpack(early_y[q], fy);
+                unpack(early_s[q], so);
+            } else if (vec_io) {
                 unpack(load_raw<bf16_t, 8>(yp), fy);
                 unpack(load_raw<ST, 8>(sp), so);
             } else {
@@ -854,34 +942,6 @@ __global__ __launch_bounds__(kCoreWaves* kWave, 1) void decode_core_kernel(
                     *reinterpret_cast<uint16_t*>(op + v) = to_bf16_bits(go[v]);
                 }
             }
-        }
-    }
-
-    // ---- 5. the window roll, by the workgroup that counted in last (s_arrival was written
-    //         before the barriers of steps 3 and 4 and is read after them)
-    if constexpr (NS > 1) {
-        if (W > 1 && s_arrival == (uint32_t)(NS - 1)) {
-            constexpr int CH = BW / 8;
-            const int H = W - 1;
-            for (int task = tid; task < kTileRows * CH; task += kCoreWaves * kWave) {
-                const int rl = task / CH, ch = task - rl * CH;
-                const int row = rt * kTileRows + rl;
-                if (row >= M) continue;
-                const int c = h * BW + ch * 8;
-                bf16_t* sb = conv_state + (size_t)row * H * D + c;
-                u32x4 win[kCoreMaxW - 1];
-#pragma unroll
-                for (int j = 1; j < kCoreMaxW - 1; ++j) {
-                    if (j < H) win[j] = *reinterpret_cast<const u32x4*>(sb + (size_t)j * D);
-                }
-                const u32x4 newest = *reinterpret_cast<const u32x4*>(x_new + (size_t)row * ldx + c);
-#pragma unroll
-                for (int j = 0; j < kCoreMaxW - 1; ++j) {
-                    if (j + 1 < H) *reinterpret_cast<u32x4*>(sb + (size_t)j * D) = win[j + 1];
-                }
-                *reinterpret_cast<u32x4*>(sb + (size_t)(H - 1) * D) = newest;
-            }
-            if (tid == 0) __hip_atomic_store(counters + pair, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
     }
 }
