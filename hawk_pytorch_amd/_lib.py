@@ -66,6 +66,7 @@ SIGNATURES = {
     ),
     "hawk_conv1d_step": (_c_int, [_c_void_p] * 5 + [_c_int] * 5 + [_c_void_p]),
     "hawk_rglru_step": (_c_int, [_c_void_p] * 6 + [_c_int] * 4 + [_c_void_p]),
+    "hawk_stream_capture_id": (_c_int, [_c_void_p, ctypes.POINTER(ctypes.c_ulonglong)]),
     "hawk_gate_proj_supported": (_c_int, [_c_int, _c_int]),
     "hawk_decode_core_supported": (_c_int, [_c_int] * 3),
     "hawk_decode_core_step": (
@@ -209,13 +210,31 @@ def scan_workspace(dev: torch.device, nbytes: int) -> torch.Tensor:
 
 
 _decode_workspaces: dict = {}
+_decode_captured: dict = {}   # (device, stream, capture id) -> counters of launches recorded into that graph
+
+
+def _capture_id(dev: torch.device) -> int:
+    cid = ctypes.c_ulonglong(0)
+    with torch.cuda.device(dev):
+        check("hawk_stream_capture_id", load().hawk_stream_capture_id(stream_ptr(dev), ctypes.byref(cid)))
+    return cid.value
 
 
 def decode_workspace(dev: torch.device, nbytes: int) -> torch.Tensor:
     """Zeroed counters for hawk_decode_core_step_ws, one buffer per (device, stream); every call
-    leaves them zero, so all layers and steps on a stream share it."""
+    leaves them zero, so all layers and steps on a stream share it.  Launches recorded into a HIP
+    graph get one buffer per (device, stream, capture) from the graph's own memory, zeroed by one
+    fill kernel that is part of the graph."""
     if torch.cuda.is_current_stream_capturing():
-        return torch.zeros(max(nbytes, 4), dtype=torch.uint8, device=dev)  # the graph's own, zeroed by a fill kernel
+        key = (_device_index(dev), stream_ptr(dev), _capture_id(dev))
+        with _lock:
+            ws = _decode_captured.get(key)
+            if ws is None or ws.numel() < nbytes:
+                ws = torch.zeros(max(nbytes, 4096), dtype=torch.uint8, device=dev)
+                _decode_captured[key] = ws
+                while len(_decode_captured) > _MAX_CAPTURED:
+                    _decode_captured.pop(next(iter(_decode_captured)))
+        return ws
     key = (_device_index(dev), stream_ptr(dev))
     with _lock:
         ws = _decode_workspaces.get(key)
@@ -231,6 +250,7 @@ def release_workspaces() -> None:
         _workspaces.clear()
         _captured.clear()
         _decode_workspaces.clear()
+        _decode_captured.clear()
 
 
 def _flag_of(ws: torch.Tensor, dev: torch.device) -> int:

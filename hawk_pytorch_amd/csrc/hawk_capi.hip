@@ -35,6 +35,15 @@ extern "C" {
 
 int hawk_version(void) { return 100; }
 
+int hawk_stream_capture_id(void* stream, unsigned long long* id) {
+    if (!id) return HAWK_ERR_NULL_POINTER;
+    hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+    unsigned long long cid = 0;
+    if (hipStreamGetCaptureInfo(as_stream(stream), &status, &cid) != hipSuccess) return HAWK_ERR_LAUNCH;
+    *id = status == hipStreamCaptureStatusActive ? cid : 0ull;
+    return HAWK_OK;
+}
+
 const char* hawk_status_string(int status) {
     switch (status) {
         case HAWK_OK: return "ok";

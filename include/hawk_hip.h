@@ -48,6 +48,12 @@ typedef enum hawk_dtype {
 int hawk_version(void);
 const char* hawk_status_string(int status);
 
+/* *id <- the identifier of the graph capture `stream` is recording into, or 0 when it is not
+ * capturing (hipStreamGetCaptureInfo).  A host that hands launches a workspace can key one
+ * buffer per (stream, capture) with it: launches recorded on one stream replay in order, so they
+ * can share what eager launches on one stream share.  No upstream counterpart. */
+int hawk_stream_capture_id(void* stream, unsigned long long* id);
+
 /* ---------------------------------------------------------------------------------------
  * Scan workspace.  The scan passes carries between tiles through a caller-owned device
  * buffer.  Query its size for a problem shape, allocate it, zero it ONCE with

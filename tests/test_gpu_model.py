@@ -501,6 +501,68 @@ def test_captured_scans_own_their_workspace():
         assert torch.equal(hk.fused_linear_scan(x, xg, ag, lam), want_a)  # eager launches in between
 
 
+def test_decode_steps_replay_from_a_hip_graph_like_eager_ones():
+    """One decode step recorded into a HIP graph and replayed, with eager work and
+    synchronisations between the replays, against the same steps launched eagerly: logits and
+    both cache states after every step.  All layers' one-launch steps share one counter buffer
+    per capture, which every launch must leave zero."""
+    from hawk_pytorch_amd import _lib
+
+    torch.manual_seed(21)
+    cfg = hk.HawkConfig(vocab_size=384, hidden_size=512, intermediate_size=512, num_hidden_layers=3,
+                        recurrent_size=512, num_blocks=2)   # block width 256: the step is cut over workgroups
+    model = hk.HawkModel(cfg, use_cache=True).cuda().eval().bfloat16()
+    for layer in model.layers:
+        r = layer.recc
+        for p_ in (r.rg_lru_a_param, r.conv1d.w, r.conv1d.b, r.rg_lru_input_gate.b, r.rg_lru_a_gate.b):
+            p_.data = p_.data.float()
+        r.conv1d.out_dtype = torch.bfloat16
+        torch.nn.init.normal_(r.resid_proj.weight, std=0.05)
+    B, steps = 40, 4
+    prompt = torch.randint(1, cfg.vocab_size, (B, 48), device="cuda")
+    toks = torch.randint(1, cfg.vocab_size, (steps, B, 1), device="cuda")
+
+    def prefilled():
+        caches = model.new_cache(B)
+        with torch.no_grad(), torch.autocast(device_type="cuda", dtype=torch.bfloat16):
+            _, caches = model(prompt, layer_past=caches)
+        return caches
+
+    with torch.no_grad(), torch.autocast(device_type="cuda", dtype=torch.bfloat16):
+        eager_caches = prefilled()
+        want = []
+        for k in range(steps):
+            logits, eager_caches = model(toks[k], layer_past=eager_caches)
+            want.append((logits.clone(), [c.conv_state.clone() for c in eager_caches],
+                         [c.recc_state.clone() for c in eager_caches]))
+
+        caches = prefilled()
+        tok = toks[0].clone()
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):      # a warm-up step on throw-away caches, as graph capture asks for
+            model(tok, layer_past=prefilled())
+        torch.cuda.current_stream().wait_stream(side)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            static_logits, _ = model(tok, layer_past=caches)
+        captured = [ws for ws in _lib._decode_captured.values()]
+        assert len(captured) >= 1
+        for k in range(steps):
+            tok.copy_(toks[k])
+            graph.replay()
+            torch.cuda.synchronize()
+            junk = torch.randn(256, 256, device="cuda") @ torch.randn(256, 256, device="cuda")   # eager work between replays
+            torch.cuda.synchronize()
+            del junk
+            logits, conv_states, recc_states = want[k]
+            assert torch.equal(static_logits, logits), k
+            for c, cs, rs in zip(caches, conv_states, recc_states):
+                assert torch.equal(c.conv_state, cs) and torch.equal(c.recc_state, rs), k
+            for ws in captured:
+                assert int(ws.sum()) == 0, k
+
+
 def test_torch_compile_traces_the_ops_without_graph_breaks():
     (x, xg, ag), lam, gout = _leaves(1, 70, 64, "f32", seed=4)
     conv = hk.Conv1D(64, 4).cuda()
