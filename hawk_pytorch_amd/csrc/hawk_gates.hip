@@ -587,7 +587,8 @@ __global__ __launch_bounds__(kSmallWaves* kWave, sizeof(XT) == 2 ? 4 : 2) void g
 // counter, and in the one that counts in last, when no reader is left, the waves that have no
 // matrix products to do roll the window while the others multiply, and set the counter back to
 // zero for the next launch.  (Rolling at the end of the workgroup's work instead put the rows'
-// round trip on the critical path.)
+// round trip on the critical path.)  At a width of 256 and 10 blocks: 13.5 us at 256 rows with two
+// workgroups per block against 18.4 us with one, 8.8 against 17.4 us at 32 rows with four.
 // ---------------------------------------------------------------------------------------
 constexpr int kCoreWaves = 8;
 constexpr int kCoreMaxW = 8;
