@@ -31,7 +31,7 @@ run up to 12 % slower than they do from then on.
 
 The default workload's line also carries, under "also", records for the long-context, the
 scan + conv and the gated-scan configurations, the gate projections, the recurrent core of one
-layer and the decode step, timed after the headline region in the same process with a quarter of the steps
+layer, the decode step and the README model's training step, timed after the headline region in the same process with a quarter of the steps
 (``--no-also`` leaves them out).
 
 Prints one JSON line:
@@ -850,12 +850,12 @@ def main():
             also[other] = {k: rec[k] for k in ("config", "value", "unit", "ms_per_step", "steps", "warmup",
                                                "settle_steps", "roofline", "fwd", "step_hbm")}
         # the matrix-core gate projections and the recurrent core of one layer at the same shape, and
-        # one-token decode steps of the 26-layer model at batch 256
-        for other, fn in (("gates", run_gates), ("block", run_block), ("decode", run_decode)):
+        # one-token decode steps of the 26-layer model at batch 256, and training steps of the README model
+        for other, fn in (("gates", run_gates), ("block", run_block), ("decode", run_decode), ("model", run_model)):
             torch.cuda.empty_cache()
             rec = fn(few, lib, dev)
             also[other] = {k: rec[k] for k in rec if k not in ("metric", "n_gpus", "higher_is_better", "scaling",
-                                                              "vs_baseline", "dtype", "data")}
+                                                              "vs_baseline", "dtype", "data") and rec[k] is not None}
         out["also"] = also
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(*cpu_args, args.seed)
