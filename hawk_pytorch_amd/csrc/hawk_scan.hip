@@ -62,7 +62,22 @@ struct ScanWsPtrs {
     unsigned long long* agg_h; // [nseg][B][D] tile aggregate: state from zero
     float* dlam_part;          // [nseg][B][D] per-tile partial sums for dLambda
     int lookback;              // distance between checkpoints of the carry chain (power of two)
+    uint32_t div_tiles[2];     // ticket / (B * nct) and ... / nct by multiplication (FastDiv)
+    uint32_t div_nct[2];
 };
+
+// Division of a 32-bit number by a launch constant as a multiplication and two shifts
+// (Granlund and Montgomery's round-up method, exact for every 32-bit dividend): a tile's first
+// instructions after its ticket arrives are two such divisions, and nothing else can start
+// before them.  m = floor(2^32 (2^l - d) / d) + 1 with l = ceil(log2 d); l == 0 means d == 1.
+struct FastDiv {
+    uint32_t m, l;
+};
+__device__ __forceinline__ uint32_t fast_div(uint32_t n, uint32_t m, uint32_t l) {
+    if (l == 0u) return n;
+    const uint32_t t = __umulhi(n, m);
+    return (t + ((n - t) >> 1)) >> (l - 1u);
+}
 
 __device__ __forceinline__ void publish(unsigned long long* p, uint32_t tag, float v) {
     unsigned long long w = ((unsigned long long)tag << 32) | (unsigned long long)__float_as_uint(v);
@@ -413,9 +428,9 @@ __global__ __launch_bounds__(NW * kWave, HAWK_FWD_WAVES_PER_SIMD) void rglru_sca
     if (nseg > 1) take_ticket(ws.ctrl, (uint32_t)nseg * (uint32_t)B * (uint32_t)nct, s_ticket, ticket, tag);
 
     const int per_seg = B * nct;
-    const int seg = ticket / per_seg;
+    const int seg = (int)fast_div(ticket, ws.div_tiles[0], ws.div_tiles[1]);
     const int rem = ticket - seg * per_seg;
-    const int b = rem / nct;
+    const int b = (int)fast_div((uint32_t)rem, ws.div_nct[0], ws.div_nct[1]);
     const int ct = rem - b * nct;
     if (seg * TS + TS <= T)
         fwd_tile<IT, OT, V, TC, NW, PRECISE, true, GATED, STORE_H>(x, xg, ag, lam, h, gate, B, T, D, nseg, seg, b, ct,
@@ -696,10 +711,10 @@ __global__ __launch_bounds__(NW * kWave, HAWK_BWD_WAVES_PER_SIMD) void rglru_sca
     if (nseg > 1) take_ticket(ws.ctrl, (uint32_t)nseg * (uint32_t)B * (uint32_t)nct, s_ticket, ticket, tag);
 
     const int per_seg = B * nct;
-    const int pos = ticket / per_seg;  // chain position: 0 is the LAST time tile
+    const int pos = (int)fast_div(ticket, ws.div_tiles[0], ws.div_tiles[1]);  // chain position: 0 is the LAST time tile
     const int seg = nseg - 1 - pos;
     const int rem = ticket - pos * per_seg;
-    const int b = rem / nct;
+    const int b = (int)fast_div((uint32_t)rem, ws.div_nct[0], ws.div_nct[1]);
     const int ct = rem - b * nct;
     if (seg > 0 && seg * TS + TS <= T)
         bwd_tile<IT, ST, V, TC, NW, PRECISE, true, GATED>(x, xg, ag, lam, hs, gout, dx, dxg, dag, gate, B, T, D, nseg,
@@ -843,6 +858,18 @@ int lookback_for(int B, int nct) {
     return chains <= kFewChains ? kMaxLookback : (chains >= kManyChains ? HAWK_LOOKBACK_MANY : 4);
 #endif
 }
+FastDiv fast_div_for(uint32_t d) {
+    FastDiv f;
+    f.l = 0;
+    while ((1ull << f.l) < d) ++f.l;
+    f.m = (uint32_t)(((1ull << 32) * ((1ull << f.l) - d)) / d + 1);
+    return f;
+}
+void set_divisors(ScanWsPtrs& p, int B, int nct) {
+    const FastDiv a = fast_div_for((uint32_t)B * (uint32_t)nct), b = fast_div_for((uint32_t)nct);
+    p.div_tiles[0] = a.m, p.div_tiles[1] = a.l;
+    p.div_nct[0] = b.m, p.div_nct[1] = b.l;
+}
 ScanWsPtrs carve(void* ws, const WsLayout& l, int lookback) {
     char* p = static_cast<char*>(ws);
     ScanWsPtrs r;
@@ -914,10 +941,12 @@ int scan_fwd_impl(const void* x, const void* xg, const void* ag, const float* la
     const int nct = ceil_div(D, s.chans());
     ScanWsPtrs p = {};
     p.lookback = 4;
+    set_divisors(p, B, nct);
     if (nseg > 1) {
         const WsLayout l = layout_for(B, D, nseg, 0);
         if (ws == nullptr || ws_bytes < l.total) return HAWK_ERR_WORKSPACE;
         p = carve(ws, l, lookback_for(B, nct));
+        set_divisors(p, B, nct);
     }
     if (in_dtype == HAWK_DTYPE_BF16) {
         if (s.V == 2)
@@ -943,7 +972,8 @@ int scan_bwd_shaped(const void* x, const void* xg, const void* ag, const float* 
     const int nct = ceil_div(D, s.chans());
     const WsLayout l = layout_for(B, D, nseg, nseg);
     if (ws == nullptr || ws_bytes < l.total) return HAWK_ERR_WORKSPACE;
-    const ScanWsPtrs p = carve(ws, l, lookback_for(B, nct));
+    ScanWsPtrs p = carve(ws, l, lookback_for(B, nct));
+    set_divisors(p, B, nct);
     int rc;
     if (in_dtype == HAWK_DTYPE_BF16) {
         if (s.V == 2)
