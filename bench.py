@@ -39,7 +39,9 @@ Prints one JSON line:
   roofline     for the dominant kernel (the backward scan): algorithmic bytes per launch
                (16 B/element in bf16: five tensors read, three written) over the mean
                duration of the backward launch measured with HIP events on the launch
-               stream, against the 8 TB/s HBM peak
+               stream, against the 8 TB/s HBM peak; `traffic` is the launch's HBM bytes as
+               rocprofv3 counted them (profiles/hbm_traffic.json, while its digest matches the
+               kernel sources) and `traffic_frac` the same launch time against those bytes
   cpu_baseline the PyTorch CPU loop over time of the same recurrence (forward + autograd
                backward, fp32) on this host's cores, on a bounded sample of the workload
 """
@@ -742,6 +744,7 @@ def run_scan(args, lib, dev, name, steps, warmup, settle, calibration_copy=False
     step_bytes = fwd_bytes + bwd_bytes + (3 * elem * N if with_conv else 0)
     bwd_gbs = bwd_bytes / (bwd_ms * 1e-3) / 1e9
 
+    traffic = measured_traffic(name)
     out = {
         "metric": "RG-LRU scan fwd+bwd tokens/s and achieved HBM GB/s (% of peak), 1 GPU",
         "value": B * T / (ms_per_step * 1e-3),
@@ -772,7 +775,10 @@ def run_scan(args, lib, dev, name, steps, warmup, settle, calibration_copy=False
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": bwd_gbs / HBM_PEAK_GBS,
-            "traffic": measured_traffic(name),
+            "traffic": traffic,
+            # the same launch time against the HBM bytes rocprofv3 counted for this launch (the
+            # algorithmic bytes plus the carry words): what "achieved HBM bandwidth in rocprof" reads
+            "traffic_frac": None if traffic is None else traffic / (bwd_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
             "algorithmic_bytes_per_launch": bwd_bytes,
             "launch_ms": bwd_ms,
         },

@@ -45,3 +45,5 @@ def test_bench_prints_one_json_line_with_the_agreed_fields():
         assert d["also"][name]["roofline"]["frac"] > 0.2, name
     # a traffic figure is reported only when it was measured on the present kernel sources
     assert roof["traffic"] is None or roof["traffic"] > roof["algorithmic_bytes_per_launch"]
+    assert (roof["traffic_frac"] is None) == (roof["traffic"] is None)
+    assert roof["traffic_frac"] is None or roof["frac"] < roof["traffic_frac"] < 1.0
