@@ -493,8 +493,6 @@ def block_core_layout_ok(xy: torch.Tensor) -> bool:
 
 
 def _launch_block_core_fwd(xy, conv_w, conv_b, w_i, b_i, w_a, b_a, lam, want_h: bool, want_last: bool):
-    from .external import _gate_workspace  # noqa: F401  (deferred: external imports nothing from here)
-
     dev = _lib.require_cuda(xy, conv_w, conv_b, w_i, b_i, w_a, b_a, lam)
     if xy.data_ptr() % 16 != 0:
         xy = xy.clone(memory_format=torch.contiguous_format)
@@ -533,7 +531,7 @@ def _launch_block_core_fwd(xy, conv_w, conv_b, w_i, b_i, w_a, b_a, lam, want_h: 
 
 
 def _launch_block_core_bwd(xy, u, xg, ag, h, conv_w, w_i, w_a, lam, grad_out):
-    from .external import _gate_workspace
+    from .external import _gate_workspace  # deferred: external imports nothing from here
 
     dev = _lib.require_cuda(xy, u, xg, ag, h, conv_w, w_i, w_a, lam, grad_out)
     if xy.data_ptr() % 16 != 0:
