@@ -23,7 +23,17 @@ README model (vocabulary 32000, hidden = recurrent = 512, MLP 1024, 8 layers, 16
 on a 1 x 2048 batch under bf16 autocast, with and without the fused gate / epilogue kernels;
 ``--workload decode`` times one-token steps of a 26-layer Hawk (R = H = 2560, I = 7680,
 10 gate blocks, vocabulary 32000, bf16 weights) at batch 256 after a 1024-token prefill,
-eagerly and as a replayed HIP graph, plus the two hot-path kernels of a layer on their own.
+eagerly and as a replayed HIP graph, plus the one-launch recurrent core of a layer and token
+(hawk_decode_core_step_ws, the kernel the model launches) on its own.
+
+Timing.  The timed region of the kernel workloads holds nothing but the launches, between one
+event and one host clock reading on either side: `ms_per_step` and `value` come from it.  An
+event recorded between two launches makes the next dispatch wait behind a marker packet, 3-4 us
+each on this GPU, which no training loop pays; the per-launch durations that the `roofline`
+and `fwd` figures divide by are therefore measured on the same steps run once more, right behind
+the timed region, with a HIP event after every launch (`launch_timing_region`).
+`stream_ceiling` (default workload) times stock PyTorch streaming kernels with the forward's and
+the backward's read/write mix on the same tensors in the same process.
 
 The kernel workloads (scan*, long, gates, block) run ``--settle-steps`` untimed steps (default 100)
 before the ``--warmup`` ones: for about 50 steps (20 ms) after the GPU leaves idle the same kernels
@@ -236,8 +246,15 @@ def run_gates(args, lib, dev):
     for _ in range(args.settle_steps + args.warmup):
         round_weights(), fwd(), bwd_input(), bwd_weights()
     torch.cuda.synchronize()
-    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(args.steps)]
+    # timed region: the launches alone (an event between two launches costs the GPU 3-4 us)
     t0 = time.perf_counter()
+    for k in range(args.steps):
+        round_weights(), fwd(), bwd_input(), bwd_weights()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall * 1e3 / args.steps
+    # launch durations: the same steps again with an event after every launch
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(args.steps)]
     for k in range(args.steps):
         round_weights()
         ev[k][0].record()
@@ -248,9 +265,7 @@ def run_gates(args, lib, dev):
         bwd_weights()
         ev[k][3].record()
     torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
     ms = [float(np.mean([e[i].elapsed_time(e[i + 1]) for e in ev])) for i in range(3)]
-    ms_per_step = wall * 1e3 / args.steps
     N = M * D
     # forward: read x, write two logits; dx: read two gradients, write dx; dw: read x and two gradients
     alg = [3 * 2 * N, 3 * 2 * N, 3 * 2 * N]
@@ -353,8 +368,14 @@ def run_block(args, lib, dev):
     for _ in range(args.settle_steps + args.warmup):
         fwd(), bwd()
     torch.cuda.synchronize()
-    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
+    # timed region: the launches alone (an event between two launches costs the GPU 3-4 us)
     t0 = time.perf_counter()
+    for k in range(args.steps):
+        fwd(), bwd()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    # forward / backward split: the same steps again with events around both halves
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
     for k in range(args.steps):
         ev[k][0].record()
         fwd()
@@ -362,7 +383,6 @@ def run_block(args, lib, dev):
         bwd()
         ev[k][2].record()
     torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
     flag = ctypes.c_int(0)
     _lib.check("status", lib.hawk_scan_workspace_status(ws.data_ptr(), st, ctypes.byref(flag)))
     assert flag.value == 0 and bool(torch.isfinite((dxin if args.unfused_conv else dxy).float()).all())
@@ -449,7 +469,9 @@ def run_model(args, lib, dev):
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
             static_loss = step()
-        for _ in range(args.warmup):
+        # the three eager steps above count as warm-up, so that every leg has taken the same
+        # number of optimiser steps when its loss is read
+        for _ in range(max(args.warmup - 3, 0)):
             graph.replay()
         torch.cuda.synchronize()
         t0 = time.perf_counter()
@@ -476,6 +498,10 @@ def run_model(args, lib, dev):
         "tokens_per_s_as_hip_graph": B * T / (graph_ms * 1e-3),
         "loss_after_last_step": {"fused": fused_loss, "separate_nodes": nodes_loss, "unfused": plain_loss,
                                  "hip_graph": graph_loss},
+        "optimizer_steps_before_that_loss": {"fused": args.warmup + args.steps - 1,
+                                             "separate_nodes": args.warmup + args.steps - 1,
+                                             "unfused": args.warmup + args.steps - 1,
+                                             "hip_graph": max(args.warmup, 3) + args.steps - 1},
         "roofline": None,
     }
 
@@ -538,51 +564,75 @@ def run_decode(args, lib, dev):
         graph_ms = (time.perf_counter() - t0) * 1e3 / args.steps
         finite = bool(torch.isfinite(static_logits.float()).all())
 
-    # the two hot-path launches of one layer, through the C ABI
-    D, W = 2560, 4
+    # The recurrent core of one layer and token through the C ABI, as `Hawk.forward` launches it:
+    # hawk_decode_core_step_ws (window roll + conv, both gate projections, biases, recurrence,
+    # output gate, both cache updates, one launch), every layer with its own weights and caches.
+    D, W, nb, L = 2560, 4, 10, 26
+    bw = D // nb
     bf, code = torch.bfloat16, _lib.HAWK_DTYPE_BF16
-    conv_state = torch.randn(B, W - 1, D, device=dev).to(bf)
     xy = torch.randn(B, 2 * D, device=dev).to(bf)
-    xn, y = xy[:, :D].contiguous(), xy[:, D:]
     cw, cb = torch.randn(W, D, device=dev) * 0.5, torch.zeros(D, device=dev)
-    u, xg, ag = (torch.randn(B, D, device=dev).to(bf) for _ in range(3))
     bi, ba = torch.zeros(D, device=dev), torch.zeros(D, device=dev)
     lam = lambda_for_a8_range(torch.Generator().manual_seed(args.seed), D, 0.9, 0.999).to(dev)
-    state = torch.zeros(B, D, device=dev).to(bf)
     out = torch.empty(B, D, device=dev, dtype=bf)
-    def layer_hot_path():
+    per_layer = [dict(conv_state=torch.randn(B, W - 1, D, device=dev).to(bf),
+                      state=torch.zeros(B, D, device=dev).to(bf),
+                      w_i=(torch.randn(nb, bw, bw, device=dev) * bw ** -0.5).to(bf),
+                      w_a=(torch.randn(nb, bw, bw, device=dev) * bw ** -0.5).to(bf)) for _ in range(L)]
+    core_ws = torch.zeros(max(lib.hawk_decode_core_workspace_bytes(B, D, nb), 4), dtype=torch.uint8, device=dev)
+
+    def layer_core(p):
         stream = torch.cuda.current_stream(dev).cuda_stream
-        _lib.check("conv1d_step", lib.hawk_conv1d_step(conv_state.data_ptr(), xn.data_ptr(), cw.data_ptr(),
+        _lib.check("decode_core_step_ws", lib.hawk_decode_core_step_ws(
+            p["conv_state"].data_ptr(), xy.data_ptr(), 2 * D, cw.data_ptr(), cb.data_ptr(), p["w_i"].data_ptr(),
+            bi.data_ptr(), p["w_a"].data_ptr(), ba.data_ptr(), lam.data_ptr(), xy.data_ptr() + 2 * D, 2 * D,
+            p["state"].data_ptr(), out.data_ptr(), B, D, nb, W, code, code, code, core_ws.data_ptr(),
+            core_ws.numel(), stream))
+
+    # the two elementwise launches of the hot path alone (no projections), for comparison
+    xn, y = xy[:, :D].contiguous(), xy[:, D:]
+    u, xg, ag = (torch.randn(B, D, device=dev).to(bf) for _ in range(3))
+
+    def layer_two_launches(p):
+        stream = torch.cuda.current_stream(dev).cuda_stream
+        _lib.check("conv1d_step", lib.hawk_conv1d_step(p["conv_state"].data_ptr(), xn.data_ptr(), cw.data_ptr(),
                                                        cb.data_ptr(), u.data_ptr(), B, D, W, code, code, stream))
         _lib.check("rglru_step_gated", lib.hawk_rglru_step_gated(
             u.data_ptr(), xg.data_ptr(), ag.data_ptr(), bi.data_ptr(), ba.data_ptr(), lam.data_ptr(), y.data_ptr(),
-            2 * D, state.data_ptr(), None, out.data_ptr(), B, D, code, code, stream))
+            2 * D, p["state"].data_ptr(), None, out.data_ptr(), B, D, code, code, stream))
 
-    # 26 layers' worth of the two launches as one HIP graph, so that the figure is the GPU's
-    # time and not the host's launch rate
-    side = torch.cuda.Stream()
-    side.wait_stream(torch.cuda.current_stream())
-    with torch.cuda.stream(side):
-        layer_hot_path()
-    torch.cuda.current_stream().wait_stream(side)
-    hot_graph = torch.cuda.CUDAGraph()
-    with torch.cuda.graph(hot_graph):
-        for _ in range(26):
-            layer_hot_path()
-    for _ in range(5):
-        hot_graph.replay()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    n_rep = 40
-    e0.record()
-    for _ in range(n_rep):
-        hot_graph.replay()
-    e1.record()
-    torch.cuda.synchronize()
-    hot_us = e0.elapsed_time(e1) * 1e3 / (n_rep * 26)
-    # conv step: read 3 state rows + new row, write y and 3 rows; RG-LRU step: read u, two logits,
-    # state, y, write state and out  (bf16)
-    hot_bytes = (4 + 4 + 7) * 2 * B * D
+    def graph_us_per_layer_step(fn):
+        # 26 layers' launches as one HIP graph, so that the figure is the GPU's time and not the
+        # host's launch rate
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            fn(per_layer[0])
+        torch.cuda.current_stream().wait_stream(side)
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            for p in per_layer:
+                fn(p)
+        for _ in range(5):
+            g.replay()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        n_rep = 40
+        e0.record()
+        for _ in range(n_rep):
+            g.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e3 / (n_rep * L)
+
+    hot_us = graph_us_per_layer_step(layer_core)
+    two_us = graph_us_per_layer_step(layer_two_launches)
+    # core: conv window read and rewritten (3 + 3 rows), x_new, y, state read and written, out
+    # (bf16), both gates' weights (bf16) and the fp32 vectors (conv taps and bias, gate biases, Lambda)
+    hot_bytes = 11 * 2 * B * D + 2 * nb * bw * bw * 2 + (W + 4) * D * 4
     gbs = hot_bytes / (hot_us * 1e-6) / 1e9
+    # two launches: conv step reads 3 state rows + new row, writes y and 3 rows; RG-LRU step reads
+    # u, two logits, state, y, writes state and out  (bf16)
+    two_bytes = (4 + 4 + 7) * 2 * B * D
 
     out_json = {
         "metric": "decode tokens/s, batch 256, 1 GPU (whole model step; hot path reported beside it)",
@@ -605,9 +655,15 @@ def run_decode(args, lib, dev):
         "hot_path_us_per_layer_step": hot_us,
         "roofline": {
             "bound": "hbm",
-            "kernel": "conv1d_step_kernel + rglru_step_kernel (two launches per layer and token; launch-bound)",
+            "kernel": "decode_core_kernel via hawk_decode_core_step_ws (one launch per layer and token, the "
+                      "path Hawk.forward takes; each of the 26 layers has its own weights; launch-bound)",
             "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS, "traffic": None,
-            "algorithmic_bytes_per_launch": hot_bytes,
+            "algorithmic_bytes_per_launch": hot_bytes, "launch_us": hot_us,
+        },
+        "two_elementwise_launches": {
+            "kernel": "conv1d_step_kernel + rglru_step_kernel (no projections; two launches per layer and token)",
+            "us_per_layer_step": two_us, "algorithmic_bytes": two_bytes,
+            "GBs": two_bytes / (two_us * 1e-6) / 1e9,
         },
     }
     return out_json
@@ -707,12 +763,27 @@ def run_scan(args, lib, dev, name, steps, warmup, settle, calibration_copy=False
             conv_bwd()
     torch.cuda.synchronize()
 
-    # Two events per step bracket the backward launch; the forward launch of step k runs from the
-    # end of step k-1 (its last event, or the event after the conv backward) to the first event of
-    # step k.
+    # Timed region: `steps` steps, nothing but the launches between one event (and one host clock
+    # reading) before and one after.  An event recorded between two launches costs the GPU 3-4 us
+    # (a marker packet that the next dispatch waits behind), which a training loop does not pay.
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    start.record()
+    for k in range(steps):
+        fwd()
+        bwd()
+        if with_conv:
+            conv_bwd()
+    end.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    region_gpu_ms = start.elapsed_time(end)
+
+    # Launch durations: the same `steps` steps again, right behind the timed region, now with an
+    # event after every launch.  The forward launch of step k runs from the end of step k-1 (its
+    # last event) to the first event of step k; two events bracket the backward launch.
     ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3 if with_conv else 2)] for _ in range(steps)]
     start = torch.cuda.Event(enable_timing=True)
-    t0 = time.perf_counter()
     start.record()
     for k in range(steps):
         fwd()
@@ -723,7 +794,6 @@ def run_scan(args, lib, dev, name, steps, warmup, settle, calibration_copy=False
             conv_bwd()
             ev[k][2].record()
     torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
 
     flag = ctypes.c_int(0)
     _lib.check("status", lib.hawk_scan_workspace_status(ws.data_ptr(), stream, ctypes.byref(flag)))
@@ -735,6 +805,7 @@ def run_scan(args, lib, dev, name, steps, warmup, settle, calibration_copy=False
     fwd_ms = float(np.mean([step_end[k].elapsed_time(ev[k][0]) for k in range(steps)]))
     bwd_ms = float(np.mean([e[0].elapsed_time(e[1]) for e in ev]))
     ms_per_step = wall * 1e3 / steps
+    ms_per_step_with_events = step_end[0].elapsed_time(step_end[-1]) / steps
     elem = 2  # bytes per bf16 activation element
     # gated: the forward also reads y and writes out; the backward also reads y and writes dy
     fwd_bytes = (6 if gated else 4) * elem * N + (2 * elem * N if with_conv else 0)
@@ -764,9 +835,16 @@ def run_scan(args, lib, dev, name, steps, warmup, settle, calibration_copy=False
             "workload": f"{name}: RG-LRU scan"
                         + (" + temporal conv1d (W=4)" if with_conv else "")
                         + (" fused with out = gelu(y) * h" if gated else "")
-                        + f" fwd+bwd, B={B}, T={T}, D={D}, " + ("f32 in / bf16 state" if mixed else "bf16"),
+                        + f" fwd+bwd, B={B}, T={T}, D={D}, " + ("f32 in / bf16 state" if mixed else "bf16")
+                        + f"; {settle} + {warmup} untimed steps before the {steps} timed ones",
             "B": B, "T": T, "D": D,
         },
+        "timed_region": {"steps": steps, "host_ms": wall * 1e3, "gpu_ms_between_events": region_gpu_ms,
+                         "events_inside": 0},
+        "launch_timing_region": {"steps": steps, "events_per_step": 3 if with_conv else 2,
+                                 "ms_per_step": ms_per_step_with_events,
+                                 "note": "the same steps run again right behind the timed region with an event "
+                                         "after every launch; roofline and fwd come from here"},
         "roofline": {
             "bound": "hbm",
             "kernel": "rglru_scan_bwd_kernel" + (" (gated)" if gated else "")
@@ -788,7 +866,60 @@ def run_scan(args, lib, dev, name, steps, warmup, settle, calibration_copy=False
                      "frac": step_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS},
     }
     out["_cpu_args"] = (B, D, lo, hi)
+    out["_buffers"] = {"x": x, "xg": xg, "ag": ag, "h": h, "gout": gout, "dx": dx, "dxg": dxg, "dag": dag}
     return out
+
+
+def run_stream_ceiling(buf, steps, settle):
+    """Stock PyTorch streaming kernels on the scan's own operands, timed like the scan's launches.
+
+    What a plain elementwise kernel with the forward's and the backward's read/write mix reaches on
+    this box in this process: the scale against which the scan's GB/s can be read."""
+    x, xg, ag, h, gout, dx, dxg, dag = (buf[k] for k in ("x", "xg", "ag", "h", "gout", "dx", "dxg", "dag"))
+    nbytes = x.numel() * x.element_size()
+
+    def copy_1r1w():
+        h.copy_(x)
+
+    def addcmul_3r1w():
+        torch.addcmul(x, xg, ag, out=h)
+
+    def composition_5r3w():
+        torch.addcmul(x, xg, ag, out=dx)   # 3 reads, 1 write
+        torch.mul(h, gout, out=dxg)        # 2 reads, 1 write
+        dag.fill_(0.5)                     # 1 write
+
+    rec = {}
+    for name, fn, tensors, kernels in (("copy_1r1w", copy_1r1w, 2, 1), ("addcmul_3r1w", addcmul_3r1w, 4, 1),
+                                       ("composition_5r3w", composition_5r3w, 8, 3)):
+        for _ in range(settle):
+            fn()
+        torch.cuda.synchronize()
+        # per call, as the scan's launches are timed: an event after every call
+        ev = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
+        ev[0].record()
+        for k in range(steps):
+            fn()
+            ev[k + 1].record()
+        torch.cuda.synchronize()
+        with_events_ms = ev[0].elapsed_time(ev[-1]) / steps
+        # and back to back, as the timed region runs
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for k in range(steps):
+            fn()
+        b.record()
+        torch.cuda.synchronize()
+        ms = a.elapsed_time(b) / steps
+        moved = tensors * nbytes
+        rec[name] = {"kernels": kernels, "bytes": moved, "us": ms * 1e3, "GBs": moved / (ms * 1e-3) / 1e9,
+                     "frac": moved / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                     "us_with_an_event_per_call": with_events_ms * 1e3,
+                     "frac_with_an_event_per_call": moved / (with_events_ms * 1e-3) / 1e9 / HBM_PEAK_GBS}
+    rec["note"] = ("torch.Tensor.copy_, torch.addcmul(out=) and addcmul + mul + fill_ on the headline's x, x_rg_lru, "
+                   "a_rg_lru, h, grad_out and gradient tensors (bf16, %d MB each), %d settling calls, then %d timed "
+                   "calls; frac is of the 8 TB/s peak" % (nbytes // 1000000, settle, steps))
+    return rec
 
 
 def main():
@@ -843,6 +974,20 @@ def main():
         return
     out = run_scan(args, lib, dev, args.workload, args.steps, args.warmup, args.settle_steps, args.calibration_copy)
     cpu_args = out.pop("_cpu_args")
+    buffers = out.pop("_buffers")
+    if args.workload == "scan":
+        # the streaming ceiling of this box, in this process, on the same tensors
+        ceiling = run_stream_ceiling(buffers, max(20, args.steps // 4), max(10, args.settle_steps // 4))
+        ceiling["scan_fwd_over_addcmul_3r1w"] = (out["fwd"]["GBs"]
+                                                 / (ceiling["addcmul_3r1w"]["bytes"]
+                                                    / (ceiling["addcmul_3r1w"]["us_with_an_event_per_call"] * 1e-6) / 1e9))
+        ceiling["scan_bwd_over_composition_5r3w"] = (out["roofline"]["achieved"]
+                                                     / (ceiling["composition_5r3w"]["bytes"]
+                                                        / (ceiling["composition_5r3w"]["us_with_an_event_per_call"] * 1e-6) / 1e9))
+        ceiling["scan_step_over_both"] = ((ceiling["addcmul_3r1w"]["us"] + ceiling["composition_5r3w"]["us"]) * 1e-3
+                                          / out["ms_per_step"])
+        out["stream_ceiling"] = ceiling
+    del buffers
     if args.workload == "scan" and not args.no_also:
         # the other scan configurations of the benchmark definition, timed after the headline
         # region in the same process (fewer steps; the GPU is already at its steady clocks)
@@ -853,6 +998,7 @@ def main():
             torch.cuda.empty_cache()
             rec = run_scan(args, lib, dev, other, few.steps, args.warmup, few.settle_steps)
             rec.pop("_cpu_args")
+            rec.pop("_buffers")
             also[other] = {k: rec[k] for k in ("config", "value", "unit", "ms_per_step", "steps", "warmup",
                                                "settle_steps", "roofline", "fwd", "step_hbm")}
         # the matrix-core gate projections and the recurrent core of one layer at the same shape, and
