@@ -41,6 +41,7 @@ SIGNATURES = {
     "hawk_scan_workspace_status": (_c_int, [_c_void_p, _c_void_p, ctypes.POINTER(_c_int)]),
     "hawk_rglru_scan_fwd": (_c_int, [_c_void_p] * 5 + [_c_int] * 4 + [_c_void_p, _c_size_t, _c_void_p]),
     "hawk_rglru_scan_fwd_static": (_c_int, [_c_void_p] * 5 + [_c_int] * 4 + [_c_void_p]),
+    "hawk_rglru_scan_fwd_static_bytes": (_c_size_t, [_c_int] * 4),
     "hawk_rglru_scan_bwd": (_c_int, [_c_void_p] * 10 + [_c_int] * 4 + [_c_void_p, _c_size_t, _c_void_p]),
     "hawk_rglru_scan_fwd_mixed": (_c_int, [_c_void_p] * 5 + [_c_int] * 5 + [_c_void_p, _c_size_t, _c_void_p]),
     "hawk_rglru_scan_bwd_mixed": (_c_int, [_c_void_p] * 10 + [_c_int] * 5 + [_c_void_p, _c_size_t, _c_void_p]),
@@ -177,10 +178,13 @@ def dense16(t: torch.Tensor) -> torch.Tensor:
 # Scans that share a workspace must be ordered on one stream, hence the key.
 # ---------------------------------------------------------------------------------------
 _workspaces: dict = {}
-# Workspaces handed to launches recorded into HIP graphs: (device index, tensor).  They belong to
-# the graph's memory pool; a reference is kept so that their carry-timeout flag can be read
-# after a replay.  At most _MAX_CAPTURED are remembered (oldest dropped first).
-_captured: list = []
+# Workspaces handed to launches recorded into HIP graphs: (device index, stream, capture id) ->
+# tensors.  They belong to the graph's memory pool; a reference is kept so that their
+# carry-timeout flag can be read after a replay.  All scans recorded into one capture on one
+# stream share one buffer (a second, larger one only if a later scan needs more), so a captured
+# training step holds one workspace, not one per layer and direction.  At most _MAX_CAPTURED
+# captures are remembered (oldest dropped first; their memory stays with the graph's pool).
+_captured: dict = {}
 _MAX_CAPTURED = 256
 
 
@@ -190,15 +194,23 @@ def _device_index(dev: torch.device) -> int:
 
 def scan_workspace(dev: torch.device, nbytes: int) -> torch.Tensor:
     if torch.cuda.is_current_stream_capturing():
-        # A captured launch gets a workspace of its own from the graph's memory pool, zeroed by a
-        # fill kernel that is part of the graph: the graph then depends on no buffer that eager
-        # code or another graph also uses, whatever stream it is replayed on and in whatever
-        # order graphs are replayed.  (A cached buffer created during a capture would hold
-        # nothing until that one graph had been replayed.)
-        ws = torch.zeros(max(nbytes, 256), dtype=torch.uint8, device=dev)
+        # Captured launches get a workspace from the graph's own memory pool, zeroed by a fill
+        # kernel that is part of the graph: the graph then depends on no buffer that eager code
+        # or another graph also uses, whatever stream it is replayed on and in whatever order
+        # graphs are replayed.  (A cached buffer created during a capture would hold nothing
+        # until that one graph had been replayed.)  The scans of one capture are ordered on their
+        # stream, every launch re-arms the control word and tags its carry words with its own
+        # epoch, so they share the buffer as eager launches on a stream do.
+        key = (_device_index(dev), stream_ptr(dev), _capture_id(dev))
         with _lock:
-            _captured.append((_device_index(dev), ws))
-            del _captured[:-_MAX_CAPTURED]
+            held = _captured.setdefault(key, [])
+            if held and held[-1].numel() >= nbytes:
+                return held[-1]
+        ws = torch.zeros(max(nbytes, 1 << 20), dtype=torch.uint8, device=dev)
+        with _lock:
+            held.append(ws)
+            while len(_captured) > _MAX_CAPTURED:
+                _captured.pop(next(iter(_captured)))
         return ws
     key = (_device_index(dev), stream_ptr(dev))
     with _lock:
@@ -280,7 +292,8 @@ def check_scan_status(device=None) -> None:
     dev = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
     idx = _device_index(dev)
     with _lock:
-        todo = [ws for (d, _s), ws in _workspaces.items() if d == idx] + [ws for d, ws in _captured if d == idx]
+        todo = [ws for (d, _s), ws in _workspaces.items() if d == idx]
+        todo += [ws for (d, _s, _c), held in _captured.items() if d == idx for ws in held]
     torch.cuda.synchronize(dev)
     for ws in todo:
         if _flag_of(ws, dev) != 0:

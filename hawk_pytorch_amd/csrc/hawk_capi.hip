@@ -55,7 +55,7 @@ const char* hawk_status_string(int status) {
         case HAWK_ERR_ALIGNMENT: return "tensor pointers must be 16-byte aligned";
         case HAWK_ERR_SCRATCH_LIMIT:
             return "shape needs more carry words than the library's fixed 16 MiB scratch array holds: "
-                   "ceil(T/128) * B * D * 24 + 256 bytes must fit; use the entry point that takes a workspace";
+                   "hawk_rglru_scan_fwd_static_bytes(B, T, D, dtype) must fit; use the entry point that takes a workspace";
         default: return "unknown status";
     }
 }
@@ -105,6 +105,11 @@ int hawk_rglru_scan_fwd_static(const void* x, const void* x_rg_lru, const void* 
     if (int rc = check_scan_shape(B, T, D)) return rc;
     if (!aligned16(x) || !aligned16(x_rg_lru) || !aligned16(a_rg_lru) || !aligned16(h)) return HAWK_ERR_ALIGNMENT;
     return hawk::scan_fwd_static(x, x_rg_lru, a_rg_lru, a_param, h, B, T, D, dtype, as_stream(stream));
+}
+
+size_t hawk_rglru_scan_fwd_static_bytes(int B, int T, int D, int dtype) {
+    if (check_scan_shape(B, T, D) != HAWK_OK || !dtype_ok(dtype)) return 0;
+    return hawk::scan_fwd_static_bytes(B, T, D, dtype);
 }
 
 int hawk_rglru_scan_bwd_mixed(const void* x, const void* x_rg_lru, const void* a_rg_lru, const float* a_param,

@@ -24,6 +24,8 @@ int scan_bwd(const void* x, const void* xg, const void* ag, const float* lam, co
 int scan_fwd_static(const void* x, const void* xg, const void* ag, const float* lam, void* h, int B, int T, int D,
                     int dtype, hipStream_t st);
 int static_scratch_status(hipStream_t st, int* flag);
+// bytes of the fixed array a shape needs (0 when T fits one tile)
+size_t scan_fwd_static_bytes(int B, int T, int D, int dtype);
 // Gated variants: out = gelu(y) * h.  y (and dy) are [B, T, D] with ldy (lddy) elements between rows.
 int scan_gated_fwd(const void* x, const void* xg, const void* ag, const float* lam, const void* y, long long ldy,
                    void* h, void* out, void* h_last, int B, int T, int D, int in_dtype, int out_dtype, void* ws,

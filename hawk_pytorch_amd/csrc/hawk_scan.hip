@@ -1063,18 +1063,15 @@ constexpr int kMaxDevices = 64;
 std::mutex g_scratch_mutex;
 void* g_scratch_ptr[kMaxDevices] = {};
 
-// Device address of the current device's scratch array; *fresh is set when this call is the
-// one that looked it up.
-int static_scratch_ptr(void** out, bool* fresh) {
+// Device address of the current device's scratch array.
+int static_scratch_ptr(void** out) {
     int dev = -1;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return HAWK_ERR_LAUNCH;
     std::lock_guard<std::mutex> guard(g_scratch_mutex);
-    *fresh = false;
     if (g_scratch_ptr[dev] == nullptr) {
         void* p = nullptr;
         if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || p == nullptr) return HAWK_ERR_LAUNCH;
         g_scratch_ptr[dev] = p;
-        *fresh = true;
     }
     *out = g_scratch_ptr[dev];
     return HAWK_OK;
@@ -1082,36 +1079,36 @@ int static_scratch_ptr(void** out, bool* fresh) {
 
 }  // namespace
 
-int scan_fwd_static(const void* x, const void* xg, const void* ag, const float* lam, void* h, int B, int T, int D,
-                    int dtype, hipStream_t st) {
+size_t scan_fwd_static_bytes(int B, int T, int D, int dtype) {
     const TileShape s = fwd_shape(D, dtype);
     const int nseg = ceil_div(T, s.rows());
-    if (nseg > 1 && layout_for(B, D, nseg, 0).total > (size_t)HAWK_STATIC_SCRATCH_BYTES) return HAWK_ERR_SCRATCH_LIMIT;
+    return nseg > 1 ? layout_for(B, D, nseg, 0).total : 0;
+}
+
+int scan_fwd_static(const void* x, const void* xg, const void* ag, const float* lam, void* h, int B, int T, int D,
+                    int dtype, hipStream_t st) {
+    if (scan_fwd_static_bytes(B, T, D, dtype) > (size_t)HAWK_STATIC_SCRATCH_BYTES) return HAWK_ERR_SCRATCH_LIMIT;
+    // Nothing is cleared, here or ever: the array starts as zeros like any object of static
+    // storage, the ticket half of its control word is back at zero when a launch ends, and the
+    // words of earlier calls carry older launch tags.  (A clearing kernel on the first caller's
+    // stream would race with a second thread's first call on another stream.)
     void* ws = nullptr;
-    bool fresh = false;
-    if (int rc = static_scratch_ptr(&ws, &fresh)) return rc;
-    if (fresh) {
-        // The array starts as zeros like any object of static storage; the first use on a
-        // device clears it all the same (with a fill kernel, ordered before the scan on the
-        // caller's stream) unless that stream is being captured: a fill recorded into a graph
-        // would rewind the launch epoch at every replay.  Afterwards nothing needs clearing:
-        // the ticket half of the control word is back at zero when a launch ends, and words
-        // of earlier calls carry older launch tags.
-        hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
-        if (hipStreamIsCapturing(st, &cap) != hipSuccess) return HAWK_ERR_LAUNCH;
-        if (cap == hipStreamCaptureStatusNone) {
-            if (int rc = workspace_init(ws, HAWK_STATIC_SCRATCH_BYTES, st)) return rc;
-        }
-    }
+    if (int rc = static_scratch_ptr(&ws)) return rc;
     return scan_fwd_impl<false>(x, xg, ag, lam, h, GateFwdHost{}, B, T, D, dtype, dtype, ws,
                                 (size_t)HAWK_STATIC_SCRATCH_BYTES, st);
 }
 
 int static_scratch_status(hipStream_t st, int* flag) {
     void* ws = nullptr;
-    bool fresh = false;
-    if (int rc = static_scratch_ptr(&ws, &fresh)) return rc;
-    return workspace_status(ws, st, flag);
+    if (int rc = static_scratch_ptr(&ws)) return rc;
+    if (int rc = workspace_status(ws, st, flag)) return rc;
+    if (*flag != 0) {
+        // the array cannot be re-initialised by the caller, so reading a raised flag lowers it
+        // (one word, with the fill kernel: nothing is allocated)
+        hipLaunchKernelGGL(fill_u32_kernel, dim3(1), dim3(64), 0, st, static_cast<uint32_t*>(ws) + 2, (size_t)1, 0u);
+        if (hipGetLastError() != hipSuccess) return HAWK_ERR_LAUNCH;
+    }
+    return HAWK_OK;
 }
 
 bool scan_dtypes_supported(int in_dtype, int state_dtype) {

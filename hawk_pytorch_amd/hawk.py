@@ -150,10 +150,11 @@ class Hawk(nn.Module):
             # last position, hawk/hawk.py:178-179, with a conv window that then spans the new
             # rows; nothing sensible can be returned for the other positions, so refuse.)
             assert layer_past is not None
-            assert x.shape[1] == 1, (
-                f"a warm cache takes one new token per call, got {x.shape[1]}; "
-                "feed longer inputs with a fresh RNNCache (prefill)"
-            )
+            if x.shape[1] != 1:
+                raise ValueError(
+                    f"a warm cache takes one new token per call, got {x.shape[1]}; "
+                    "feed longer inputs with a fresh RNNCache (prefill)"
+                )
             layer_past.own_buffers()
             fused_gates = self.config.fused_gates and gate_projections_supported(branch, self.rg_lru_input_gate)
             gate_branch = gate_branch[:, -1:, :]

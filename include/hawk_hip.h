@@ -68,7 +68,9 @@ int hawk_scan_workspace_init(void* workspace_device, size_t workspace_bytes, voi
 /* Synchronises `stream` and reports in *flag whether any scan on this workspace gave up
  * waiting for a carry (0 = all carries arrived).  A non-zero flag means results of that
  * launch are invalid and the workspace must be re-initialised.  workspace_device == NULL
- * asks about the current device's fixed scratch array (hawk_rglru_scan_fwd_static). */
+ * asks about the current device's fixed scratch array (hawk_rglru_scan_fwd_static), which the
+ * caller cannot re-initialise: reading a raised flag there lowers it again (a one-word fill
+ * kernel on `stream`), so one lost carry is reported once. */
 int hawk_scan_workspace_status(const void* workspace_device, void* stream, int* flag);
 
 /* ---------------------------------------------------------------------------------------
@@ -95,16 +97,19 @@ int hawk_rglru_scan_fwd(const void* x, const void* x_rg_lru, const void* a_rg_lr
  * live in an array of HAWK_STATIC_SCRATCH_BYTES that is part of the library's device code:
  * every GPU the library is used on holds one such array from the first call there until the
  * process ends.  The call allocates and frees nothing.
- *   limit   ceil(T / 128) * B * D * 24 bytes + 256 must not exceed HAWK_STATIC_SCRATCH_BYTES
- *           (T <= 128 always fits); beyond it the call returns HAWK_ERR_SCRATCH_LIMIT and
- *           launches nothing.  B=8, T=4096, D=2560 needs 15.0 MiB.
+ *   limit   hawk_rglru_scan_fwd_static_bytes(B, T, D, dtype), the bytes of the array a shape
+ *           uses, must not exceed HAWK_STATIC_SCRATCH_BYTES: at most
+ *           ceil(T / 128) * B * D * 24 + 1024 bytes, and 0 when T <= 128; beyond it the call
+ *           returns HAWK_ERR_SCRATCH_LIMIT and launches nothing.  B=8, T=4096, D=2560 needs
+ *           15.0 MiB.
  *   sharing every call on a GPU uses that GPU's one array, so calls must not overlap there:
  *           order them on one stream (or with events).  Two overlapping calls race.
  *   set-up  the first call on a device looks up the array's device address (the device must
- *           be current, as for every call) and clears the array with a fill kernel ahead of
- *           the scan on `stream`; when that first call is being captured into a graph the
- *           fill is left out and the array's zero initialisation is relied on. */
+ *           be current, as for every call).  Nothing is ever cleared: the array starts as
+ *           zeros, a launch leaves its ticket counter at zero, and carry words are tagged with
+ *           their launch's epoch, so the call records nothing but its kernel into a graph. */
 #define HAWK_STATIC_SCRATCH_BYTES (16u << 20)
+size_t hawk_rglru_scan_fwd_static_bytes(int B, int T, int D, int dtype);
 int hawk_rglru_scan_fwd_static(const void* x, const void* x_rg_lru, const void* a_rg_lru,
                                const float* a_param, void* h, int B, int T, int D, int dtype,
                                void* stream);

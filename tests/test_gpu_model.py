@@ -885,7 +885,7 @@ def test_warm_cache_refuses_more_than_one_new_token():
     ids = torch.randint(1, cfg.vocab_size, (1, 9), device="cuda")
     with torch.no_grad():
         _, caches = model(ids[:, :6], layer_past=model.new_cache(1))
-        with pytest.raises(AssertionError, match="one new token"):
+        with pytest.raises(ValueError, match="one new token"):
             model(ids[:, 6:9], layer_past=caches)
 
 

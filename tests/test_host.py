@@ -119,6 +119,16 @@ def test_scan_shape_limits_are_checked_before_any_launch():
     # 64 tiles in time x 8 x 2560 channels x 24 bytes = 31.5 MB of carry words > 16 MiB
     assert lib.hawk_rglru_scan_fwd_static(*args, 8, 8192, 2560, 0, None) == _lib.HAWK_ERR_SCRATCH_LIMIT
     assert lib.hawk_rglru_scan_fwd_static(None, p, p, p, p, 1, 8, 64, 0, None) == _lib.HAWK_ERR_NULL_POINTER
+    # the size query states the limit exactly: the largest chain that fits, and one tile more
+    limit = 16 << 20
+    fits, over = 10922 * 128, 10923 * 128
+    assert 0 < lib.hawk_rglru_scan_fwd_static_bytes(1, fits, 64, 0) <= limit
+    assert lib.hawk_rglru_scan_fwd_static_bytes(1, over, 64, 0) > limit
+    assert lib.hawk_rglru_scan_fwd_static_bytes(1, 128, 64, 0) == 0          # one tile: no carry words
+    assert lib.hawk_rglru_scan_fwd_static_bytes(8, 4096, 2560, 0) <= 32 * 8 * 2560 * 24 + 1024
+    assert lib.hawk_rglru_scan_fwd_static(*args, 1, over, 64, 0, None) == _lib.HAWK_ERR_SCRATCH_LIMIT
+    if not torch.cuda.is_available():   # with a GPU this call would launch on the host buffer above
+        assert lib.hawk_rglru_scan_fwd_static(*args, 1, fits, 64, 0, None) != _lib.HAWK_ERR_SCRATCH_LIMIT
     assert lib.hawk_rglru_scan_fwd_static(*args, 1, 8, 64, 5, None) == _lib.HAWK_ERR_BAD_DTYPE
 
 

@@ -86,6 +86,30 @@ def test_static_scan_refuses_shapes_beyond_its_array():
     assert "scratch" in _lib.status_string(rc)
 
 
+def test_static_scan_at_the_exact_limit_of_its_array():
+    """The size query is the limit: the longest chain whose words fit runs and matches the
+    workspace scan; one tile more is refused."""
+    lib = _lib.load()
+    B, D = 1, 64
+    fits, over = 10922 * 128, 10923 * 128
+    assert lib.hawk_rglru_scan_fwd_static_bytes(B, fits, D, _lib.HAWK_DTYPE_BF16) <= 16 << 20
+    assert lib.hawk_rglru_scan_fwd_static_bytes(B, over, D, _lib.HAWK_DTYPE_BF16) > 16 << 20
+    g = torch.Generator(device="cuda").manual_seed(5)
+    x, xg, ag = (torch.randn((B, over, D), generator=g, device="cuda").to(torch.bfloat16) for _ in range(3))
+    lam = capi.to_dev(np.random.default_rng(5).uniform(-7.0, -2.0, D), "f32")
+    h = torch.empty_like(x)
+    rc = lib.hawk_rglru_scan_fwd_static(x.data_ptr(), xg.data_ptr(), ag.data_ptr(), lam.data_ptr(), h.data_ptr(),
+                                        B, over, D, _lib.HAWK_DTYPE_BF16, torch.cuda.current_stream().cuda_stream)
+    assert rc == _lib.HAWK_ERR_SCRATCH_LIMIT
+    xs, xgs, ags = (t[:, :fits].contiguous() for t in (x, xg, ag))
+    print(f"static scan at the limit B={B} T={fits} D={D}", flush=True)
+    got = _static_fwd(xs, xgs, ags, lam)
+    want = capi.scan_fwd(xs, xgs, ags, lam)
+    torch.cuda.synchronize()
+    assert _static_flag() == 0
+    assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+
+
 def test_static_scan_at_the_benchmark_shape_fits_and_matches():
     B, T, D = 8, 4096, 2560
     g = torch.Generator(device="cuda").manual_seed(3)
