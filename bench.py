@@ -356,14 +356,16 @@ def run_block(args, lib, dev):
         # the projections' input gradient accumulates onto the scan's, in place
         _lib.check("gate_bwd_input", lib.hawk_gate_proj_bwd_input(p(dxg), p(dag), p(wi16), p(wa16), p(du), p(du), M,
                                                                   D, nb, code, code, code, st))
-        _lib.check("gate_bwd_weights", lib.hawk_gate_proj_bwd_weights(
-            p(u), p(dxg), p(dag), p(dwi), p(dbi), p(dwa), p(dba), M, D, nb, code, code, p(gws), gws.numel(), st))
+        # the conv's backward right behind the kernel that wrote its input gradient (part of those
+        # 168 MB is then still in the memory-side cache: 1 % of the step), the weight gradients last
         if inplace:
             _lib.check("conv_bwd", lib.hawk_conv1d_bwd_strided(p(du), p(xy), 2 * D, p(cw), p(dxy), 2 * D, p(dcw),
                                                                p(dcb), B, T, D, W, code, code, p(cws), cws.numel(), st))
         else:
             _lib.check("conv_bwd", lib.hawk_conv1d_bwd(p(du), p(xin), p(cw), p(dxin), p(dcw), p(dcb), B, T, D, W,
                                                        code, code, p(cws), cws.numel(), st))
+        _lib.check("gate_bwd_weights", lib.hawk_gate_proj_bwd_weights(
+            p(u), p(dxg), p(dag), p(dwi), p(dbi), p(dwa), p(dba), M, D, nb, code, code, p(gws), gws.numel(), st))
 
     for _ in range(args.settle_steps + args.warmup):
         fwd(), bwd()

@@ -567,12 +567,14 @@ def _launch_block_core_bwd(xy, u, xg, ag, h, conv_w, w_i, w_a, lam, grad_out):
         _lib.check("hawk_gate_proj_bwd_input", lib.hawk_gate_proj_bwd_input(
             dxg.data_ptr(), dag.data_ptr(), w_i.data_ptr(), w_a.data_ptr(), du.data_ptr(), du.data_ptr(), M, D, nb,
             code, wcode, code, st))
-        _lib.check("hawk_gate_proj_bwd_weights", lib.hawk_gate_proj_bwd_weights(
-            u.data_ptr(), dxg.data_ptr(), dag.data_ptr(), dw_i.data_ptr(), db_i.data_ptr(), dw_a.data_ptr(),
-            db_a.data_ptr(), M, D, nb, code, code, gws.data_ptr(), gws.numel(), st))
+        # the conv's backward right behind the kernel that wrote its input gradient (part of it is
+        # then still in the memory-side cache), the weight gradients last
         _lib.check("hawk_conv1d_bwd_strided", lib.hawk_conv1d_bwd_strided(
             du.data_ptr(), xy.data_ptr(), ld, conv_w.data_ptr(), d_xy.data_ptr(), D2, dcw.data_ptr(),
             dcb.data_ptr(), B, T, D, W, code, code, cws.data_ptr(), cws.numel(), st))
+        _lib.check("hawk_gate_proj_bwd_weights", lib.hawk_gate_proj_bwd_weights(
+            u.data_ptr(), dxg.data_ptr(), dag.data_ptr(), dw_i.data_ptr(), db_i.data_ptr(), dw_a.data_ptr(),
+            db_a.data_ptr(), M, D, nb, code, code, gws.data_ptr(), gws.numel(), st))
     return d_xy, dcw, dcb, dw_i, db_i, dw_a, db_a, dlam
 
 
