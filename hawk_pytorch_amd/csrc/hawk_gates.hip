@@ -44,7 +44,7 @@ constexpr int kTileRows = 32;                  // rows per MFMA tile
 constexpr int kGateThreads = 1024;             // 16 waves
 constexpr int kARowBytes = kGroup * 2 + 16;    // bf16 row + pad: 8 lanes' 16-byte reads cover all banks
 constexpr int kATileBytes = kTileRows * kARowBytes;
-constexpr int kNumCU = 256;
+constexpr int kDefaultNumCU = 256;   // MI355X; used when the device cannot be asked
 // Row counts up to this one take the forward kernel that is cut by output columns.
 #ifndef HAWK_GATE_MIN_SPLIT_TILES
 #define HAWK_GATE_MIN_SPLIT_TILES 4
@@ -1316,6 +1316,21 @@ __global__ void gate_proj_reduce_kernel(const float* __restrict__ part_w, const 
 
 inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
 
+// Compute units of the current device (asked once per device): the persistent kernels launch one
+// workgroup per compute unit, and the size of the weight-gradient workspace follows from it.
+int num_cu() {
+    static std::atomic<int> cached[64] = {};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return kDefaultNumCU;
+    int n = cached[dev].load(std::memory_order_relaxed);
+    if (n == 0) {
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+            n = kDefaultNumCU;
+        cached[dev].store(n, std::memory_order_relaxed);
+    }
+    return n;
+}
+
 // Raises a kernel's dynamic LDS limit once per device instead of on every launch.
 template <auto Kernel>
 bool allow_dynamic_lds(size_t bytes) {
@@ -1340,7 +1355,7 @@ int launch_gate_fwd(const void* x, const void* w_i, const float* b_i, const void
         // enough workgroups to give every compute unit a few waves; each wave keeps its weights
         // for all the row tiles it walks over
         const int ncolblocks = 2 * (D / 32);
-        int rsplit = ceil_div(8 * kNumCU, ncolblocks * kSmallWaves);
+        int rsplit = ceil_div(8 * num_cu(), ncolblocks * kSmallWaves);
         const int max_split = ceil_div(ntiles, kSmallWaves);
         if (rsplit > max_split) rsplit = max_split;
         hipLaunchKernelGGL((gate_proj_fwd_small_kernel<XT, WT, OT, BW>), dim3((unsigned)ncolblocks, (unsigned)rsplit),
@@ -1349,7 +1364,7 @@ int launch_gate_fwd(const void* x, const void* w_i, const float* b_i, const void
                            D, ntiles);
         return hipGetLastError() == hipSuccess ? HAWK_OK : HAWK_ERR_LAUNCH;
     }
-    int nworkers = kNumCU / ngroups;
+    int nworkers = num_cu() / ngroups;
     if (nworkers < 1) nworkers = 1;
     if (nworkers > ntiles) nworkers = ntiles;
     size_t smem = gate_fwd_lds_bytes<OT>(false);
@@ -1370,7 +1385,7 @@ int launch_conv_gate_fwd(const void* x, long long ldx, const float* conv_w, cons
                          int M, int T, int D, int nb, hipStream_t st) {
     const int ngroups = ceil_div(D, kGroup);
     const int ntiles = ceil_div(M, kTileRows);
-    int nworkers = kNumCU / ngroups;
+    int nworkers = num_cu() / ngroups;
     if (nworkers < 1) nworkers = 1;
     if (nworkers > ntiles) nworkers = ntiles;
     constexpr size_t smem = gate_fwd_lds_bytes<bf16_t>(true);
@@ -1422,7 +1437,7 @@ int launch_gate_bwd_input(const void* dxg, const void* dag, const void* w_i, con
                           void* dx, int M, int D, int nb, hipStream_t st) {
     const int ngroups = ceil_div(D, kGroup);
     const int ntiles = ceil_div(M, kTileRows);
-    int nworkers = kNumCU / ngroups;
+    int nworkers = num_cu() / ngroups;
     if (nworkers < 1) nworkers = 1;
     if (nworkers > ntiles) nworkers = ntiles;
     const size_t smem = 4 * kATileBytes + 2 * (size_t)kTileRows * (kGroup * 4 + 16);
@@ -1460,7 +1475,7 @@ int gate_bwd_input_out(const void* dxg, const void* dag, const void* w_i, const 
 
 int weight_splits(int M, int D) {
     const int ngroups = ceil_div(D, kGroup);
-    int n = kNumCU / (2 * ngroups);
+    int n = num_cu() / (2 * ngroups);
     if (n < 1) n = 1;
     // at least HAWK_GATE_MIN_SPLIT_TILES row tiles per split: every split costs a pass over its
     // partial sums in the reduction
@@ -1496,14 +1511,13 @@ int gate_bwd_weights_bw(const void* x, const void* dg_i, const void* dg_a, float
 // 9.5 against 8.1 us at 256 rows), and only while the launch fits the device in one round:
 // at 256 rows and 10 blocks two workgroups per block take 14.9 us against 18.7 for one and 21.8
 // for four (320 workgroups); at 32 rows four take 10.3 against 17.6 us.
-#ifndef HAWK_CORE_MAX_GRID
-#define HAWK_CORE_MAX_GRID 256
-#endif
-constexpr int kCoreMaxGrid = HAWK_CORE_MAX_GRID;
+// (the grid is kept within one workgroup per compute unit of the device)
+int num_cu();
 inline int decode_core_parts(int pairs, int bw, bool have_counters) {
     if (!have_counters || bw < 256) return 1;
-    if ((long long)pairs * 4 <= kCoreMaxGrid) return 4;
-    if ((long long)pairs * 2 <= kCoreMaxGrid) return 2;
+    const int max_grid = num_cu();
+    if ((long long)pairs * 4 <= max_grid) return 4;
+    if ((long long)pairs * 2 <= max_grid) return 2;
     return 1;
 }
 
