@@ -14,10 +14,12 @@ y being one half of a [B, T, 2D] projection), 12 + 20 bytes per element;
 forward, input gradient, weight gradients) on 32768 tokens, D = 2560, 10 blocks, bf16;
 ``--workload block`` chains the whole recurrent core of one layer at B=8, T=4096, D=2560 (conv and
 both gate projections in one kernel, scan fused with the output gate, and the backward of all of
-them) through the C ABI on the [B,T,2D] output of the block's input projection in place, six
-launches that move 30 activation-sized tensors (plus two casts of the fp32 gate weights to bf16,
-as the Python host does at this size); ``--unfused-conv`` runs the conv as a launch of its own on
-a copy of the x half, seven launches and 31 tensors;
+them) through the C ABI on the [B,T,2D] output of the block's input projection in place, one host call
+per direction: six large launches that move 30 activation-sized tensors, one that rounds the fp32
+weights of both gates to bf16 (as the Python host does at this size) and one for the three closing
+reductions of the backward; ``--unfused-conv`` runs the single entry points instead (the conv as a
+launch of its own on a copy of the x half, seven large launches and 31 tensors, two weight casts,
+a reduction launch per backward call);
 ``--workload model`` runs full training steps (forward, backward, AdamW) of the upstream
 README model (vocabulary 32000, hidden = recurrent = 512, MLP 1024, 8 layers, 16 gate blocks)
 on a 1 x 2048 batch under bf16 autocast, with and without the fused gate / epilogue kernels;
@@ -328,42 +330,47 @@ def run_block(args, lib, dev):
     st = torch.cuda.current_stream(dev).cuda_stream
     p = lambda t: t.data_ptr()  # noqa: E731
 
-    wi16, wa16 = torch.empty_like(wi, dtype=bf), torch.empty_like(wa, dtype=bf)
+    w16 = torch.empty((2, nb, bw, bw), device=dev, dtype=bf)
+    wi16, wa16 = w16[0], w16[1]
+    F32 = _lib.HAWK_DTYPE_F32
 
     def fwd():
-        # as the Python host does from 8192 rows on: the fp32 gate weights are rounded to bf16 once
-        # per step (two small kernels, inside the timed region) instead of by every workgroup
+        if not args.unfused_conv:
+            # one host call: the fp32 gate weights rounded to bf16 once per step (one launch for both
+            # gates, inside the timed region), conv and both projections in one kernel reading the x
+            # half of xy in place, then the scan with the output gate
+            _lib.check("block_core_fwd", lib.hawk_block_core_fwd(
+                p(xy), 2 * D, p(cw), p(cb), p(wi), p(bi), p(wa), p(ba), F32, p(w16), p(lam), p(u), p(xg), p(ag),
+                p(h), p(out), None, B, T, D, nb, W, p(ws), ws.numel(), st))
+            return
+        # the single calls, as the Python host does from 8192 rows on: the fp32 gate weights are
+        # rounded to bf16 once per step instead of by every workgroup
         wi16.copy_(wi)
         wa16.copy_(wa)
-        if args.unfused_conv:
-            _lib.check("conv_fwd", lib.hawk_conv1d_fwd(p(xin), p(cw), p(cb), None, p(u), B, T, D, W, code, code, st))
-            _lib.check("gate_fwd", lib.hawk_gate_proj_fwd(p(u), p(wi16), p(bi), p(wa16), p(ba), p(xg), p(ag), M, D,
-                                                          nb, code, code, code, st))
-        else:
-            # conv and both projections in one kernel, reading the x half of xy in place
-            _lib.check("conv_gate_fwd", lib.hawk_conv_gate_proj_fwd(
-                p(xy), 2 * D, p(cw), p(cb), p(wi16), p(bi), p(wa16), p(ba), p(u), p(xg), p(ag), B, T, D, nb, W,
-                code, st))
+        _lib.check("conv_fwd", lib.hawk_conv1d_fwd(p(xin), p(cw), p(cb), None, p(u), B, T, D, W, code, code, st))
+        _lib.check("gate_fwd", lib.hawk_gate_proj_fwd(p(u), p(wi16), p(bi), p(wa16), p(ba), p(xg), p(ag), M, D,
+                                                      nb, code, code, code, st))
         _lib.check("scan_gated_fwd", lib.hawk_rglru_scan_gated_fwd(
             p(u), p(xg), p(ag), p(lam), p(y), 2 * D, p(h), p(out), None, B, T, D, code, code, p(ws), ws.numel(), st))
 
     def bwd():
-        inplace = not args.unfused_conv
+        if not args.unfused_conv:
+            # one host call: gated scan -> the projections' input gradient onto the scan's, in place
+            # -> conv (right behind the kernel that wrote its input gradient: part of those 168 MB is
+            # then still in the memory-side cache, 1 % of the step) -> the projections' weight
+            # gradients -> one launch for the three closing reductions
+            _lib.check("block_core_bwd", lib.hawk_block_core_bwd(
+                p(xy), 2 * D, p(u), p(xg), p(ag), p(h), p(cw), p(wi16), p(wa16), code, p(lam), p(gout), p(dxy),
+                2 * D, p(du), p(dxg), p(dag), p(dcw), p(dcb), p(dwi), p(dbi), p(dwa), p(dba), p(dlam), B, T, D, nb,
+                W, p(ws), ws.numel(), p(gws), gws.numel(), p(cws), cws.numel(), st))
+            return
         _lib.check("scan_gated_bwd", lib.hawk_rglru_scan_gated_bwd(
-            p(u), p(xg), p(ag), p(lam), p(y), 2 * D, p(h), p(gout), p(du), p(dxg), p(dag),
-            p(dxy) + 2 * D if inplace else p(dy), 2 * D if inplace else D, p(dlam),
+            p(u), p(xg), p(ag), p(lam), p(y), 2 * D, p(h), p(gout), p(du), p(dxg), p(dag), p(dy), D, p(dlam),
             B, T, D, code, code, p(ws), ws.numel(), st))
-        # the projections' input gradient accumulates onto the scan's, in place
         _lib.check("gate_bwd_input", lib.hawk_gate_proj_bwd_input(p(dxg), p(dag), p(wi16), p(wa16), p(du), p(du), M,
                                                                   D, nb, code, code, code, st))
-        # the conv's backward right behind the kernel that wrote its input gradient (part of those
-        # 168 MB is then still in the memory-side cache: 1 % of the step), the weight gradients last
-        if inplace:
-            _lib.check("conv_bwd", lib.hawk_conv1d_bwd_strided(p(du), p(xy), 2 * D, p(cw), p(dxy), 2 * D, p(dcw),
-                                                               p(dcb), B, T, D, W, code, code, p(cws), cws.numel(), st))
-        else:
-            _lib.check("conv_bwd", lib.hawk_conv1d_bwd(p(du), p(xin), p(cw), p(dxin), p(dcw), p(dcb), B, T, D, W,
-                                                       code, code, p(cws), cws.numel(), st))
+        _lib.check("conv_bwd", lib.hawk_conv1d_bwd(p(du), p(xin), p(cw), p(dxin), p(dcw), p(dcb), B, T, D, W,
+                                                   code, code, p(cws), cws.numel(), st))
         _lib.check("gate_bwd_weights", lib.hawk_gate_proj_bwd_weights(
             p(u), p(dxg), p(dag), p(dwi), p(dbi), p(dwa), p(dba), M, D, nb, code, code, p(gws), gws.numel(), st))
 
@@ -936,9 +943,10 @@ def main():
                     help="workload gates: hand the projection kernels the fp32 weights instead of rounding them "
                          "to bf16 once per step")
     ap.add_argument("--unfused-conv", action="store_true",
-                    help="workload block: conv and gate projections as two launches on a copy of the x half of the "
-                         "input projection, gradients into separate tensors, instead of one launch on the "
-                         "projection's output in place and one gradient tensor")
+                    help="workload block: the single entry points (two weight casts, conv and gate projections as "
+                         "two launches on a copy of the x half of the input projection, gradients into separate "
+                         "tensors, a closing reduction per backward call) instead of one host call per direction "
+                         "on the projection's output in place")
     ap.add_argument("--workload", choices=sorted(WORKLOADS) + ["block", "decode", "gates", "model"], default="scan")
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--no-cpu-baseline", action="store_true")

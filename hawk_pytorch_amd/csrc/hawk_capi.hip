@@ -364,4 +364,71 @@ int hawk_gate_proj_bwd_weights(const void* x, const void* d_x_rg_lru, const void
                                        g_dtype, workspace_device, workspace_bytes, as_stream(stream));
 }
 
+int hawk_gate_weights_to_bf16(const float* w_i, const float* w_a, void* w_i_bf16, void* w_a_bf16, int num_blocks,
+                              int block_width, void* stream) {
+    if (!w_i || !w_a || !w_i_bf16 || !w_a_bf16) return HAWK_ERR_NULL_POINTER;
+    if (num_blocks < 1 || block_width < 1 || block_width % 4 != 0 ||
+        (long long)num_blocks * block_width * block_width > 0x7fffffffLL)
+        return HAWK_ERR_BAD_SHAPE;
+    if (!aligned16(w_i) || !aligned16(w_a) || !aligned16(w_i_bf16) || !aligned16(w_a_bf16)) return HAWK_ERR_ALIGNMENT;
+    return hawk::gate_weights_to_bf16(w_i, w_a, w_i_bf16, w_a_bf16, (size_t)num_blocks * block_width * block_width,
+                                      as_stream(stream));
+}
+
+int hawk_block_core_fwd(const void* xy, long long xy_row_stride, const float* conv_w, const float* conv_b,
+                        const void* w_i, const float* b_i, const void* w_a, const float* b_a, int w_dtype,
+                        void* w_bf16, const float* a_param, void* u, void* x_rg_lru, void* a_rg_lru, void* h, void* out,
+                        void* h_last, int B, int T, int D, int num_blocks, int temporal_width,
+                        void* scan_workspace, size_t scan_workspace_bytes, void* stream) {
+    if (!xy || !conv_w || !conv_b || !w_i || !w_a || !a_param || !u || !x_rg_lru || !a_rg_lru || !out)
+        return HAWK_ERR_NULL_POINTER;
+    if (!dtype_ok(w_dtype)) return HAWK_ERR_BAD_DTYPE;
+    if (int rc = check_scan_shape(B, T, D)) return rc;
+    // the conv in front of the projections: one wrap of the position per 32-row tile, 32-bit byte
+    // offsets over a tile and its history; y = xy + D must stay 16-byte aligned row by row
+    if (T < 32 || temporal_width != 4 || !hawk_gate_proj_supported(D, num_blocks) || D % 8 != 0 ||
+        (long long)B * T > 0x7fffffffLL || xy_row_stride < 2LL * D || xy_row_stride > kMaxRowStride ||
+        xy_row_stride % 8 != 0)
+        return HAWK_ERR_BAD_SHAPE;
+    if (!aligned16(xy) || !aligned16(u) || !aligned16(x_rg_lru) || !aligned16(a_rg_lru) || !aligned16(w_i) ||
+        !aligned16(w_a) || !aligned16(out) || (h && !aligned16(h)) || (h_last && !aligned16(h_last)) ||
+        (w_bf16 && !aligned16(w_bf16)) || (scan_workspace && !aligned16(scan_workspace)))
+        return HAWK_ERR_ALIGNMENT;
+    return hawk::block_core_fwd(xy, xy_row_stride, conv_w, conv_b, w_i, b_i, w_a, b_a, w_dtype, w_bf16, a_param, u,
+                                x_rg_lru, a_rg_lru, h, out, h_last, B, T, D, num_blocks, scan_workspace,
+                                scan_workspace_bytes, as_stream(stream));
+}
+
+int hawk_block_core_bwd(const void* xy, long long xy_row_stride, const void* u, const void* x_rg_lru,
+                        const void* a_rg_lru, const void* h_saved, const float* conv_w, const void* w_i,
+                        const void* w_a, int w_dtype, const float* a_param, const void* grad_out, void* d_xy,
+                        long long d_xy_row_stride, void* du, void* d_x_rg_lru, void* d_a_rg_lru, float* d_conv_w,
+                        float* d_conv_b, float* dw_i, float* db_i, float* dw_a, float* db_a, float* da_param, int B,
+                        int T, int D, int num_blocks, int temporal_width, void* scan_workspace,
+                        size_t scan_workspace_bytes, void* gate_workspace, size_t gate_workspace_bytes,
+                        void* conv_workspace, size_t conv_workspace_bytes, void* stream) {
+    if (!xy || !u || !x_rg_lru || !a_rg_lru || !h_saved || !conv_w || !w_i || !w_a || !a_param || !grad_out || !d_xy ||
+        !du || !d_x_rg_lru || !d_a_rg_lru || !d_conv_w || !d_conv_b || !dw_i || !dw_a || !da_param)
+        return HAWK_ERR_NULL_POINTER;
+    if (!dtype_ok(w_dtype)) return HAWK_ERR_BAD_DTYPE;
+    if (int rc = check_scan_shape(B, T, D)) return rc;
+    if (temporal_width < 1 || temporal_width > 8 || B > kMaxGridY || !hawk_gate_proj_supported(D, num_blocks) ||
+        D % 8 != 0 || (long long)B * T > 0x7fffffffLL || xy_row_stride < 2LL * D || xy_row_stride > kMaxRowStride ||
+        xy_row_stride % 8 != 0 || d_xy_row_stride < 2LL * D || d_xy_row_stride > kMaxRowStride ||
+        d_xy_row_stride % 8 != 0)
+        return HAWK_ERR_BAD_SHAPE;
+    if (!aligned16(xy) || !aligned16(u) || !aligned16(x_rg_lru) || !aligned16(a_rg_lru) || !aligned16(h_saved) ||
+        !aligned16(w_i) || !aligned16(w_a) || !aligned16(grad_out) || !aligned16(d_xy) || !aligned16(du) ||
+        !aligned16(d_x_rg_lru) || !aligned16(d_a_rg_lru))
+        return HAWK_ERR_ALIGNMENT;
+    if (!scan_workspace || !gate_workspace || !conv_workspace) return HAWK_ERR_WORKSPACE;
+    if (!aligned16(scan_workspace) || !aligned16(gate_workspace) || !aligned16(conv_workspace))
+        return HAWK_ERR_ALIGNMENT;
+    return hawk::block_core_bwd(xy, xy_row_stride, u, x_rg_lru, a_rg_lru, h_saved, conv_w, w_i, w_a, w_dtype, a_param,
+                                grad_out, d_xy, d_xy_row_stride, du, d_x_rg_lru, d_a_rg_lru, d_conv_w, d_conv_b, dw_i,
+                                db_i, dw_a, db_a, da_param, B, T, D, num_blocks, temporal_width, scan_workspace,
+                                scan_workspace_bytes, gate_workspace, gate_workspace_bytes, conv_workspace,
+                                conv_workspace_bytes, as_stream(stream));
+}
+
 }  // extern "C"

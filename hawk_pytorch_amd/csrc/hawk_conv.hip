@@ -312,37 +312,10 @@ __global__ __launch_bounds__(256) void conv1d_bwd_anyw_kernel(
     prow[(size_t)W * D + c] = dbk;
 }
 
-// Column sums of a [rows, cols] fp32 matrix in a fixed order; the first n_first columns go
-// to out_first, the rest to out_second (dw then db).
-__global__ __launch_bounds__(1024) void colsum_kernel(const float* __restrict__ part, float* __restrict__ out_first,
-                                                     float* __restrict__ out_second, int rows, int cols,
-                                                     int n_first) {
+// Column sums of the [rows, (W + 1) D] partials in a fixed order: dw, then db.
+__global__ __launch_bounds__(kColsumThreads) void colsum_kernel(ColsumTask t) {
     __shared__ float s[16][kWave];
-    const int lane = threadIdx.x & (kWave - 1);
-    const int slice = threadIdx.x / kWave;
-    const int c = blockIdx.x * kWave + lane;
-    float sum = 0.0f;
-    if (c < cols) {
-        // eight independent loads in flight per thread; the order of additions is fixed
-        int r = slice;
-        for (; r + 16 * 7 < rows; r += 16 * 8) {
-            float v[8];
-#pragma unroll
-            for (int k = 0; k < 8; ++k) v[k] = part[(size_t)(r + 16 * k) * cols + c];
-#pragma unroll
-            for (int k = 0; k < 8; ++k) sum += v[k];
-        }
-        for (; r < rows; r += 16) sum += part[(size_t)r * cols + c];
-    }
-    s[slice][lane] = sum;
-    __syncthreads();
-    if (slice == 0 && c < cols) {
-        float tot = 0.0f;
-#pragma unroll
-        for (int k = 0; k < 16; ++k) tot += s[k][lane];
-        if (c < n_first) out_first[c] = tot;
-        else out_second[c - n_first] = tot;
-    }
+    colsum_block(t, (int)blockIdx.x, s);
 }
 
 // Channels per lane: every row of every tensor must start on a multiple of it.
@@ -400,7 +373,7 @@ BwdPlan bwd_plan(int T, int W) {
 
 template <typename XT, typename GT>
 int bwd_dispatch(const void* gy, const void* x, const float* w, void* dx, float* dw, float* db, int B, int T, int D,
-                 int W, size_t ldx, size_t lddx, float* part, hipStream_t st) {
+                 int W, size_t ldx, size_t lddx, float* part, hipStream_t st, ColsumTask* deferred) {
     const GT* gp = static_cast<const GT*>(gy);
     const XT* xp = static_cast<const XT*>(x);
     XT* dxp = static_cast<XT*>(dx);
@@ -417,9 +390,12 @@ int bwd_dispatch(const void* gy, const void* x, const float* w, void* dx, float*
         hipLaunchKernelGGL((conv1d_bwd_anyw_kernel<XT, GT>), grid, block, 0, st, gp, xp, w, dxp, part, T, D, W, p.rows_per_group, ldx, lddx);
     }
     if (hipGetLastError() != hipSuccess) return HAWK_ERR_LAUNCH;
-    const int cols = (W + 1) * D;
-    hipLaunchKernelGGL(colsum_kernel, dim3((unsigned)ceil_div(cols, kWave)), dim3(1024), 0, st, part, dw, db,
-                       p.ngroups * B, cols, W * D);
+    const ColsumTask reduce{part, dw, db, nullptr, p.ngroups * B, (W + 1) * D, W * D};
+    if (deferred != nullptr) {   // the caller runs it, together with its other closing reductions
+        *deferred = reduce;
+        return HAWK_OK;
+    }
+    hipLaunchKernelGGL(colsum_kernel, dim3((unsigned)reduce.blocks()), dim3(kColsumThreads), 0, st, reduce);
     return hipGetLastError() == hipSuccess ? HAWK_OK : HAWK_ERR_LAUNCH;
 }
 
@@ -443,17 +419,17 @@ size_t conv1d_bwd_workspace_bytes(int B, int T, int D, int W) {
 
 int conv1d_bwd(const void* gy, const void* x, long long ldx, const float* w, void* dx, long long lddx, float* dw,
                float* db, int B, int T, int D, int W, int x_dtype, int gy_dtype, void* ws, size_t ws_bytes,
-               hipStream_t st) {
+               hipStream_t st, ColsumTask* deferred) {
     if (ws == nullptr || ws_bytes < conv1d_bwd_workspace_bytes(B, T, D, W)) return HAWK_ERR_WORKSPACE;
     float* part = static_cast<float*>(ws);
     const size_t lx = (size_t)ldx, ld = (size_t)lddx;
     if (x_dtype == HAWK_DTYPE_BF16) {
         if (gy_dtype == HAWK_DTYPE_BF16)
-            return bwd_dispatch<bf16_t, bf16_t>(gy, x, w, dx, dw, db, B, T, D, W, lx, ld, part, st);
-        return bwd_dispatch<bf16_t, float>(gy, x, w, dx, dw, db, B, T, D, W, lx, ld, part, st);
+            return bwd_dispatch<bf16_t, bf16_t>(gy, x, w, dx, dw, db, B, T, D, W, lx, ld, part, st, deferred);
+        return bwd_dispatch<bf16_t, float>(gy, x, w, dx, dw, db, B, T, D, W, lx, ld, part, st, deferred);
     }
-    if (gy_dtype == HAWK_DTYPE_BF16) return bwd_dispatch<float, bf16_t>(gy, x, w, dx, dw, db, B, T, D, W, lx, ld, part, st);
-    return bwd_dispatch<float, float>(gy, x, w, dx, dw, db, B, T, D, W, lx, ld, part, st);
+    if (gy_dtype == HAWK_DTYPE_BF16) return bwd_dispatch<float, bf16_t>(gy, x, w, dx, dw, db, B, T, D, W, lx, ld, part, st, deferred);
+    return bwd_dispatch<float, float>(gy, x, w, dx, dw, db, B, T, D, W, lx, ld, part, st, deferred);
 }
 
 }  // namespace hawk

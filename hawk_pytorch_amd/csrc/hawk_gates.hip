@@ -1291,27 +1291,8 @@ __global__ __launch_bounds__(kGateThreads, 1) void gate_proj_bwd_weights_kernel(
 }
 
 // dw_g = sum over splits of the partial tiles, db_g likewise; fixed order.
-__global__ void gate_proj_reduce_kernel(const float* __restrict__ part_w, const float* __restrict__ part_b,
-                                        float* __restrict__ dw_i, float* __restrict__ dw_a, float* __restrict__ db_i,
-                                        float* __restrict__ db_a, int nsplit, size_t wcount, int D) {
-    const size_t total = 2 * wcount + 2 * (size_t)D;
-    for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
-         idx += (size_t)gridDim.x * blockDim.x) {
-        float sum = 0.0f;
-        if (idx < 2 * wcount) {
-            for (int s = 0; s < nsplit; ++s) sum += part_w[(size_t)s * 2 * wcount + idx];
-            if (idx < wcount) dw_i[idx] = sum;
-            else dw_a[idx - wcount] = sum;
-        } else {
-            const size_t k = idx - 2 * wcount;
-            for (int s = 0; s < nsplit; ++s) sum += part_b[(size_t)s * 2 * D + k];
-            if (k < (size_t)D) {
-                if (db_i != nullptr) db_i[k] = sum;
-            } else if (db_a != nullptr) {
-                db_a[k - D] = sum;
-            }
-        }
-    }
+__global__ void gate_proj_reduce_kernel(GateReduceTask t) {
+    gate_reduce_span(t, (size_t)blockIdx.x * blockDim.x + threadIdx.x, (size_t)gridDim.x * blockDim.x);
 }
 
 inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
@@ -1658,7 +1639,7 @@ size_t gate_proj_bwd_weights_workspace_bytes(int M, int D, int nb) {
 
 int gate_proj_bwd_weights(const void* x, const void* dg_i, const void* dg_a, float* dw_i, float* db_i, float* dw_a,
                           float* db_a, int M, int D, int nb, int x_dtype, int g_dtype, void* ws, size_t ws_bytes,
-                          hipStream_t st) {
+                          hipStream_t st, GateReduceTask* deferred) {
     const int bw = D / nb;
     const int nsplit = weight_splits(M, D);
     const size_t wcount = (size_t)nb * bw * bw;
@@ -1676,11 +1657,14 @@ int gate_proj_bwd_weights(const void* x, const void* dg_i, const void* dg_a, flo
                  : gate_bwd_weights_bw<float, float>(x, dg_i, dg_a, part_w, part_b, M, D, nb, bw, nsplit, st);
     }
     if (rc != HAWK_OK) return rc;
-    const size_t total = 2 * wcount + 2 * (size_t)D;
-    size_t blocks = (total + 255) / 256;
+    const GateReduceTask reduce{part_w, part_b, dw_i, dw_a, db_i, db_a, nsplit, D, wcount};
+    if (deferred != nullptr) {   // the caller runs it, together with its other closing reductions
+        *deferred = reduce;
+        return HAWK_OK;
+    }
+    size_t blocks = (reduce.items() + 255) / 256;
     if (blocks > 4096) blocks = 4096;
-    hipLaunchKernelGGL(gate_proj_reduce_kernel, dim3((unsigned)blocks), dim3(256), 0, st, part_w, part_b, dw_i, dw_a,
-                       db_i, db_a, nsplit, wcount, D);
+    hipLaunchKernelGGL(gate_proj_reduce_kernel, dim3((unsigned)blocks), dim3(256), 0, st, reduce);
     return hipGetLastError() == hipSuccess ? HAWK_OK : HAWK_ERR_LAUNCH;
 }
 

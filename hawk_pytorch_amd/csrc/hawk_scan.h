@@ -5,8 +5,13 @@
 #include <stddef.h>
 
 #include "../../include/hawk_hip.h"
+#include "hawk_reduce.h"
 
 namespace hawk {
+
+// The backward entry points below that take a `deferred` pointer end in a small reduction of
+// per-tile partial sums; with the pointer set they hand its description back instead of
+// launching it, and the caller runs it (block_core_bwd: three of them in one launch).
 
 // hawk_scan.hip
 size_t scan_workspace_bytes(int B, int T, int D, int dtype);
@@ -33,7 +38,7 @@ int scan_gated_fwd(const void* x, const void* xg, const void* ag, const float* l
 int scan_gated_bwd(const void* x, const void* xg, const void* ag, const float* lam, const void* y, long long ldy,
                    const void* hs, const void* gout, void* dx, void* dxg, void* dag, void* dy, long long lddy,
                    float* dlam, int B, int T, int D, int in_dtype, int state_dtype, void* ws, size_t ws_bytes,
-                   hipStream_t st);
+                   hipStream_t st, ColsumTask* deferred = nullptr);
 
 // hawk_conv.hip
 // ldx, ldy, lddx: row strides in elements (>= D); batch rows lie T rows apart
@@ -42,7 +47,7 @@ int conv1d_fwd(const void* x, long long ldx, const float* w, const float* bias, 
 size_t conv1d_bwd_workspace_bytes(int B, int T, int D, int W);
 int conv1d_bwd(const void* gy, const void* x, long long ldx, const float* w, void* dx, long long lddx, float* dw,
                float* db, int B, int T, int D, int W, int x_dtype, int gy_dtype, void* ws, size_t ws_bytes,
-               hipStream_t st);
+               hipStream_t st, ColsumTask* deferred = nullptr);
 
 // hawk_step.hip
 int conv1d_step(void* conv_state, const void* x_new, const float* w, const float* bias, void* y, int B, int D,
@@ -76,6 +81,24 @@ size_t decode_core_workspace_bytes(int B, int D, int nb);
 size_t gate_proj_bwd_weights_workspace_bytes(int M, int D, int nb);
 int gate_proj_bwd_weights(const void* x, const void* dg_i, const void* dg_a, float* dw_i, float* db_i, float* dw_a,
                           float* db_a, int M, int D, int nb, int x_dtype, int g_dtype, void* ws, size_t ws_bytes,
-                          hipStream_t st);
+                          hipStream_t st, GateReduceTask* deferred = nullptr);
+
+// hawk_block.hip
+// two fp32 arrays of `count` elements (a multiple of 4) rounded to bf16 by one launch
+int gate_weights_to_bf16(const float* w_i, const float* w_a, void* w_i16, void* w_a16, size_t count, hipStream_t st);
+// conv + both projections + gated scan on the [B,T,2D] bf16 projection output xy (rows ld elements
+// apart: x half, then y half).  fp32 weights are rounded once into w16 ([2][nb][bw][bw] bf16) when
+// it is not NULL, and the kernels read those.
+int block_core_fwd(const void* xy, long long ld, const float* conv_w, const float* conv_b, const void* w_i,
+                   const float* b_i, const void* w_a, const float* b_a, int w_dtype, void* w16, const float* lam,
+                   void* u, void* xg, void* ag, void* h, void* out, void* h_last, int B, int T, int D, int nb,
+                   void* scan_ws, size_t scan_ws_bytes, hipStream_t st);
+// The backward of all of it; du, dxg, dag: [B,T,D] bf16 scratch for the gradients in between.
+int block_core_bwd(const void* xy, long long ld, const void* u, const void* xg, const void* ag, const void* h,
+                   const float* conv_w, const void* w_i, const void* w_a, int w_dtype, const float* lam,
+                   const void* gout, void* d_xy, long long ldd, void* du, void* dxg, void* dag, float* d_conv_w,
+                   float* d_conv_b, float* dw_i, float* db_i, float* dw_a, float* db_a, float* dlam, int B, int T,
+                   int D, int nb, int W, void* scan_ws, size_t scan_ws_bytes, void* gate_ws, size_t gate_ws_bytes,
+                   void* conv_ws, size_t conv_ws_bytes, hipStream_t st);
 
 }  // namespace hawk

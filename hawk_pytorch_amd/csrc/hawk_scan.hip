@@ -727,34 +727,9 @@ __global__ __launch_bounds__(NW * kWave, HAWK_BWD_WAVES_PER_SIMD) void rglru_sca
 // dLambda[c] = -8 sigmoid(Lambda_c) * sum over rows of the [rows, D] partials.
 // 64 channels x 16 row slices per block; fixed summation order, so the result is
 // reproducible run to run.
-__global__ __launch_bounds__(1024) void dlam_reduce_kernel(const float* __restrict__ part,
-                                                          const float* __restrict__ lam,
-                                                          float* __restrict__ dlam, int rows, int D) {
+__global__ __launch_bounds__(kColsumThreads) void dlam_reduce_kernel(ColsumTask t) {
     __shared__ float s[16][kWave];
-    const int lane = threadIdx.x & (kWave - 1);
-    const int slice = threadIdx.x / kWave;
-    const int c = blockIdx.x * kWave + lane;
-    float sum = 0.0f;
-    if (c < D) {
-        // eight independent loads in flight per thread; the order of additions is fixed
-        int r = slice;
-        for (; r + 16 * 7 < rows; r += 16 * 8) {
-            float v[8];
-#pragma unroll
-            for (int k = 0; k < 8; ++k) v[k] = part[(size_t)(r + 16 * k) * D + c];
-#pragma unroll
-            for (int k = 0; k < 8; ++k) sum += v[k];
-        }
-        for (; r < rows; r += 16) sum += part[(size_t)r * D + c];
-    }
-    s[slice][lane] = sum;
-    __syncthreads();
-    if (slice == 0 && c < D) {
-        float tot = 0.0f;
-#pragma unroll
-        for (int k = 0; k < 16; ++k) tot += s[k][lane];
-        dlam[c] = -8.0f * sigmoid_precise(lam[c]) * tot;
-    }
+    colsum_block(t, (int)blockIdx.x, s);
 }
 
 __global__ void fill_u32_kernel(uint32_t* p, size_t n, uint32_t v) {
@@ -893,6 +868,7 @@ struct GateBwdHost {
     const void* y = nullptr;
     void* dy = nullptr;
     uint32_t ldy = 0, lddy = 0;
+    ColsumTask* deferred = nullptr;   // not NULL: receives the dLambda reduction instead of a launch
 };
 
 template <typename IT, typename OT, int V, int TC, int NW, bool PRECISE, bool GATED>
@@ -990,8 +966,12 @@ int scan_bwd_shaped(const void* x, const void* xg, const void* ag, const float* 
                                                                   nseg, nct, p, st);
     }
     if (rc != HAWK_OK) return rc;
-    hipLaunchKernelGGL(dlam_reduce_kernel, dim3((unsigned)ceil_div(D, kWave)), dim3(1024), 0, st, p.dlam_part, lam,
-                       dlam, nseg * B, D);
+    const ColsumTask reduce{p.dlam_part, dlam, nullptr, lam, nseg * B, D, D};
+    if (g.deferred != nullptr) {   // the caller runs it, together with its other closing reductions
+        *g.deferred = reduce;
+        return HAWK_OK;
+    }
+    hipLaunchKernelGGL(dlam_reduce_kernel, dim3((unsigned)reduce.blocks()), dim3(kColsumThreads), 0, st, reduce);
     return hipGetLastError() == hipSuccess ? HAWK_OK : HAWK_ERR_LAUNCH;
 }
 
@@ -1142,12 +1122,13 @@ int scan_gated_fwd(const void* x, const void* xg, const void* ag, const float* l
 int scan_gated_bwd(const void* x, const void* xg, const void* ag, const float* lam, const void* y, long long ldy,
                    const void* hs, const void* gout, void* dx, void* dxg, void* dag, void* dy, long long lddy,
                    float* dlam, int B, int T, int D, int in_dtype, int state_dtype, void* ws, size_t ws_bytes,
-                   hipStream_t st) {
+                   hipStream_t st, ColsumTask* deferred) {
     GateBwdHost g;
     g.y = y;
     g.dy = dy;
     g.ldy = (uint32_t)ldy;
     g.lddy = (uint32_t)lddy;
+    g.deferred = deferred;
     return scan_bwd_impl<true>(x, xg, ag, lam, hs, gout, dx, dxg, dag, dlam, g, B, T, D, in_dtype, state_dtype, ws,
                                ws_bytes, st);
 }

@@ -489,6 +489,16 @@ _CAST_WEIGHTS_MIN_ROWS = 8192
 
 def kernel_weights(w_i: torch.Tensor, w_a: torch.Tensor, rows: int):
     if w_i.dtype == torch.float32 and rows >= _CAST_WEIGHTS_MIN_ROWS:
+        nb, bw, _ = w_i.shape
+        if w_i.is_cuda and w_a.dtype == torch.float32 and w_a.shape == w_i.shape and bw % 4 == 0:
+            # both gates in one launch
+            wi, wa = _lib.dense16(w_i.detach()), _lib.dense16(w_a.detach())
+            both = torch.empty((2, nb, bw, bw), dtype=torch.bfloat16, device=w_i.device)
+            with torch.cuda.device(w_i.device):
+                _lib.check("hawk_gate_weights_to_bf16", _lib.load().hawk_gate_weights_to_bf16(
+                    wi.data_ptr(), wa.data_ptr(), both[0].data_ptr(), both[1].data_ptr(), nb, bw,
+                    _lib.stream_ptr(w_i.device)))
+            return both[0], both[1]
         return w_i.detach().to(torch.bfloat16), w_a.detach().to(torch.bfloat16)
     return w_i, w_a
 

@@ -512,10 +512,12 @@ def _launch_block_core_fwd(xy, conv_w, conv_b, w_i, b_i, w_a, b_a, lam, want_h: 
     with torch.cuda.device(dev):
         st = _lib.stream_ptr(dev)
         if W == 4 and T >= _FUSED_CONV_MIN_T:
-            _lib.check("hawk_conv_gate_proj_fwd", lib.hawk_conv_gate_proj_fwd(
+            # conv + both projections, then the gated scan: one host call
+            _lib.check("hawk_block_core_fwd", lib.hawk_block_core_fwd(
                 xy.data_ptr(), ld, conv_w.data_ptr(), conv_b.data_ptr(), w_i.data_ptr(), b_i.data_ptr(),
-                w_a.data_ptr(), b_a.data_ptr(), u.data_ptr(), xg.data_ptr(), ag.data_ptr(), B, T, D, nb, W,
-                _lib.dtype_code(w_i.dtype), st))
+                w_a.data_ptr(), b_a.data_ptr(), _lib.dtype_code(w_i.dtype), None, lam.data_ptr(), u.data_ptr(),
+                xg.data_ptr(), ag.data_ptr(), h.data_ptr() if want_h else None, out.data_ptr(),
+                h_last.data_ptr() if want_last else None, B, T, D, nb, W, ws.data_ptr(), ws.numel(), st))
         else:
             _lib.check("hawk_conv1d_fwd_strided", lib.hawk_conv1d_fwd_strided(
                 xy.data_ptr(), ld, conv_w.data_ptr(), conv_b.data_ptr(), None, u.data_ptr(), D, B, T, D, W, code,
@@ -523,10 +525,10 @@ def _launch_block_core_fwd(xy, conv_w, conv_b, w_i, b_i, w_a, b_a, lam, want_h: 
             _lib.check("hawk_gate_proj_fwd", lib.hawk_gate_proj_fwd(
                 u.data_ptr(), w_i.data_ptr(), b_i.data_ptr(), w_a.data_ptr(), b_a.data_ptr(), xg.data_ptr(),
                 ag.data_ptr(), B * T, D, nb, code, _lib.dtype_code(w_i.dtype), code, st))
-        _lib.check("hawk_rglru_scan_gated_fwd", lib.hawk_rglru_scan_gated_fwd(
-            u.data_ptr(), xg.data_ptr(), ag.data_ptr(), lam.data_ptr(), y_ptr, ld,
-            h.data_ptr() if want_h else None, out.data_ptr(), h_last.data_ptr() if want_last else None,
-            B, T, D, code, code, ws.data_ptr(), ws.numel(), st))
+            _lib.check("hawk_rglru_scan_gated_fwd", lib.hawk_rglru_scan_gated_fwd(
+                u.data_ptr(), xg.data_ptr(), ag.data_ptr(), lam.data_ptr(), y_ptr, ld,
+                h.data_ptr() if want_h else None, out.data_ptr(), h_last.data_ptr() if want_last else None,
+                B, T, D, code, code, ws.data_ptr(), ws.numel(), st))
     return out, u, xg, ag, h, h_last
 
 
@@ -554,27 +556,16 @@ def _launch_block_core_bwd(xy, u, xg, ag, h, conv_w, w_i, w_a, lam, grad_out):
     ws = _lib.scan_workspace(dev, lib.hawk_scan_workspace_bytes(B, T, D, code))
     gws = _gate_workspace(dev, lib.hawk_gate_proj_bwd_weights_workspace_bytes(M, D, nb))
     cws = torch.empty(lib.hawk_conv1d_bwd_workspace_bytes(B, T, D, W), dtype=torch.uint8, device=dev)
-    y_ptr = xy.data_ptr() + D * xy.element_size()
-    dy_ptr = d_xy.data_ptr() + D * d_xy.element_size()
-    wcode = _lib.dtype_code(w_i.dtype)
     with torch.cuda.device(dev):
-        st = _lib.stream_ptr(dev)
-        _lib.check("hawk_rglru_scan_gated_bwd", lib.hawk_rglru_scan_gated_bwd(
-            u.data_ptr(), xg.data_ptr(), ag.data_ptr(), lam.data_ptr(), y_ptr, ld, h.data_ptr(),
-            grad_out.data_ptr(), du.data_ptr(), dxg.data_ptr(), dag.data_ptr(), dy_ptr, D2, dlam.data_ptr(),
-            B, T, D, code, code, ws.data_ptr(), ws.numel(), st))
-        # the projections' input gradient accumulates onto the scan's, in place
-        _lib.check("hawk_gate_proj_bwd_input", lib.hawk_gate_proj_bwd_input(
-            dxg.data_ptr(), dag.data_ptr(), w_i.data_ptr(), w_a.data_ptr(), du.data_ptr(), du.data_ptr(), M, D, nb,
-            code, wcode, code, st))
-        # the conv's backward right behind the kernel that wrote its input gradient (part of it is
-        # then still in the memory-side cache), the weight gradients last
-        _lib.check("hawk_conv1d_bwd_strided", lib.hawk_conv1d_bwd_strided(
-            du.data_ptr(), xy.data_ptr(), ld, conv_w.data_ptr(), d_xy.data_ptr(), D2, dcw.data_ptr(),
-            dcb.data_ptr(), B, T, D, W, code, code, cws.data_ptr(), cws.numel(), st))
-        _lib.check("hawk_gate_proj_bwd_weights", lib.hawk_gate_proj_bwd_weights(
-            u.data_ptr(), dxg.data_ptr(), dag.data_ptr(), dw_i.data_ptr(), db_i.data_ptr(), dw_a.data_ptr(),
-            db_a.data_ptr(), M, D, nb, code, code, gws.data_ptr(), gws.numel(), st))
+        # scan (with the output gate) -> projections' input gradient onto the scan's, in place ->
+        # conv -> projections' weight gradients, and one launch for the three closing reductions
+        _lib.check("hawk_block_core_bwd", lib.hawk_block_core_bwd(
+            xy.data_ptr(), ld, u.data_ptr(), xg.data_ptr(), ag.data_ptr(), h.data_ptr(), conv_w.data_ptr(),
+            w_i.data_ptr(), w_a.data_ptr(), _lib.dtype_code(w_i.dtype), lam.data_ptr(), grad_out.data_ptr(),
+            d_xy.data_ptr(), D2, du.data_ptr(), dxg.data_ptr(), dag.data_ptr(), dcw.data_ptr(), dcb.data_ptr(),
+            dw_i.data_ptr(), db_i.data_ptr(), dw_a.data_ptr(), db_a.data_ptr(), dlam.data_ptr(), B, T, D, nb, W,
+            ws.data_ptr(), ws.numel(), gws.data_ptr(), gws.numel(), cws.data_ptr(), cws.numel(),
+            _lib.stream_ptr(dev)))
     return d_xy, dcw, dcb, dw_i, db_i, dw_a, db_a, dlam
 
 

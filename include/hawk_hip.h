@@ -351,6 +351,55 @@ int hawk_gate_proj_bwd_weights(const void* x, const void* d_x_rg_lru, const void
                                int num_blocks, int x_dtype, int g_dtype, void* workspace_device,
                                size_t workspace_bytes, void* stream);
 
+/* ---------------------------------------------------------------------------------------
+ * The recurrent core of a block as one call per direction.
+ * Hawk.forward between the input projection and the output projection (hawk/hawk.py:169-198:
+ * Conv1D, the two BlockDiagonalLinear gates, rnn_scan / the fused scan, gelu(y) * h) on the
+ * projection's output xy [B,T,2D] bf16 in place (x half, then y half; rows xy_row_stride >= 2D
+ * elements apart, a multiple of 8; D a multiple of 8).  The kernels and the results are those of
+ * hawk_conv_gate_proj_fwd + hawk_rglru_scan_gated_fwd and of hawk_rglru_scan_gated_bwd +
+ * hawk_gate_proj_bwd_input (onto the scan's dx, in place) + hawk_conv1d_bwd_strided +
+ * hawk_gate_proj_bwd_weights, bit for bit; what the single calls cannot do is share their small
+ * launches: here fp32 gate weights are rounded to bf16 by one launch for both gates, and the three
+ * closing reductions of the backward run as one launch.
+ * ------------------------------------------------------------------------------------- */
+
+/* fp32 -> bf16 (round to nearest even) of both gates' weights [num_blocks, bw, bw] in one launch;
+ * bw a multiple of 4.  What `w.to(torch.bfloat16)` gives, twice. */
+int hawk_gate_weights_to_bf16(const float* w_i, const float* w_a, void* w_i_bf16, void* w_a_bf16,
+                              int num_blocks, int block_width, void* stream);
+
+/* Forward.  Gate weights have w_dtype; when they are fp32 and w_bf16 is not NULL, they are first
+ * rounded into w_bf16 ([2][num_blocks][bw][bw] bf16: w_i, then w_a), which the kernels then read
+ * and which hawk_block_core_bwd can be handed as its weights (w_dtype bf16).  u, x_rg_lru,
+ * a_rg_lru, out [B,T,D] bf16 dense; h [B,T,D] bf16 and h_last [B,D] bf16 may be NULL (h is what
+ * the backward needs).  temporal_width must be 4 and T >= 32 (HAWK_ERR_BAD_SHAPE otherwise: use
+ * the single calls).  scan_workspace as for hawk_rglru_scan_fwd. */
+int hawk_block_core_fwd(const void* xy, long long xy_row_stride, const float* conv_w,
+                        const float* conv_b, const void* w_i, const float* b_i, const void* w_a,
+                        const float* b_a, int w_dtype, void* w_bf16, const float* a_param, void* u,
+                        void* x_rg_lru, void* a_rg_lru, void* h, void* out, void* h_last, int B, int T,
+                        int D, int num_blocks, int temporal_width, void* scan_workspace,
+                        size_t scan_workspace_bytes, void* stream);
+
+/* Backward.  grad_out [B,T,D] bf16 dense; d_xy [B,T,2D] bf16 (rows d_xy_row_stride elements
+ * apart) receives both halves; du, d_x_rg_lru, d_a_rg_lru [B,T,D] bf16 are the caller's scratch
+ * for the gradients in between (du ends as the gradient of the conv output).  d_conv_w
+ * [temporal_width, D], d_conv_b [D], dw_i, dw_a [num_blocks, bw, bw], db_i, db_a [D] (may be
+ * NULL), da_param [D]: fp32, overwritten.  The three workspaces are those of the single calls
+ * (hawk_scan_workspace_bytes, hawk_gate_proj_bwd_weights_workspace_bytes,
+ * hawk_conv1d_bwd_workspace_bytes). */
+int hawk_block_core_bwd(const void* xy, long long xy_row_stride, const void* u, const void* x_rg_lru,
+                        const void* a_rg_lru, const void* h_saved, const float* conv_w,
+                        const void* w_i, const void* w_a, int w_dtype, const float* a_param,
+                        const void* grad_out, void* d_xy, long long d_xy_row_stride, void* du,
+                        void* d_x_rg_lru, void* d_a_rg_lru, float* d_conv_w, float* d_conv_b,
+                        float* dw_i, float* db_i, float* dw_a, float* db_a, float* da_param, int B, int T,
+                        int D, int num_blocks, int temporal_width, void* scan_workspace,
+                        size_t scan_workspace_bytes, void* gate_workspace,
+                        size_t gate_workspace_bytes, void* conv_workspace,
+                        size_t conv_workspace_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -315,3 +315,65 @@ def gate_proj_bwd_weights(x, dxg, dag, nb, with_bias=True):
         M, D, nb, _lib.dtype_code(x.dtype), _lib.dtype_code(dxg.dtype), ws.data_ptr(), n, _stream())
     _lib.check("hawk_gate_proj_bwd_weights", rc)
     return dwi, dbi, dwa, dba
+
+
+def gate_weights_to_bf16(w_i, w_a):
+    nb, bw, _ = w_i.shape
+    oi, oa = (torch.empty((nb, bw, bw), dtype=torch.bfloat16, device="cuda") for _ in range(2))
+    rc = _lib.load().hawk_gate_weights_to_bf16(w_i.data_ptr(), w_a.data_ptr(), oi.data_ptr(), oa.data_ptr(), nb, bw,
+                                               _stream())
+    _lib.check("hawk_gate_weights_to_bf16", rc)
+    return oi, oa
+
+
+def block_core_fwd(xy, conv_w, conv_b, w_i, b_i, w_a, b_a, lam, round_weights=True, want_h=True, want_last=True,
+                   ws=None):
+    """xy [B,T,2D] bf16 with unit channel stride and dense batch/time.  Returns
+    (out, u, xg, ag, h or None, h_last or None, w16 or None)."""
+    B, T, D2 = xy.shape
+    D = D2 // 2
+    assert xy.stride(2) == 1 and xy.stride(0) == T * xy.stride(1)
+    nb, bw, _ = w_i.shape
+    e = lambda: torch.empty((B, T, D), dtype=torch.bfloat16, device="cuda")  # noqa: E731
+    u, xg, ag, out = e(), e(), e(), e()
+    h = e() if want_h else None
+    h_last = torch.full((B, D), float("nan"), dtype=torch.bfloat16, device="cuda") if want_last else None
+    w16 = None
+    if round_weights and w_i.dtype == torch.float32:
+        w16 = torch.full((2, nb, bw, bw), float("nan"), dtype=torch.bfloat16, device="cuda")
+    if ws is None:
+        ws = new_workspace(B, T, D, "bf16")
+    rc = _lib.load().hawk_block_core_fwd(
+        xy.data_ptr(), xy.stride(1), conv_w.data_ptr(), conv_b.data_ptr(), w_i.data_ptr(), _lib.ptr(b_i),
+        w_a.data_ptr(), _lib.ptr(b_a), _lib.dtype_code(w_i.dtype), _lib.ptr(w16), lam.data_ptr(), u.data_ptr(),
+        xg.data_ptr(), ag.data_ptr(), _lib.ptr(h), out.data_ptr(), _lib.ptr(h_last), B, T, D, nb, conv_w.shape[0],
+        ws.data_ptr(), ws.numel(), _stream())
+    _lib.check("hawk_block_core_fwd", rc)
+    return out, u, xg, ag, h, h_last, w16
+
+
+def block_core_bwd(xy, u, xg, ag, h, conv_w, w_i, w_a, lam, gout, with_bias=True, ws=None):
+    """Returns (d_xy, d_conv_w, d_conv_b, dw_i, db_i, dw_a, db_a, dlam, du)."""
+    B, T, D2 = xy.shape
+    D = D2 // 2
+    nb, bw, _ = w_i.shape
+    W = conv_w.shape[0]
+    lib = _lib.load()
+    d_xy = torch.full((B, T, D2), float("nan"), dtype=torch.bfloat16, device="cuda")
+    du, dxg, dag = (torch.empty((B, T, D), dtype=torch.bfloat16, device="cuda") for _ in range(3))
+    f = lambda *s: torch.full(s, float("nan"), dtype=torch.float32, device="cuda")  # noqa: E731
+    dcw, dcb, dwi, dwa, dlam = f(W, D), f(D), f(nb, bw, bw), f(nb, bw, bw), f(D)
+    dbi, dba = (f(D), f(D)) if with_bias else (None, None)
+    if ws is None:
+        ws = new_workspace(B, T, D, "bf16")
+    garbage = lambda n: torch.full((max(n, 16),), 0xAB, dtype=torch.uint8, device="cuda")  # noqa: E731
+    gws = garbage(lib.hawk_gate_proj_bwd_weights_workspace_bytes(B * T, D, nb))
+    cws = garbage(lib.hawk_conv1d_bwd_workspace_bytes(B, T, D, W))
+    rc = lib.hawk_block_core_bwd(
+        xy.data_ptr(), xy.stride(1), u.data_ptr(), xg.data_ptr(), ag.data_ptr(), h.data_ptr(), conv_w.data_ptr(),
+        w_i.data_ptr(), w_a.data_ptr(), _lib.dtype_code(w_i.dtype), lam.data_ptr(), gout.data_ptr(), d_xy.data_ptr(),
+        D2, du.data_ptr(), dxg.data_ptr(), dag.data_ptr(), dcw.data_ptr(), dcb.data_ptr(), dwi.data_ptr(),
+        _lib.ptr(dbi), dwa.data_ptr(), _lib.ptr(dba), dlam.data_ptr(), B, T, D, nb, W, ws.data_ptr(), ws.numel(),
+        gws.data_ptr(), gws.numel(), cws.data_ptr(), cws.numel(), _stream())
+    _lib.check("hawk_block_core_bwd", rc)
+    return d_xy, dcw, dcb, dwi, dbi, dwa, dba, dlam, du
