@@ -196,6 +196,30 @@ def cpu_baseline(B, D, lo, hi, seed, budget_elements=1024 * 8 * 2560):
     }
 
 
+ALLOCATION = {
+    False: "every tensor placed as the library's host code places the activations it allocates: base addresses "
+           "256 bytes apart modulo 1 KiB (hawk_pytorch_amd._lib.activation_empty); --plain-alloc for torch.empty",
+    True: "plain torch.empty (large blocks start on 2 MiB boundaries)",
+}
+
+
+def act_empty(args, shape, dtype, dev):
+    """An activation tensor placed as the library's host code places the ones it allocates (base
+    addresses 256 bytes apart modulo 1 KiB, hawk_pytorch_amd._lib.activation_empty), or by a
+    plain torch.empty with --plain-alloc."""
+    from hawk_pytorch_amd import _lib
+
+    if args.plain_alloc:
+        return torch.empty(shape, dtype=dtype, device=dev)
+    return _lib.activation_empty(shape, dtype, dev)
+
+
+def act_randn(args, shape, dtype, dev, gen):
+    t = act_empty(args, shape, dtype, dev)
+    t.copy_(torch.randn(shape, device=dev, generator=gen).to(dtype))
+    return t
+
+
 def run_gates(args, lib, dev):
     """Both gate projections of a layer on B*T = 32768 tokens: forward, dx, dw/db."""
     from hawk_pytorch_amd import _lib
@@ -204,10 +228,10 @@ def run_gates(args, lib, dev):
     bw = D // nb
     bf, code, f32 = torch.bfloat16, _lib.HAWK_DTYPE_BF16, _lib.HAWK_DTYPE_F32
     gen = torch.Generator(device=dev).manual_seed(args.seed)
-    x, gi, ga = (torch.randn(M, D, device=dev, generator=gen).to(bf) for _ in range(3))
+    x, gi, ga = (act_randn(args, (M, D), bf, dev, gen) for _ in range(3))
     wi, wa = (torch.randn(nb, bw, bw, device=dev, generator=gen) / bw ** 0.5 for _ in range(2))
     bi, ba = (torch.randn(D, device=dev, generator=gen) for _ in range(2))
-    oi, oa, dx = torch.empty_like(x), torch.empty_like(x), torch.empty_like(x)
+    oi, oa, dx = (act_empty(args, (M, D), bf, dev) for _ in range(3))
     dwi, dwa = torch.empty_like(wi), torch.empty_like(wa)
     dbi, dba = torch.empty_like(bi), torch.empty_like(ba)
     nws = lib.hawk_gate_proj_bwd_weights_workspace_bytes(M, D, nb)
@@ -285,7 +309,7 @@ def run_gates(args, lib, dev):
         "config": {"workload": f"gates: both block-diagonal gate projections fwd + input grad + weight grads, "
                                f"M={M}, D={D}, {nb} blocks of {bw}, bf16, fp32 weights "
                                + ("rounded to bf16 once per step" if cast else "rounded by every workgroup"),
-                   "M": M, "D": D, "num_blocks": nb},
+                   "M": M, "D": D, "num_blocks": nb, "allocation": ALLOCATION[bool(args.plain_alloc)]},
         "roofline": {
             "bound": "hbm",
             "kernel": "gate_proj_bwd_weights_kernel (+ gate_proj_reduce_kernel, same launch call)",
@@ -308,19 +332,19 @@ def run_block(args, lib, dev):
     M, bw, N = B * T, D // nb, B * T * D
     bf, code = torch.bfloat16, _lib.HAWK_DTYPE_BF16
     gen = torch.Generator(device=dev).manual_seed(args.seed)
-    xy = torch.randn(B, T, 2 * D, device=dev, generator=gen).to(bf)
+    xy = act_randn(args, (B, T, 2 * D), bf, dev, gen)
     xin = xy[..., :D].contiguous()          # conv input; the gate half stays in place
     y = xy[..., D:]
-    gout = torch.randn(B, T, D, device=dev, generator=gen).to(bf)
+    gout = act_randn(args, (B, T, D), bf, dev, gen)
     cw = (torch.randn(W, D, device=dev, generator=gen) * 0.5).float()
     cb = torch.zeros(D, device=dev)
     wi, wa = (torch.randn(nb, bw, bw, device=dev, generator=gen) / bw ** 0.5 for _ in range(2))
     bi, ba = (torch.randn(D, device=dev, generator=gen) * 0.1 for _ in range(2))
     lam = lambda_for_a8_range(torch.Generator().manual_seed(args.seed), D, 0.9, 0.999).to(dev)
-    e = lambda: torch.empty(B, T, D, device=dev, dtype=bf)  # noqa: E731
+    e = lambda: act_empty(args, (B, T, D), bf, dev)  # noqa: E731
     u, xg, ag, h, out = e(), e(), e(), e(), e()
     du, dxg, dag, dy, dxin = e(), e(), e(), e(), e()
-    dxy = torch.empty(B, T, 2 * D, device=dev, dtype=bf)   # gradient of xy, both halves written in place
+    dxy = act_empty(args, (B, T, 2 * D), bf, dev)   # gradient of xy, both halves written in place
     dlam = torch.empty(D, device=dev)
     dwi, dwa, dbi, dba = torch.empty_like(wi), torch.empty_like(wa), torch.empty_like(bi), torch.empty_like(ba)
     dcw, dcb = torch.empty_like(cw), torch.empty_like(cb)
@@ -410,7 +434,8 @@ def run_block(args, lib, dev):
         "vs_baseline": None, "dtype": "bf16 activations, f32 parameters, state and accumulation",
         "data": f"synthetic, seed {args.seed}",
         "config": {"workload": f"block: conv1d(4) + gate projections ({nb} blocks) + scan fused with gelu(y)*h, "
-                               f"fwd+bwd, B={B}, T={T}, D={D}, bf16", "B": B, "T": T, "D": D},
+                               f"fwd+bwd, B={B}, T={T}, D={D}, bf16", "B": B, "T": T, "D": D,
+                   "allocation": ALLOCATION[bool(args.plain_alloc)]},
         "roofline": {"bound": "hbm", "kernel": "all launches of the step", "achieved": step_gbs,
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": step_gbs / HBM_PEAK_GBS, "traffic": None,
                      "algorithmic_bytes_per_launch": fwd_bytes + bwd_bytes},
@@ -691,28 +716,28 @@ def run_scan(args, lib, dev, name, steps, warmup, settle, calibration_copy=False
     in_dt = torch.float32 if mixed else bf
     in_code = _lib.HAWK_DTYPE_F32 if mixed else code
     gen = torch.Generator(device=dev).manual_seed(args.seed)
-    x, xg, ag = (torch.randn(B, T, D, device=dev, generator=gen).to(in_dt) for _ in range(3))
-    gout = torch.randn(B, T, D, device=dev, generator=gen).to(bf)
+    x, xg, ag = (act_randn(args, (B, T, D), in_dt, dev, gen) for _ in range(3))
+    gout = act_randn(args, (B, T, D), bf, dev, gen)
     lam = lambda_for_a8_range(torch.Generator().manual_seed(args.seed), D, lo, hi).to(dev)
-    h = torch.empty_like(gout)
-    dx, dxg, dag = torch.empty_like(x), torch.empty_like(x), torch.empty_like(x)
+    h = act_empty(args, (B, T, D), bf, dev)
+    dx, dxg, dag = (act_empty(args, (B, T, D), in_dt, dev) for _ in range(3))
     dlam = torch.empty(D, dtype=torch.float32, device=dev)
     ws = torch.zeros(lib.hawk_scan_workspace_bytes(B, T, D, in_code), dtype=torch.uint8, device=dev)
     if with_conv:
         W = 4
         cw = (torch.randn(W, D, device=dev, generator=gen) * 0.5).float()
         cb = torch.zeros(D, device=dev)
-        u = torch.empty_like(x)       # conv output, the scan's x
-        du = torch.empty_like(x)      # conv input gradient
+        u = act_empty(args, (B, T, D), in_dt, dev)       # conv output, the scan's x
+        du = act_empty(args, (B, T, D), in_dt, dev)      # conv input gradient
         dw = torch.empty(W, D, device=dev)
         db = torch.empty(D, device=dev)
         cws = torch.empty(lib.hawk_conv1d_bwd_workspace_bytes(B, T, D, W), dtype=torch.uint8, device=dev)
     gated = name == "scan_gated"
     if gated:
-        xy = torch.randn(B, T, 2 * D, device=dev, generator=gen).to(bf)
+        xy = act_randn(args, (B, T, 2 * D), bf, dev, gen)
         y = xy[..., D:]               # the gate half of the block's input projection, in place
-        gated_out = torch.empty_like(x)
-        dy = torch.empty_like(x)
+        gated_out = act_empty(args, (B, T, D), bf, dev)
+        dy = act_empty(args, (B, T, D), bf, dev)
     stream = torch.cuda.current_stream(dev).cuda_stream
 
     def fwd():
@@ -847,6 +872,7 @@ def run_scan(args, lib, dev, name, steps, warmup, settle, calibration_copy=False
                         + f" fwd+bwd, B={B}, T={T}, D={D}, " + ("f32 in / bf16 state" if mixed else "bf16")
                         + f"; {settle} + {warmup} untimed steps before the {steps} timed ones",
             "B": B, "T": T, "D": D,
+            "allocation": ALLOCATION[bool(args.plain_alloc)],
         },
         "timed_region": {"steps": steps, "host_ms": wall * 1e3, "gpu_ms_between_events": region_gpu_ms,
                          "events_inside": 0},
@@ -947,6 +973,10 @@ def main():
                          "two launches on a copy of the x half of the input projection, gradients into separate "
                          "tensors, a closing reduction per backward call) instead of one host call per direction "
                          "on the projection's output in place")
+    ap.add_argument("--plain-alloc", action="store_true",
+                    help="kernel workloads: allocate every tensor with a plain torch.empty (large blocks then start "
+                         "on 2 MiB boundaries) instead of the library's placement of activation tensors, bases "
+                         "256 bytes apart modulo 1 KiB")
     ap.add_argument("--workload", choices=sorted(WORKLOADS) + ["block", "decode", "gates", "model"], default="scan")
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -1004,13 +1034,18 @@ def main():
         also = {}
         few = argparse.Namespace(**vars(args))
         few.steps, few.settle_steps, few.calibration_copy = max(20, args.steps // 4), max(10, args.settle_steps // 4), False
-        for other in ("long", "scan_conv", "scan_gated"):
+        plain = argparse.Namespace(**vars(args))
+        plain.plain_alloc = not args.plain_alloc
+        for other in ("scan", "long", "scan_conv", "scan_gated"):
             torch.cuda.empty_cache()
-            rec = run_scan(args, lib, dev, other, few.steps, args.warmup, few.settle_steps)
+            # the headline's shape once more with the other placement of its tensors
+            rec = run_scan(plain if other == "scan" else args, lib, dev, other, few.steps, args.warmup,
+                           few.settle_steps)
             rec.pop("_cpu_args")
             rec.pop("_buffers")
-            also[other] = {k: rec[k] for k in ("config", "value", "unit", "ms_per_step", "steps", "warmup",
-                                               "settle_steps", "roofline", "fwd", "step_hbm")}
+            key = ("scan_plain_alloc" if plain.plain_alloc else "scan_library_alloc") if other == "scan" else other
+            also[key] = {k: rec[k] for k in ("config", "value", "unit", "ms_per_step", "steps", "warmup",
+                                             "settle_steps", "roofline", "fwd", "step_hbm")}
         # the matrix-core gate projections and the recurrent core of one layer at the same shape, and
         # one-token decode steps of the 26-layer model at batch 256, and training steps of the README model
         for other, fn in (("gates", run_gates), ("block", run_block), ("decode", run_decode), ("model", run_model)):

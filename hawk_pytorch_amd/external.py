@@ -32,7 +32,7 @@ def _launch_conv_fwd(x, w, b, state, out_dtype) -> torch.Tensor:
         state = _lib.dense16(state)
     B, T, D = x.shape
     W = w.shape[0]
-    y = torch.empty((B, T, D), dtype=out_dtype, device=dev)
+    y = _lib.activation_empty((B, T, D), out_dtype, dev)
     lib = _lib.load()
     with torch.cuda.device(dev):
         status = lib.hawk_conv1d_fwd(
@@ -48,7 +48,7 @@ def _launch_conv_bwd(grad_y, x, w):
     grad_y, x, w = _lib.dense16(grad_y), _lib.dense16(x), _lib.dense16(w)
     B, T, D = x.shape
     W = w.shape[0]
-    dx = torch.empty_like(x)
+    dx = _lib.activation_empty(x.shape, x.dtype, dev)
     dw = torch.empty((W, D), dtype=torch.float32, device=dev)
     db = torch.empty((D,), dtype=torch.float32, device=dev)
     lib = _lib.load()
@@ -403,8 +403,8 @@ def _launch_gate_fwd(x, w_i, b_i, w_a, b_a, out_bf16: bool):
     M = x.numel() // D
     x2, w_i, w_a, b_i, b_a = (_lib.dense16(t) for t in (x.reshape(M, D), w_i, w_a, b_i, b_a))
     out_dtype = torch.bfloat16 if out_bf16 else torch.float32
-    xg = torch.empty(x.shape, dtype=out_dtype, device=dev)
-    ag = torch.empty(x.shape, dtype=out_dtype, device=dev)
+    xg = _lib.activation_empty(x.shape, out_dtype, dev)
+    ag = _lib.activation_empty(x.shape, out_dtype, dev)
     with torch.cuda.device(dev):
         status = _lib.load().hawk_gate_proj_fwd(
             x2.data_ptr(), w_i.data_ptr(), b_i.data_ptr(), w_a.data_ptr(), b_a.data_ptr(), xg.data_ptr(),
@@ -422,7 +422,7 @@ def _launch_gate_bwd(x, d_xg, d_ag, w_i, w_a, addend=None):
     M = x.numel() // D
     x2, g_i, g_a, w_i, w_a = (_lib.dense16(t) for t in (x.reshape(M, D), d_xg.reshape(M, D), d_ag.reshape(M, D), w_i, w_a))
     lib = _lib.load()
-    dx = torch.empty(x.shape, dtype=x.dtype, device=dev)
+    dx = _lib.activation_empty(x.shape, x.dtype, dev)
     if addend is not None:
         addend = _lib.dense16(addend.reshape(M, D).to(x.dtype))
     dw_i = torch.empty((nb, bw, bw), dtype=torch.float32, device=dev)

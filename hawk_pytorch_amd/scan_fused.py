@@ -51,7 +51,7 @@ def _launch_scan_fwd(x, x_rg_lru, a_rg_lru, a_param, h_bf16: bool) -> torch.Tens
     in_code = _lib.dtype_code(x.dtype)
     out_dtype = torch.bfloat16 if h_bf16 else x.dtype
     lib = _lib.load()
-    h = torch.empty((b, sq, d), dtype=out_dtype, device=dev)
+    h = _lib.activation_empty((b, sq, d), out_dtype, dev)
     nbytes = lib.hawk_scan_workspace_bytes(b, sq, d, in_code)
     ws = _lib.scan_workspace(dev, nbytes)
     with torch.cuda.device(dev):
@@ -71,9 +71,7 @@ def _launch_scan_bwd(x, x_rg_lru, a_rg_lru, a_param, h_saved, grad_out):
     b, sq, d = x.shape
     in_code = _lib.dtype_code(x.dtype)
     lib = _lib.load()
-    dx = torch.empty_like(x)
-    dxg = torch.empty_like(x)
-    dag = torch.empty_like(x)
+    dx, dxg, dag = (_lib.activation_empty(x.shape, x.dtype, dev) for _ in range(3))
     dlam = torch.empty(d, dtype=torch.float32, device=dev)
     nbytes = lib.hawk_scan_workspace_bytes(b, sq, d, in_code)
     ws = _lib.scan_workspace(dev, nbytes)
@@ -272,8 +270,8 @@ def _launch_scan_gated_fwd(x, x_rg_lru, a_rg_lru, a_param, y, h_bf16: bool, want
         y = _lib.dense16(y)
         ldy = d
     lib = _lib.load()
-    out = torch.empty((b, sq, d), dtype=out_dtype, device=dev)
-    h = torch.empty((b, sq, d) if want_h else (0,), dtype=out_dtype, device=dev)
+    out = _lib.activation_empty((b, sq, d), out_dtype, dev)
+    h = _lib.activation_empty((b, sq, d) if want_h else (0,), out_dtype, dev)
     h_last = torch.empty((b, 1, d) if want_last else (0,), dtype=out_dtype, device=dev)
     nbytes = lib.hawk_scan_workspace_bytes(b, sq, d, in_code)
     ws = _lib.scan_workspace(dev, nbytes)
@@ -301,10 +299,8 @@ def _launch_scan_gated_bwd(x, x_rg_lru, a_rg_lru, a_param, y, h_saved, grad_out)
         y = _lib.dense16(y)
         ldy = d
     lib = _lib.load()
-    dx = torch.empty_like(x)
-    dxg = torch.empty_like(x)
-    dag = torch.empty_like(x)
-    dy = torch.empty((b, sq, d), dtype=h_saved.dtype, device=dev)
+    dx, dxg, dag = (_lib.activation_empty(x.shape, x.dtype, dev) for _ in range(3))
+    dy = _lib.activation_empty((b, sq, d), h_saved.dtype, dev)
     dlam = torch.empty(d, dtype=torch.float32, device=dev)
     nbytes = lib.hawk_scan_workspace_bytes(b, sq, d, in_code)
     ws = _lib.scan_workspace(dev, nbytes)
@@ -503,8 +499,8 @@ def _launch_block_core_fwd(xy, conv_w, conv_b, w_i, b_i, w_a, b_a, lam, want_h: 
     nb = w_i.shape[0]
     conv_w, conv_b, w_i, w_a, b_i, b_a, lam = (_lib.dense16(t) for t in (conv_w, conv_b, w_i, w_a, b_i, b_a, lam))
     bf, code = torch.bfloat16, _lib.HAWK_DTYPE_BF16
-    u, xg, ag, out = (torch.empty((B, T, D), dtype=bf, device=dev) for _ in range(4))
-    h = torch.empty((B, T, D) if want_h else (0,), dtype=bf, device=dev)
+    u, xg, ag, out = (_lib.activation_empty((B, T, D), bf, dev) for _ in range(4))
+    h = _lib.activation_empty((B, T, D) if want_h else (0,), bf, dev)
     h_last = torch.empty((B, 1, D) if want_last else (0,), dtype=bf, device=dev)
     lib = _lib.load()
     ws = _lib.scan_workspace(dev, lib.hawk_scan_workspace_bytes(B, T, D, code))
@@ -547,8 +543,8 @@ def _launch_block_core_bwd(xy, u, xg, ag, h, conv_w, w_i, w_a, lam, grad_out):
     conv_w, w_i, w_a, lam, grad_out = (_lib.dense16(t) for t in (conv_w, w_i, w_a, lam, grad_out))
     bf, code, f32 = torch.bfloat16, _lib.HAWK_DTYPE_BF16, torch.float32
     lib = _lib.load()
-    d_xy = torch.empty((B, T, D2), dtype=bf, device=dev)
-    du, dxg, dag = (torch.empty((B, T, D), dtype=bf, device=dev) for _ in range(3))
+    d_xy = _lib.activation_empty((B, T, D2), bf, dev)
+    du, dxg, dag = (_lib.activation_empty((B, T, D), bf, dev) for _ in range(3))
     dlam = torch.empty(D, dtype=f32, device=dev)
     dw_i, dw_a = (torch.empty((nb, bw, bw), dtype=f32, device=dev) for _ in range(2))
     db_i, db_a, dcb = (torch.empty(D, dtype=f32, device=dev) for _ in range(3))

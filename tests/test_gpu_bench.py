@@ -36,12 +36,17 @@ def test_bench_prints_one_json_line_with_the_agreed_fields():
     # tokens/s is B*T over the step time
     assert abs(d["value"] - 8 * 4096 / (d["ms_per_step"] * 1e-3)) < 1e-6 * d["value"]
     # the other configurations of the benchmark definition ride along as sub-records
-    assert set(d["also"]) == {"long", "scan_conv", "scan_gated", "gates", "block", "decode", "model"}
+    assert set(d["also"]) == {"scan_plain_alloc", "long", "scan_conv", "scan_gated", "gates", "block", "decode",
+                              "model"}
+    # the headline's tensors are placed as the library places its own; the same shape with plain
+    # torch.empty rides along
+    assert "activation_empty" in d["config"]["allocation"]
+    assert d["also"]["scan_plain_alloc"]["config"]["allocation"].startswith("plain torch.empty")
     for name, rec in d["also"].items():
         assert rec["value"] > 0 and "workload" in rec["config"], name
         if name != "model":   # launch-bound end to end: no roofline is claimed for it
             assert 0.0 < rec["roofline"]["frac"] < 1.0, name
-    for name in ("long", "scan_conv", "scan_gated", "gates", "block"):
+    for name in ("scan_plain_alloc", "long", "scan_conv", "scan_gated", "gates", "block"):
         assert d["also"][name]["roofline"]["frac"] > 0.2, name
     # a traffic figure is reported only when it was measured on the present kernel sources
     assert roof["traffic"] is None or roof["traffic"] > roof["algorithmic_bytes_per_launch"]

@@ -330,3 +330,43 @@ def test_two_streams_scan_concurrently_with_their_own_workspaces():
             assert torch.equal(h, h_ref)
             for a, b in zip(grads, grads_ref):
                 assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "f32"])
+def test_results_do_not_depend_on_where_the_tensors_start(dtype):
+    """The same values in tensors whose bases are 0, 16, 48, 256 or 272 bytes apart modulo 1 KiB
+    (the host code places the activations it allocates 256 bytes apart, callers may pass any
+    16-byte aligned pointers): the same bits."""
+    B, T, D = 3, 700, 640
+    arrs = make_scan_inputs(B, T, D, seed=21)
+    x, xg, ag, lam, gout = arrs
+    lam_d = capi.to_dev(lam, "f32")
+    n = x.size
+    td = capi.TORCH_DTYPE[dtype]
+    esz = 2 if dtype == "bf16" else 4
+
+    def carve(step):
+        pad = step // esz
+        buf = torch.zeros(4 * (n + pad) + 2048, dtype=td, device="cuda")
+        first = ((-buf.data_ptr()) % 1024) // esz
+        out = []
+        for i, a in enumerate((x, xg, ag, gout)):
+            t = buf[first + i * (n + pad): first + i * (n + pad) + n].view(a.shape)
+            t.copy_(capi.to_dev(a, dtype))
+            out.append(t)
+        return out, buf
+
+    ref = None
+    for step in (0, 16, 48, 256, 272):
+        (xd, xgd, agd, god), keep = carve(step)
+        assert [(t.data_ptr() - xd.data_ptr()) % 1024 for t in (xgd, agd, god)] == [step % 1024, 2 * step % 1024,
+                                                                                    3 * step % 1024]
+        h = capi.scan_fwd(xd, xgd, agd, lam_d)
+        grads = capi.scan_bwd(xd, xgd, agd, lam_d, h, god)
+        torch.cuda.synchronize()
+        got = [h, *grads]
+        if ref is None:
+            ref = [t.clone() for t in got]
+        else:
+            for k, (a, b) in enumerate(zip(got, ref)):
+                assert torch.equal(a, b), (step, k)

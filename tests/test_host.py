@@ -378,3 +378,30 @@ def test_bench_refuses_more_than_one_gpu():
                        capture_output=True, text=True, timeout=300, cwd=root)
     assert r.returncode == 2
     assert "one GPU" in r.stderr and r.stdout.strip() == ""
+
+
+def test_activation_placement_steps_through_the_kilobyte(monkeypatch):
+    """_lib.activation_empty: large tensors start 256 bytes further on (modulo 1 KiB) from one call
+    to the next, are contiguous and 16-byte aligned; small ones and HAWK_STAGGER_BYTES=0 give a
+    plain torch.empty."""
+    from hawk_pytorch_amd import _lib
+
+    monkeypatch.delenv("HAWK_STAGGER_BYTES", raising=False)
+    shape = (4, 512, 512)
+    ts = [_lib.activation_empty(shape, torch.bfloat16, "cpu") for _ in range(6)]
+    pos = [t.data_ptr() % 1024 for t in ts]
+    assert all((b - a) % 1024 == 256 for a, b in zip(pos, pos[1:])), pos
+    for t in ts:
+        assert t.shape == shape and t.is_contiguous() and t.data_ptr() % 16 == 0 and t.dtype == torch.bfloat16
+        t.zero_()   # the whole view lies inside its buffer
+    f = _lib.activation_empty((1024, 1024), torch.float32, "cpu")
+    assert (f.data_ptr() - ts[-1].data_ptr()) % 1024 == 256 and f.is_contiguous()
+    small = _lib.activation_empty((8, 64), torch.bfloat16, "cpu")
+    assert small.storage_offset() == 0 and small.numel() == 512
+    empty = _lib.activation_empty((0,), torch.bfloat16, "cpu")
+    assert empty.numel() == 0
+    monkeypatch.setenv("HAWK_STAGGER_BYTES", "0")
+    assert _lib.activation_empty(shape, torch.bfloat16, "cpu").storage_offset() == 0
+    monkeypatch.setenv("HAWK_STAGGER_BYTES", "100")
+    with pytest.raises(ValueError):
+        _lib.activation_empty(shape, torch.bfloat16, "cpu")
