@@ -82,9 +82,9 @@ HBM_PEAK_GBS = 8000.0
 # with the digest of the kernel sources they were measured on.  A record taken on other
 # sources is stale and is not reported.
 TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic.json")
-KERNEL_SOURCES = {"gates": ("hawk_gates.hip", "hawk_device.h"),
-                  "scan_conv": ("hawk_scan.hip", "hawk_conv.hip", "hawk_device.h")}
-SCAN_KERNEL_SOURCES = ("hawk_scan.hip", "hawk_device.h")
+KERNEL_SOURCES = {"gates": ("hawk_gates.hip", "hawk_device.h", "hawk_reduce.h"),
+                  "scan_conv": ("hawk_scan.hip", "hawk_conv.hip", "hawk_device.h", "hawk_reduce.h")}
+SCAN_KERNEL_SOURCES = ("hawk_scan.hip", "hawk_device.h", "hawk_reduce.h")
 
 
 def kernel_source_digest(workload):
