@@ -7,6 +7,8 @@ cannot be found or built, or a call reports a non-zero status, an exception is r
 from __future__ import annotations
 
 import ctypes
+import itertools
+import math
 import os
 import threading
 
@@ -191,12 +193,12 @@ def dense16(t: torch.Tensor) -> torch.Tensor:
 # workgroup that streams one column tile of several tensors then keeps a quarter of the channels
 # busy.  Bases 256 bytes further on from one tensor to the next (modulo 1 KiB) put the columns of
 # four tensors side by side over all of them: 1-2 % on the scan kernels and on a whole block
-# step at D = 2560.  The cost is 1 KiB per tensor.
+# step at D = 2560.  The cost is 1 KiB per tensor; tensors under 16 MiB are left alone.
 # HAWK_STAGGER_BYTES=0 switches it off (plain torch.empty).
 # ---------------------------------------------------------------------------------------
 _STAGGER_PERIOD = 1024
-_STAGGER_MIN_BYTES = 1 << 20
-_stagger_count = 0
+_STAGGER_MIN_BYTES = 16 << 20   # smaller tensors stream from the caches, and a host-bound step feels every call
+_stagger_count = itertools.count()
 
 
 def _stagger_bytes() -> int:
@@ -208,21 +210,20 @@ def _stagger_bytes() -> int:
 
 def activation_empty(shape, dtype: torch.dtype, device) -> torch.Tensor:
     """torch.empty(shape) whose base address follows the previous call's by HAWK_STAGGER_BYTES
-    modulo 1 KiB.  Contiguous; a view of a private buffer 1 KiB larger than the tensor."""
-    global _stagger_count
-    n = 1
-    for d in shape:
-        n *= int(d)
-    esz = torch.empty((), dtype=dtype).element_size()
+    modulo 1 KiB (tensors of 16 MiB and more; smaller ones are a plain torch.empty).
+    Contiguous; a view of a private buffer 1 KiB larger than the tensor."""
+    shape = tuple(shape)
+    n = math.prod(shape)
+    esz = dtype.itemsize
+    if n * esz < _STAGGER_MIN_BYTES:
+        return torch.empty(shape, dtype=dtype, device=device)
     step = _stagger_bytes()
-    if step == 0 or n * esz < _STAGGER_MIN_BYTES:
-        return torch.empty(tuple(shape), dtype=dtype, device=device)
+    if step == 0:
+        return torch.empty(shape, dtype=dtype, device=device)
     buf = torch.empty(n + _STAGGER_PERIOD // esz, dtype=dtype, device=device)
-    with _lock:
-        want = (_stagger_count * step) % _STAGGER_PERIOD
-        _stagger_count += 1
+    want = (next(_stagger_count) * step) % _STAGGER_PERIOD
     off = ((want - buf.data_ptr()) % _STAGGER_PERIOD) // esz
-    return buf[off:off + n].view(tuple(shape))
+    return buf[off:off + n].view(shape)
 
 
 # ---------------------------------------------------------------------------------------

@@ -387,14 +387,14 @@ def test_activation_placement_steps_through_the_kilobyte(monkeypatch):
     from hawk_pytorch_amd import _lib
 
     monkeypatch.delenv("HAWK_STAGGER_BYTES", raising=False)
-    shape = (4, 512, 512)
+    shape = (4, 2048, 1024)
     ts = [_lib.activation_empty(shape, torch.bfloat16, "cpu") for _ in range(6)]
     pos = [t.data_ptr() % 1024 for t in ts]
     assert all((b - a) % 1024 == 256 for a, b in zip(pos, pos[1:])), pos
     for t in ts:
         assert t.shape == shape and t.is_contiguous() and t.data_ptr() % 16 == 0 and t.dtype == torch.bfloat16
         t.zero_()   # the whole view lies inside its buffer
-    f = _lib.activation_empty((1024, 1024), torch.float32, "cpu")
+    f = _lib.activation_empty((2048, 2048), torch.float32, "cpu")
     assert (f.data_ptr() - ts[-1].data_ptr()) % 1024 == 256 and f.is_contiguous()
     small = _lib.activation_empty((8, 64), torch.bfloat16, "cpu")
     assert small.storage_offset() == 0 and small.numel() == 512
@@ -405,3 +405,4 @@ def test_activation_placement_steps_through_the_kilobyte(monkeypatch):
     monkeypatch.setenv("HAWK_STAGGER_BYTES", "100")
     with pytest.raises(ValueError):
         _lib.activation_empty(shape, torch.bfloat16, "cpu")
+    assert _lib.activation_empty((8, 64), torch.bfloat16, "cpu").numel() == 512   # small: the setting is not read
