@@ -337,6 +337,46 @@ def test_argument_validation_of_the_conv_front_and_the_strided_conv():
         == E.HAWK_ERR_WORKSPACE
 
 
+def test_argument_validation_of_the_block_core_entry_points():
+    lib = _lib.load()
+    E = _lib
+    p = 4096  # never dereferenced: every call below is refused before a launch
+    # xy, stride, conv_w, conv_b, w_i, b_i, w_a, b_a, w_dtype, w_bf16, a_param, u, xg, ag, h, out, h_last,
+    # B, T, D, nb, W, scan_ws, bytes, stream
+    ok = [p, 512, p, p, p, None, p, None, 1, p, p, p, p, p, None, p, None, 2, 64, 256, 1, 4, p, 1 << 20, None]
+    for idx, what in ((18, 31), (21, 3), (1, 511), (1, 516), (20, 3), (19, 252)):   # T, width, stride, stride % 8, blocks, D % 8
+        bad = list(ok); bad[idx] = what
+        assert lib.hawk_block_core_fwd(*bad) == E.HAWK_ERR_BAD_SHAPE, (idx, what)
+    for idx in (0, 2, 3, 4, 6, 10, 11, 12, 13, 15):
+        bad = list(ok); bad[idx] = None
+        assert lib.hawk_block_core_fwd(*bad) == E.HAWK_ERR_NULL_POINTER, idx
+    bad = list(ok); bad[8] = 7
+    assert lib.hawk_block_core_fwd(*bad) == E.HAWK_ERR_BAD_DTYPE
+    bad = list(ok); bad[15] = p + 8
+    assert lib.hawk_block_core_fwd(*bad) == E.HAWK_ERR_ALIGNMENT
+    # xy, stride, u, xg, ag, h, conv_w, w_i, w_a, w_dtype, a_param, grad_out, d_xy, stride, du, dxg, dag, dcw, dcb,
+    # dw_i, db_i, dw_a, db_a, da_param, B, T, D, nb, W, 3 x (workspace, bytes), stream
+    ok = [p, 512, p, p, p, p, p, p, p, 0, p, p, p, 512, p, p, p, p, p, p, None, p, None, p, 2, 64, 256, 1, 4,
+          p, 1 << 20, p, 1 << 20, p, 1 << 20, None]
+    for idx, what in ((28, 9), (28, 0), (1, 511), (13, 511), (13, 516), (27, 3), (26, 252), (24, 70000)):
+        bad = list(ok); bad[idx] = what
+        assert lib.hawk_block_core_bwd(*bad) == E.HAWK_ERR_BAD_SHAPE, (idx, what)
+    for idx in (0, 2, 3, 4, 5, 6, 7, 8, 10, 11, 12, 14, 15, 16, 17, 18, 19, 21, 23):
+        bad = list(ok); bad[idx] = None
+        assert lib.hawk_block_core_bwd(*bad) == E.HAWK_ERR_NULL_POINTER, idx
+    for idx in (29, 31, 33):
+        bad = list(ok); bad[idx] = None
+        assert lib.hawk_block_core_bwd(*bad) == E.HAWK_ERR_WORKSPACE, idx
+    bad = list(ok); bad[9] = 7
+    assert lib.hawk_block_core_bwd(*bad) == E.HAWK_ERR_BAD_DTYPE
+    bad = list(ok); bad[12] = p + 4
+    assert lib.hawk_block_core_bwd(*bad) == E.HAWK_ERR_ALIGNMENT
+    # both gates' weights in one launch
+    assert lib.hawk_gate_weights_to_bf16(p, p, p, None, 2, 64, None) == E.HAWK_ERR_NULL_POINTER
+    assert lib.hawk_gate_weights_to_bf16(p, p, p, p, 2, 6, None) == E.HAWK_ERR_BAD_SHAPE
+    assert lib.hawk_gate_weights_to_bf16(p, p, p + 2, p, 2, 64, None) == E.HAWK_ERR_ALIGNMENT
+
+
 def test_argument_validation_of_the_fused_decode_step():
     lib = _lib.load()
     buf = (ctypes.c_char * 4096)()
