@@ -924,9 +924,32 @@ def run_stream_ceiling(buf, steps, settle):
         torch.mul(h, gout, out=dxg)        # 2 reads, 1 write
         dag.fill_(0.5)                     # 1 write
 
+    # The library's own streaming probes: copies with the scan kernels' memory instructions, flat
+    # (16 KiB of every tensor per workgroup) and in the scan's workgroup shape (eight waves stacked
+    # in time on 16 rows x 256 bytes each), for the forward's and the backward's mix.
+    from hawk_pytorch_amd import _lib
+
+    lib = _lib.load()
+    stream = torch.cuda.current_stream(x.device).cuda_stream
+    row_pitch = x.shape[-1] * x.element_size()
+
+    def probe(reads, writes, shape):
+        r = (ctypes.c_void_p * len(reads))(*[t.data_ptr() for t in reads])
+        w = (ctypes.c_void_p * len(writes))(*[t.data_ptr() for t in writes])
+
+        def call():
+            _lib.check("stream_probe", lib.hawk_stream_probe(r, len(reads), w, len(writes), nbytes, row_pitch, shape,
+                                                             stream))
+        return call
+
+    fwd_mix, bwd_mix = ((x, xg, ag), (h,)), ((x, xg, ag, h, gout), (dx, dxg, dag))
     rec = {}
     for name, fn, tensors, kernels in (("copy_1r1w", copy_1r1w, 2, 1), ("addcmul_3r1w", addcmul_3r1w, 4, 1),
-                                       ("composition_5r3w", composition_5r3w, 8, 3)):
+                                       ("composition_5r3w", composition_5r3w, 8, 3),
+                                       ("probe_flat_3r1w", probe(*fwd_mix, 0), 4, 1),
+                                       ("probe_flat_5r3w", probe(*bwd_mix, 0), 8, 1),
+                                       ("probe_scan_shape_3r1w", probe(*fwd_mix, 1), 4, 1),
+                                       ("probe_scan_shape_5r3w", probe(*bwd_mix, 1), 8, 1)):
         for _ in range(settle):
             fn()
         torch.cuda.synchronize()
@@ -952,8 +975,11 @@ def run_stream_ceiling(buf, steps, settle):
                      "us_with_an_event_per_call": with_events_ms * 1e3,
                      "frac_with_an_event_per_call": moved / (with_events_ms * 1e-3) / 1e9 / HBM_PEAK_GBS}
     rec["note"] = ("torch.Tensor.copy_, torch.addcmul(out=) and addcmul + mul + fill_ on the headline's x, x_rg_lru, "
-                   "a_rg_lru, h, grad_out and gradient tensors (bf16, %d MB each), %d settling calls, then %d timed "
-                   "calls; frac is of the 8 TB/s peak" % (nbytes // 1000000, settle, steps))
+                   "a_rg_lru, h, grad_out and gradient tensors (bf16, %d MB each), and the library's copy kernels "
+                   "(hawk_stream_probe: non-temporal buffer loads and stores; flat = 16 KiB of every tensor per "
+                   "workgroup, scan_shape = eight waves stacked in time on 16 rows x 256 bytes each, as a scan "
+                   "workgroup reads its tile) on the same tensors; %d settling calls, then %d timed calls; frac is "
+                   "of the 8 TB/s peak" % (nbytes // 1000000, settle, steps))
     return rec
 
 
@@ -1026,6 +1052,16 @@ def main():
                                                         / (ceiling["composition_5r3w"]["us_with_an_event_per_call"] * 1e-6) / 1e9))
         ceiling["scan_step_over_both"] = ((ceiling["addcmul_3r1w"]["us"] + ceiling["composition_5r3w"]["us"]) * 1e-3
                                           / out["ms_per_step"])
+        # the same three ratios against the library's copy kernels in the scan's own workgroup shape
+        ceiling["scan_fwd_over_probe_scan_shape_3r1w"] = (
+            ceiling["probe_scan_shape_3r1w"]["us_with_an_event_per_call"] * 1e-3 / out["fwd"]["ms"])
+        ceiling["scan_bwd_over_probe_scan_shape_5r3w"] = (
+            ceiling["probe_scan_shape_5r3w"]["us_with_an_event_per_call"] * 1e-3 / out["roofline"]["launch_ms"])
+        ceiling["scan_step_over_probe_scan_shape"] = (
+            (ceiling["probe_scan_shape_3r1w"]["us"] + ceiling["probe_scan_shape_5r3w"]["us"]) * 1e-3
+            / out["ms_per_step"])
+        ceiling["scan_step_over_probe_flat"] = (
+            (ceiling["probe_flat_3r1w"]["us"] + ceiling["probe_flat_5r3w"]["us"]) * 1e-3 / out["ms_per_step"])
         out["stream_ceiling"] = ceiling
     del buffers
     if args.workload == "scan" and not args.no_also:

@@ -93,6 +93,7 @@ SIGNATURES = {
     "hawk_rglru_step_gated": (
         _c_int, [_c_void_p] * 7 + [ctypes.c_longlong] + [_c_void_p] * 3 + [_c_int] * 4 + [_c_void_p]
     ),
+    "hawk_stream_probe": (_c_int, [_c_void_p, _c_int, _c_void_p, _c_int, _c_size_t, _c_size_t, _c_int, _c_void_p]),
     "hawk_gate_weights_to_bf16": (_c_int, [_c_void_p] * 4 + [_c_int] * 2 + [_c_void_p]),
     "hawk_block_core_fwd": (
         _c_int, [_c_void_p, ctypes.c_longlong] + [_c_void_p] * 6 + [_c_int] + [_c_void_p] * 8 + [_c_int] * 5

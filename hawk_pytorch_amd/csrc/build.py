@@ -14,7 +14,7 @@ from concurrent.futures import ThreadPoolExecutor
 CSRC = os.path.dirname(os.path.abspath(__file__))
 LIB_NAME = "libhawk_hip.so"
 LIB_PATH = os.path.join(CSRC, LIB_NAME)
-SOURCES = ["hawk_scan.hip", "hawk_conv.hip", "hawk_step.hip", "hawk_gates.hip", "hawk_block.hip", "hawk_capi.hip"]
+SOURCES = ["hawk_scan.hip", "hawk_conv.hip", "hawk_step.hip", "hawk_gates.hip", "hawk_block.hip", "hawk_probe.hip", "hawk_capi.hip"]
 HEADERS = ["hawk_scan.h", "hawk_device.h", "hawk_reduce.h", os.path.join("..", "..", "include", "hawk_hip.h")]
 
 # Packed-FP32 VALU instructions are switched off for all device code.

@@ -431,4 +431,20 @@ int hawk_block_core_bwd(const void* xy, long long xy_row_stride, const void* u, 
                                 conv_workspace_bytes, as_stream(stream));
 }
 
+int hawk_stream_probe(const void* const* reads, int n_reads, void* const* writes, int n_writes, size_t bytes,
+                      size_t row_pitch_bytes, int shape, void* stream) {
+    if (!reads || !writes) return HAWK_ERR_NULL_POINTER;
+    if (n_reads < 1 || n_reads > 5 || n_writes < 1 || n_writes > 3) return HAWK_ERR_BAD_SHAPE;
+    for (int i = 0; i < n_reads; ++i) {
+        if (!reads[i]) return HAWK_ERR_NULL_POINTER;
+        if (!aligned16(reads[i])) return HAWK_ERR_ALIGNMENT;
+    }
+    for (int i = 0; i < n_writes; ++i) {
+        if (!writes[i]) return HAWK_ERR_NULL_POINTER;
+        if (!aligned16(writes[i])) return HAWK_ERR_ALIGNMENT;
+    }
+    if (!hawk::stream_probe_shape_ok(bytes, row_pitch_bytes, shape)) return HAWK_ERR_BAD_SHAPE;
+    return hawk::stream_probe(reads, n_reads, writes, n_writes, bytes, row_pitch_bytes, shape, as_stream(stream));
+}
+
 }  // extern "C"

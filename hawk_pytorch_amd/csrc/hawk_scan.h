@@ -101,4 +101,9 @@ int block_core_bwd(const void* xy, long long ld, const void* u, const void* xg, 
                    int D, int nb, int W, void* scan_ws, size_t scan_ws_bytes, void* gate_ws, size_t gate_ws_bytes,
                    void* conv_ws, size_t conv_ws_bytes, hipStream_t st);
 
+// hawk_probe.hip
+bool stream_probe_shape_ok(size_t bytes, size_t row_pitch, int shape);
+int stream_probe(const void* const* reads, int n_reads, void* const* writes, int n_writes, size_t bytes,
+                 size_t row_pitch, int shape, hipStream_t st);
+
 }  // namespace hawk
