@@ -26,7 +26,7 @@ __global__ __launch_bounds__(256) void round_pair_kernel(const float* __restrict
 // Blocks [0, n0) run the dLambda reduction, [n0, n0 + n1) the conv's, the rest the projections'.
 __global__ __launch_bounds__(kColsumThreads) void block_finish_kernel(ColsumTask dlam, ColsumTask conv,
                                                                       GateReduceTask gates, int n0, int n1) {
-    __shared__ float s[16][kWave];
+    __shared__ float s[kColsumSlices][kColsumCols];
     const int blk = (int)blockIdx.x;
     if (blk < n0) {
         colsum_block(dlam, blk, s);

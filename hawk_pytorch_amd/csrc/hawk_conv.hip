@@ -314,7 +314,7 @@ __global__ __launch_bounds__(256) void conv1d_bwd_anyw_kernel(
 
 // Column sums of the [rows, (W + 1) D] partials in a fixed order: dw, then db.
 __global__ __launch_bounds__(kColsumThreads) void colsum_kernel(ColsumTask t) {
-    __shared__ float s[16][kWave];
+    __shared__ float s[kColsumSlices][kColsumCols];
     colsum_block(t, (int)blockIdx.x, s);
 }
 

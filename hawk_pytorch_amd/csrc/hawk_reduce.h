@@ -8,6 +8,9 @@
 
 namespace hawk {
 
+constexpr int kColsumThreads = 1024;   // kColsumCols columns x kColsumSlices row slices per block
+constexpr int kColsumCols = 32, kColsumSlices = kColsumThreads / kColsumCols;
+
 // Column sums of a [rows, cols] fp32 matrix in a fixed order.  Columns below n_first go to
 // out_first, the rest to out_second.  With `lam` the sums are the partials of dLambda:
 // out_first[c] = -8 sigmoid(lam[c]) * sum.
@@ -17,34 +20,36 @@ struct ColsumTask {
     float* out_second;
     const float* lam;
     int rows, cols, n_first;
-    int blocks() const { return (cols + kWave - 1) / kWave; }
+    int blocks() const { return (cols + kColsumCols - 1) / kColsumCols; }
 };
-constexpr int kColsumThreads = 1024;   // 64 columns x 16 row slices per block
 
-// Block `block` of the task, by a workgroup of kColsumThreads threads; `s` is its LDS scratch.
-__device__ __forceinline__ void colsum_block(const ColsumTask& t, int block, float (*s)[kWave]) {
-    const int lane = threadIdx.x & (kWave - 1);
-    const int slice = threadIdx.x / kWave;
-    const int c = block * kWave + lane;
+// Block `block` of the task, by a workgroup of kColsumThreads threads: kColsumCols adjacent columns
+// (one 128-byte line of a row) x kColsumSlices row slices; `s` is its LDS scratch.  The few rows a
+// thread takes are all asked for at once: the launch is a handful of memory round trips long, so
+// their number, not the bytes, sets its duration.
+__device__ __forceinline__ void colsum_block(const ColsumTask& t, int block, float (*s)[kColsumCols]) {
+    const int lane = threadIdx.x & (kColsumCols - 1);
+    const int slice = threadIdx.x / kColsumCols;
+    const int c = block * kColsumCols + lane;
     float sum = 0.0f;
     if (c < t.cols) {
         // eight independent loads in flight per thread; the order of additions is fixed
         int r = slice;
-        for (; r + 16 * 7 < t.rows; r += 16 * 8) {
+        for (; r + kColsumSlices * 7 < t.rows; r += kColsumSlices * 8) {
             float v[8];
 #pragma unroll
-            for (int k = 0; k < 8; ++k) v[k] = t.part[(size_t)(r + 16 * k) * t.cols + c];
+            for (int k = 0; k < 8; ++k) v[k] = t.part[(size_t)(r + kColsumSlices * k) * t.cols + c];
 #pragma unroll
             for (int k = 0; k < 8; ++k) sum += v[k];
         }
-        for (; r < t.rows; r += 16) sum += t.part[(size_t)r * t.cols + c];
+        for (; r < t.rows; r += kColsumSlices) sum += t.part[(size_t)r * t.cols + c];
     }
     s[slice][lane] = sum;
     __syncthreads();
     if (slice == 0 && c < t.cols) {
         float tot = 0.0f;
 #pragma unroll
-        for (int k = 0; k < 16; ++k) tot += s[k][lane];
+        for (int k = 0; k < kColsumSlices; ++k) tot += s[k][lane];
         if (t.lam != nullptr) tot *= -8.0f * sigmoid_precise(t.lam[c]);
         if (c < t.n_first) t.out_first[c] = tot;
         else t.out_second[c - t.n_first] = tot;

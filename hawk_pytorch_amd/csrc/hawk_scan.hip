@@ -725,10 +725,10 @@ __global__ __launch_bounds__(NW * kWave, HAWK_BWD_WAVES_PER_SIMD) void rglru_sca
 }
 
 // dLambda[c] = -8 sigmoid(Lambda_c) * sum over rows of the [rows, D] partials.
-// 64 channels x 16 row slices per block; fixed summation order, so the result is
+// 32 channels x 32 row slices per block; fixed summation order, so the result is
 // reproducible run to run.
 __global__ __launch_bounds__(kColsumThreads) void dlam_reduce_kernel(ColsumTask t) {
-    __shared__ float s[16][kWave];
+    __shared__ float s[kColsumSlices][kColsumCols];
     colsum_block(t, (int)blockIdx.x, s);
 }
 
