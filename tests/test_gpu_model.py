@@ -753,6 +753,43 @@ def test_block_core_matches_its_parts_bit_for_bit(B, T, D, nb, W):
         assert torch.equal(a, b), (name, max_rel(capi.to_np(a), capi.to_np(b)))
 
 
+def test_large_activations_are_placed_apart_and_the_ops_give_the_same_bits(monkeypatch):
+    """From 16 MiB up the host code starts the activation tensors it allocates 256 bytes apart
+    modulo 1 KiB (views of private buffers coming out of custom ops and autograd nodes); the block
+    core, the gated scan and the plain scan give the same bits with that placement switched off."""
+    B, T, D, nb = 2, 2048, 2048, 8           # one [B,T,D] bf16 tensor is 16 MiB
+    torch.manual_seed(14)
+    gi = hk.BlockDiagonalLinear(D, nb).cuda()
+    ga = hk.BlockDiagonalLinear(D, nb).cuda()
+    conv = hk.Conv1D(width=D, temporal_width=4).cuda()
+    lam = torch.nn.Parameter(torch.tensor(make_scan_inputs(1, 1, D, seed=1)[3], device="cuda", dtype=torch.float32))
+    xy = torch.randn(B, T, 2 * D, device="cuda").to(torch.bfloat16).requires_grad_(True)
+    go = torch.randn(B, T, D, device="cuda").to(torch.bfloat16)
+    params = (xy, lam, gi.w, gi.b, ga.w, ga.b, conv.w, conv.b)
+
+    def run():
+        for p in params:
+            p.grad = None
+        with torch.autocast(device_type="cuda", dtype=torch.bfloat16):
+            out = hk.recurrent_block_core(xy, conv, gi, ga, lam)
+        out.backward(go)
+        x, y = xy.detach().chunk(2, dim=-1)
+        h = hk.fused_linear_scan(x.contiguous(), y.contiguous(), y.contiguous(), lam.detach())
+        return out.detach(), h, [p.grad.detach().clone() for p in params]
+
+    monkeypatch.delenv("HAWK_STAGGER_BYTES", raising=False)
+    out, h, grads = run()
+    assert out.is_contiguous() and h.is_contiguous() and grads[0].is_contiguous()
+    assert out.storage_offset() + h.storage_offset() > 0          # views into their own, larger buffers
+    assert (h.data_ptr() - out.data_ptr()) % 256 == 0 and out.data_ptr() % 16 == 0
+    monkeypatch.setenv("HAWK_STAGGER_BYTES", "0")
+    out0, h0, grads0 = run()
+    assert out0.storage_offset() == 0 and h0.storage_offset() == 0
+    assert torch.equal(out, out0) and torch.equal(h, h0)
+    for a, b in zip(grads, grads0):
+        assert torch.equal(a, b)
+
+
 def test_model_uses_the_block_core_and_agrees_with_the_separate_nodes():
     cfg = dict(vocab_size=512, hidden_size=256, intermediate_size=512, num_hidden_layers=2, recurrent_size=256,
                num_blocks=4)
