@@ -126,3 +126,38 @@ def test_refuses_what_it_does_not_serve():
     args = list(_inputs(1, 64, 256, 1, "bf16", seed=1, W=3))
     with pytest.raises(Exception, match="status 2"):
         capi.block_core_fwd(*args[:8])                       # conv width 3
+
+
+def test_backward_without_bias_gradients_and_with_misaligned_weight_gradients():
+    """db_i / db_a may be NULL; weight-gradient tensors that do not start on 16 bytes take the
+    element-by-element reduction and get the same bits."""
+    args = _inputs(2, 96, 512, 2, "bf16", seed=8)
+    xy, cw, cb, wi, bi, wa, ba, lam, gout = args
+    out, u, xg, ag, h, _, _ = capi.block_core_fwd(xy, cw, cb, wi, bi, wa, ba, lam)
+    ref = capi.block_core_bwd(xy, u, xg, ag, h, cw, wi, wa, lam, gout)
+    nob = capi.block_core_bwd(xy, u, xg, ag, h, cw, wi, wa, lam, gout, with_bias=False)
+    torch.cuda.synchronize()
+    assert nob[4] is None and nob[6] is None
+    for k in (0, 1, 2, 3, 5, 7):
+        assert torch.equal(ref[k], nob[k]), k
+    # the single entry point with dw tensors 4 bytes off a 16-byte boundary
+    from hawk_pytorch_amd import _lib
+    lib = _lib.load()
+    B, T, D2 = xy.shape
+    D, nb, bw, M = D2 // 2, 2, 256, B * T
+    du, dxg, dag, _, _ = capi.scan_gated_bwd(u, xg, ag, lam, xy[..., D:], h, gout)
+    buf = torch.zeros(2 * nb * bw * bw + 2 * D + 16, dtype=torch.float32, device="cuda")
+    dwi = buf[1:1 + nb * bw * bw]
+    dwa = buf[1 + nb * bw * bw:1 + 2 * nb * bw * bw]
+    dbi = buf[1 + 2 * nb * bw * bw:1 + 2 * nb * bw * bw + D]
+    dba = buf[1 + 2 * nb * bw * bw + D:1 + 2 * nb * bw * bw + 2 * D]
+    assert dwi.data_ptr() % 16 == 4
+    n = lib.hawk_gate_proj_bwd_weights_workspace_bytes(M, D, nb)
+    ws = torch.empty(n, dtype=torch.uint8, device="cuda")
+    code = _lib.HAWK_DTYPE_BF16
+    _lib.check("bwd_weights", lib.hawk_gate_proj_bwd_weights(
+        u.data_ptr(), dxg.data_ptr(), dag.data_ptr(), dwi.data_ptr(), dbi.data_ptr(), dwa.data_ptr(), dba.data_ptr(),
+        M, D, nb, code, code, ws.data_ptr(), n, torch.cuda.current_stream().cuda_stream))
+    torch.cuda.synchronize()
+    assert torch.equal(dwi.view(nb, bw, bw), ref[3]) and torch.equal(dwa.view(nb, bw, bw), ref[5])
+    assert torch.equal(dbi, ref[4]) and torch.equal(dba, ref[6])
