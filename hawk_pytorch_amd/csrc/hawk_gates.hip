@@ -194,7 +194,7 @@ constexpr int kConvTaps = 4;
 constexpr int kRTileBytes = (kTileRows + kConvTaps - 1) * kARowBytes;   // a raw tile and its history rows
 template <typename OT>
 constexpr size_t gate_fwd_lds_bytes(bool conv) {
-    return 2 * kATileBytes + (size_t)kTileRows * (2 * kGroup * sizeof(OT) + 16) +
+    return 2 * kATileBytes + (sizeof(OT) > 2 ? 1 : 2) * (size_t)kTileRows * (2 * kGroup * sizeof(OT) + 16) +
            (conv ? 2 * (size_t)kRTileBytes + (kConvTaps + 1) * kGroup * sizeof(float) : 0);
 }
 
@@ -210,8 +210,10 @@ __global__ __launch_bounds__(kGateThreads, 1) void gate_proj_fwd_kernel(
     constexpr int kORowBytes = 2 * kGroup * (int)sizeof(OT) + 16;   // both gates' columns of one row + pad
     extern __shared__ __align__(16) unsigned char smem[];
     unsigned char* sA = smem;                     // two activation tiles
-    unsigned char* sO = smem + 2 * kATileBytes;   // one result tile
-    unsigned char* sR = sO + kTileRows * kORowBytes;                      // CONV: two raw tiles
+    constexpr bool kTwoResultTiles = sizeof(OT) == 2;                     // fp32 results: no room for two
+    constexpr int kOBuf = kTwoResultTiles ? kTileRows * kORowBytes : 0;   // distance between the two result tiles
+    unsigned char* sO = smem + 2 * kATileBytes;                           // result tiles
+    unsigned char* sR = sO + (kTwoResultTiles ? 2 : 1) * kTileRows * kORowBytes;   // CONV: two raw tiles
     float* sCW = reinterpret_cast<float*>(sR + 2 * kRTileBytes);          // CONV: taps and bias of the group
 
     const int tid = threadIdx.x;
@@ -406,10 +408,12 @@ __global__ __launch_bounds__(kGateThreads, 1) void gate_proj_fwd_kernel(
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
             const int m = 8 * (r / 4) + (r % 4);
-            store_out(o_base + m * kORowBytes, acc[r] + bias, static_cast<OT*>(nullptr));
+            store_out(o_base + cur * kOBuf + m * kORowBytes, acc[r] + bias, static_cast<OT*>(nullptr));
         }
         if constexpr (CONV) {
-            // raw tile it+2 into the raw buffer tile it has left, tile it+4 into its registers
+            // the conv of tile it+1 (raw since the last step) into the other A buffer, then raw tile
+            // it+2 into the raw buffer tile it has left and tile it+4 into its registers
+            if constexpr (kTwoResultTiles) conv_tile(it + 1, cur ^ 1);
             stage_raw_tile(cur, rnext, hnext);
             load_raw_tile(it + 4, rnext, hnext);
         } else {
@@ -429,7 +433,7 @@ __global__ __launch_bounds__(kGateThreads, 1) void gate_proj_fwd_kernel(
             const int row = (worker + it * nworkers) * kTileRows + prow;
             const int ocol = group * kGroup + pc * (16 / (int)sizeof(OT));
             if (ocol < D && row < M) {
-                const unsigned char* src = sO + prow * kORowBytes + pc * 16;
+                const unsigned char* src = sO + cur * kOBuf + prow * kORowBytes + pc * 16;
                 const u32x4 vi = *reinterpret_cast<const u32x4*>(src);
                 const u32x4 va = *reinterpret_cast<const u32x4*>(src + kGroup * (int)sizeof(OT));
                 __builtin_nontemporal_store(vi, reinterpret_cast<u32x4*>(out_i + (size_t)row * D + ocol));
@@ -438,8 +442,13 @@ __global__ __launch_bounds__(kGateThreads, 1) void gate_proj_fwd_kernel(
         }
         // (issued behind the matrix products instead, the conv spills and the kernel takes 194 us
         // against 150 us at 32768 rows of 2560 channels)
-        if constexpr (CONV) conv_tile(it + 1, cur ^ 1);
-        __syncthreads();
+        // Without the conv the next tile's results go to the other result tile, and the barrier in
+        // the middle of the next step orders everything else: a wave that is done with its stores
+        // goes straight on to the next tile's products.
+        if constexpr (!kTwoResultTiles) {
+            if constexpr (CONV) conv_tile(it + 1, cur ^ 1);
+            __syncthreads();
+        }
     };
 
     for (int it = 0; worker + it * nworkers < ntiles; it += 2) {
