@@ -51,6 +51,9 @@ constexpr uint32_t kSpinLimit = 1u << 22;
 #ifndef HAWK_BWD_WAVES_PER_SIMD
 #define HAWK_BWD_WAVES_PER_SIMD 4
 #endif
+#ifndef HAWK_BWD_KEEP_ALPHA
+#define HAWK_BWD_KEEP_ALPHA 1
+#endif
 
 // Control block at the start of the workspace:
 //   bytes 0-7   one 64-bit word: launch epoch (high half) and ticket counter (low half)
@@ -330,7 +333,8 @@ __device__ __forceinline__ void fwd_tile(const IT* __restrict__ x, const IT* __r
             if (!PACK_P) pj[j][v] = p_run[v];
             hj[j][v] = h_run[v];
         }
-        if (PACK_P) pjh[j] = pack_f16x2(p_run[0], p_run[V - 1]);
+        // (packed now: left alone, the conversion sinks below the exchange and the products stay in fp32)
+        if (PACK_P) pjh[j] = opaque(pack_f16x2(p_run[0], p_run[V - 1]));
         __builtin_amdgcn_sched_barrier(0);  // one row's temporaries live at a time
     }
 
@@ -352,7 +356,11 @@ __device__ __forceinline__ void fwd_tile(const IT* __restrict__ x, const IT* __r
     for (int v = 0; v < V; ++v) s_agg[w][lane * V + v] = make_float2(p_run[v], h_run[v]);
     __syncthreads();
     float pre_p[V], pre_h[V], tot_p[V], tot_h[V];
-    combine_slices<V, NW, false, GATED>(s_agg, w, lane, pre_p, pre_h, tot_p, tot_h);
+    combine_slices<V, NW, false, true>(s_agg, w, lane, pre_p, pre_h, tot_p, tot_h);
+    // This wave's prefix is picked here: left to itself the compiler keeps all NW candidates in
+    // registers through the carry exchange and picks afterwards (30 registers at 16 rows).
+#pragma unroll
+    for (int v = 0; v < V; ++v) { pre_p[v] = opaque(pre_p[v]); pre_h[v] = opaque(pre_h[v]); }
 
     // 3. carry across tiles
     float cin[V];
@@ -529,6 +537,9 @@ __device__ __forceinline__ void bwd_tile(const IT* __restrict__ x, const IT* __r
     constexpr bool PACK_R = (V == 2) && (sizeof(IT) == 2);
     float rr[PACK_R ? 1 : TC][V];
     uint32_t rrh[PACK_R ? TC : 1];
+    // alpha is kept for the replay where the registers are there for it (short tiles)
+    constexpr bool KEEP_ALPHA = HAWK_BWD_KEEP_ALPHA && TC <= 8;
+    float al[KEEP_ALPHA ? TC : 1][V];
     float q_run[V], c_run[V];
 #pragma unroll
     for (int v = 0; v < V; ++v) { q_run[v] = 1.0f; c_run[v] = 0.0f; }
@@ -573,6 +584,7 @@ __device__ __forceinline__ void bwd_tile(const IT* __restrict__ x, const IT* __r
             float alpha = hw_exp2(c2[v] * rv[v]);
             if (!ok) alpha = 1.0f;  // rows past T are the identity
             if (!PACK_R) rr[j][v] = rv[v];
+            if (KEEP_ALPHA) al[j][v] = alpha;
             c_run[v] = alpha * (fgo[v] + c_run[v]);
             q_run[v] *= alpha;
         }
@@ -594,7 +606,9 @@ __device__ __forceinline__ void bwd_tile(const IT* __restrict__ x, const IT* __r
     for (int v = 0; v < V; ++v) s_agg[w][lane * V + v] = make_float2(q_run[v], c_run[v]);
     __syncthreads();
     float pre_p[V], pre_h[V], tot_p[V], tot_h[V];
-    combine_slices<V, NW, true>(s_agg, w, lane, pre_p, pre_h, tot_p, tot_h);
+    combine_slices<V, NW, true, true>(s_agg, w, lane, pre_p, pre_h, tot_p, tot_h);
+#pragma unroll
+    for (int v = 0; v < V; ++v) { pre_p[v] = opaque(pre_p[v]); pre_h[v] = opaque(pre_h[v]); }  // as in the forward
 
     // 3. carry across tiles
     float cin[V];
@@ -644,8 +658,13 @@ __device__ __forceinline__ void bwd_tile(const IT* __restrict__ x, const IT* __r
 #pragma unroll
         for (int v = 0; v < V; ++v) {
             const float r = PACK_R ? (v == 0 ? f16_lo(rpair) : f16_hi(rpair)) : opaque(rr[j][v]);
-            float alpha = hw_exp2(c2[v] * r);  // cheaper to re-evaluate than to keep in a register
-            if (!ok) alpha = 1.0f;
+            float alpha;
+            if (KEEP_ALPHA) {
+                alpha = opaque(al[j][v]);
+            } else {
+                alpha = hw_exp2(c2[v] * r);  // cheaper to re-evaluate than to keep in a register
+                if (!ok) alpha = 1.0f;
+            }
             const float g = fgo[v] + c_true[v];
             c_true[v] = alpha * g;
             const float i = sigmoid_fast(fxg[v]);
@@ -754,7 +773,10 @@ struct TileShape {
 // Tile shapes.  A lane moves 4 bytes per row access: two bf16 channels (one when D is
 // odd) or one fp32 channel, so a wave covers 256 contiguous bytes of a row.  The forward
 // keeps 2 floats per element across the carry exchange, the backward keeps the packed
-// inputs and one float, which sets how many rows fit in 128 VGPRs (4 waves per SIMD).
+// inputs and one float.  Two workgroups of 8 waves share a CU (4 waves per SIMD, 128 VGPRs each);
+// the heights below are the fastest measured, not the tallest that fit: the forward kernels use
+// 86 (102 gated) registers at 16 rows, and 20 to 28 rows, or three workgroups of 10 to 14 rows, are
+// 1-10 % slower.
 #ifndef HAWK_FWD_TC
 #define HAWK_FWD_TC 16
 #endif
@@ -768,7 +790,7 @@ struct TileShape {
 #define HAWK_BWD_NW 8
 #endif
 #ifndef HAWK_FWD_GATED_TC
-#define HAWK_FWD_GATED_TC 12
+#define HAWK_FWD_GATED_TC 16
 #endif
 #ifndef HAWK_BWD_GATED_TC
 #define HAWK_BWD_GATED_TC 10
