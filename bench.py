@@ -932,6 +932,7 @@ def run_stream_ceiling(buf, steps, settle):
     lib = _lib.load()
     stream = torch.cuda.current_stream(x.device).cuda_stream
     row_pitch = x.shape[-1] * x.element_size()
+    seq_groups = x.shape[1] // 128   # 128-row tiles per sequence: the probe then walks tiles in the scan's launch order
 
     def probe(reads, writes, shape):
         r = (ctypes.c_void_p * len(reads))(*[t.data_ptr() for t in reads])
@@ -949,7 +950,9 @@ def run_stream_ceiling(buf, steps, settle):
                                        ("probe_flat_3r1w", probe(*fwd_mix, 0), 4, 1),
                                        ("probe_flat_5r3w", probe(*bwd_mix, 0), 8, 1),
                                        ("probe_scan_shape_3r1w", probe(*fwd_mix, 1), 4, 1),
-                                       ("probe_scan_shape_5r3w", probe(*bwd_mix, 1), 8, 1)):
+                                       ("probe_scan_shape_5r3w", probe(*bwd_mix, 1), 8, 1),
+                                       ("probe_scan_order_3r1w", probe(*fwd_mix, seq_groups), 4, 1),
+                                       ("probe_scan_order_5r3w", probe(*bwd_mix, seq_groups), 8, 1)):
         for _ in range(settle):
             fn()
         torch.cuda.synchronize()
@@ -978,7 +981,9 @@ def run_stream_ceiling(buf, steps, settle):
                    "a_rg_lru, h, grad_out and gradient tensors (bf16, %d MB each), and the library's copy kernels "
                    "(hawk_stream_probe: non-temporal buffer loads and stores; flat = 16 KiB of every tensor per "
                    "workgroup, scan_shape = eight waves stacked in time on 16 rows x 256 bytes each, as a scan "
-                   "workgroup reads its tile) on the same tensors; %d settling calls, then %d timed calls; frac is "
+                   "workgroup reads its tile, tiles in memory order; scan_order = the same tiles in the order the "
+                   "scan's launch takes them: position along the sequence slowest, then batch row, then channel "
+                   "tile) on the same tensors; %d settling calls, then %d timed calls; frac is "
                    "of the 8 TB/s peak" % (nbytes // 1000000, settle, steps))
     return rec
 
@@ -1059,6 +1064,14 @@ def main():
             ceiling["probe_scan_shape_5r3w"]["us_with_an_event_per_call"] * 1e-3 / out["roofline"]["launch_ms"])
         ceiling["scan_step_over_probe_scan_shape"] = (
             (ceiling["probe_scan_shape_3r1w"]["us"] + ceiling["probe_scan_shape_5r3w"]["us"]) * 1e-3
+            / out["ms_per_step"])
+        # ... and against the same copies with the tiles taken in the scan's launch order
+        ceiling["scan_fwd_over_probe_scan_order_3r1w"] = (
+            ceiling["probe_scan_order_3r1w"]["us_with_an_event_per_call"] * 1e-3 / out["fwd"]["ms"])
+        ceiling["scan_bwd_over_probe_scan_order_5r3w"] = (
+            ceiling["probe_scan_order_5r3w"]["us_with_an_event_per_call"] * 1e-3 / out["roofline"]["launch_ms"])
+        ceiling["scan_step_over_probe_scan_order"] = (
+            (ceiling["probe_scan_order_3r1w"]["us"] + ceiling["probe_scan_order_5r3w"]["us"]) * 1e-3
             / out["ms_per_step"])
         ceiling["scan_step_over_probe_flat"] = (
             (ceiling["probe_flat_3r1w"]["us"] + ceiling["probe_flat_5r3w"]["us"]) * 1e-3 / out["ms_per_step"])

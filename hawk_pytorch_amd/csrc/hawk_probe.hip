@@ -2,7 +2,8 @@
 // kernels' own memory instructions (non-temporal buffer loads and stores through a resource in
 // scalar registers) and no arithmetic to speak of, in two shapes: flat (a 256-thread workgroup
 // takes 16 KiB of every tensor, 16 bytes a lane) and in the scan's workgroup shape (eight waves
-// stacked in time, each on 16 rows x 256 bytes with 4 bytes a lane, column tiles fastest).  They
+// stacked in time, each on 16 rows x 256 bytes with 4 bytes a lane; the tiles are taken in memory
+// order or in the order a scan launch takes them, position along the sequence slowest).  They
 // exist so that a benchmark can state, on its own tensors and in its own process, what the part
 // delivers for the scan's mix of reads and writes with and without the scan's access shape.
 // Every output element receives the sum of the inputs' 32-bit words at its place plus the
@@ -43,8 +44,13 @@ constexpr int kTileWaves = 8, kTileRowsPerWave = 16, kTileRowBytes = 256;
 
 template <int NR, int NW>
 __global__ __launch_bounds__(kTileWaves* kWave) void stream_probe_tile_kernel(ProbeTensors t, uint32_t row_pitch,
-                                                                             int column_tiles) {
-    const int tile = (int)blockIdx.x, ct = tile % column_tiles, rg = tile / column_tiles;
+                                                                             int column_tiles, int groups_per_seq,
+                                                                             int sequences) {
+    // the scan's launch order: position along the sequence slowest, then sequence, then column tile
+    const int tile = (int)blockIdx.x, per_pos = sequences * column_tiles;
+    const int seg = tile / per_pos, rem = tile - seg * per_pos;
+    const int seq = rem / column_tiles, ct = rem - seq * column_tiles;
+    const int rg = seq * groups_per_seq + seg;
     const int w = __builtin_amdgcn_readfirstlane((int)threadIdx.x / kWave);
     const size_t origin = ((size_t)rg * kTileWaves + w) * kTileRowsPerWave * row_pitch + (size_t)ct * kTileRowBytes;
     const uint32_t window = (kTileRowsPerWave - 1) * row_pitch + kTileRowBytes;
@@ -73,7 +79,8 @@ int launch_probe(const ProbeTensors& t, size_t bytes, uint32_t row_pitch, int sh
         const int column_tiles = (int)(row_pitch / kTileRowBytes);
         const size_t row_groups = bytes / row_pitch / (kTileWaves * kTileRowsPerWave);
         hipLaunchKernelGGL((stream_probe_tile_kernel<NR, NW>), dim3((unsigned)(row_groups * column_tiles)),
-                           dim3(kTileWaves * kWave), 0, st, t, row_pitch, column_tiles);
+                           dim3(kTileWaves * kWave), 0, st, t, row_pitch, column_tiles, shape,
+                           (int)(row_groups / (size_t)shape));
     }
     return hipGetLastError() == hipSuccess ? HAWK_OK : HAWK_ERR_LAUNCH;
 }
@@ -83,8 +90,10 @@ int launch_probe(const ProbeTensors& t, size_t bytes, uint32_t row_pitch, int sh
 bool stream_probe_shape_ok(size_t bytes, size_t row_pitch, int shape) {
     if (bytes == 0 || bytes / kFlatBytes > 0x7fffffffull) return false;
     if (shape == 0) return bytes % kFlatBytes == 0;
-    if (shape != 1 || row_pitch == 0 || row_pitch % kTileRowBytes != 0 || row_pitch > (1u << 24)) return false;
-    return bytes % row_pitch == 0 && (bytes / row_pitch) % (kTileWaves * kTileRowsPerWave) == 0;
+    if (shape < 1 || row_pitch == 0 || row_pitch % kTileRowBytes != 0 || row_pitch > (1u << 24)) return false;
+    if (bytes % row_pitch != 0 || (bytes / row_pitch) % (kTileWaves * kTileRowsPerWave) != 0) return false;
+    const size_t row_groups = bytes / row_pitch / (kTileWaves * kTileRowsPerWave);
+    return row_groups % (size_t)shape == 0 && row_groups * (row_pitch / kTileRowBytes) <= 0x7fffffffull;
 }
 
 int stream_probe(const void* const* reads, int n_reads, void* const* writes, int n_writes, size_t bytes,

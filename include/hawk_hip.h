@@ -405,11 +405,14 @@ int hawk_block_core_bwd(const void* xy, long long xy_row_stride, const void* u, 
  * tensors in and n_writes tensors out (`bytes` each, 16-byte aligned, all distinct) with the scan
  * kernels' memory instructions and no arithmetic to speak of, so that a benchmark can state on its
  * own tensors what the part delivers for a mix of reads and writes.  shape 0: flat, a workgroup
- * takes 16 KiB of every tensor (bytes a multiple of 16384).  shape 1: the scan's workgroup shape,
- * eight waves stacked in time on 16 rows x 256 bytes each, over [rows, row_pitch_bytes] tensors
- * (row_pitch_bytes a multiple of 256, rows a multiple of 128).  Every 32-bit word of output i
- * receives the sum of the inputs' words at its place plus i.  Supported mixes (reads + writes):
- * 1+1, 1+2, 1+3, 2+1, 3+1, 5+3; HAWK_ERR_BAD_SHAPE otherwise.
+ * takes 16 KiB of every tensor (bytes a multiple of 16384).  shape S >= 1: the scan's workgroup
+ * shape, eight waves stacked in time on 16 rows x 256 bytes each, over [rows, row_pitch_bytes]
+ * tensors (row_pitch_bytes a multiple of 256, rows a multiple of 128 * S), with the tiles taken in
+ * the order a scan launch over sequences of S row groups (128 * S rows) takes them: position along
+ * the sequence slowest, then sequence, then column tile; S = 1 is plain memory order, S = T / 128
+ * the order of a [B, T, D] scan.  Every 32-bit word of output i receives the sum of the inputs'
+ * words at its place plus i.  Supported mixes (reads + writes): 1+1, 1+2, 1+3, 2+1, 3+1, 5+3;
+ * HAWK_ERR_BAD_SHAPE otherwise.
  * ------------------------------------------------------------------------------------- */
 int hawk_stream_probe(const void* const* reads, int n_reads, void* const* writes, int n_writes,
                       size_t bytes, size_t row_pitch_bytes, int shape, void* stream);

@@ -56,20 +56,22 @@ def test_bench_prints_one_json_line_with_the_agreed_fields():
 
 def test_stream_probe_moves_all_of_every_tensor():
     """hawk_stream_probe: every 32-bit word of output i is the sum of the inputs' words at its place
-    plus i, in both shapes and for every supported mix; other mixes and shapes are refused."""
+    plus i, flat, tiled in memory order and tiled in the scan's launch order (sequences of 2 row
+    groups: position along the sequence slowest), for every supported mix; other mixes and shapes are
+    refused."""
     import ctypes
 
     import torch
     from hawk_pytorch_amd import _lib
 
     lib = _lib.load()
-    rows, pitch = 256, 1280          # bytes per row: five column tiles of 256 bytes
+    rows, pitch = 512, 1280          # four row groups of 128 rows; bytes per row: five column tiles of 256 bytes
     n = rows * pitch // 4
     gen = torch.Generator(device="cuda").manual_seed(4)
     ins = [torch.randint(0, 1 << 20, (n,), dtype=torch.int32, device="cuda", generator=gen) for _ in range(5)]
     st = torch.cuda.current_stream().cuda_stream
     for nr, nw in ((1, 1), (1, 2), (1, 3), (2, 1), (3, 1), (5, 3)):
-        for shape in (0, 1):
+        for shape in (0, 1, 2):
             if shape == 0 and (n * 4) % 16384:
                 continue
             outs = [torch.full((n,), -1, dtype=torch.int32, device="cuda") for _ in range(nw)]
@@ -85,3 +87,5 @@ def test_stream_probe_moves_all_of_every_tensor():
     assert lib.hawk_stream_probe(r, 2, w, 2, n * 4, pitch, 0, st) == _lib.HAWK_ERR_BAD_SHAPE      # no 2 + 2
     assert lib.hawk_stream_probe(r, 2, w, 1, n * 4, pitch + 4, 1, st) == _lib.HAWK_ERR_BAD_SHAPE  # pitch % 256
     assert lib.hawk_stream_probe(r, 2, w, 1, n * 4 - 16384, pitch, 1, st) == _lib.HAWK_ERR_BAD_SHAPE
+    assert lib.hawk_stream_probe(r, 2, w, 1, n * 4, pitch, 3, st) == _lib.HAWK_ERR_BAD_SHAPE      # 4 groups % 3
+    assert lib.hawk_stream_probe(r, 2, w, 1, n * 4, pitch, -1, st) == _lib.HAWK_ERR_BAD_SHAPE
