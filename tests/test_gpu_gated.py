@@ -78,6 +78,13 @@ def test_time_lengths_around_tile_edges(T, dtypes):
 
 
 @pytest.mark.parametrize("dtypes", [("f32", "f32"), ("bf16", "bf16")])
+@pytest.mark.parametrize("T", [1, 63, 65, 100, 129, 200])
+def test_time_lengths_around_tile_edges_with_many_chains(T, dtypes):
+    """The 64-row backward tiles that launches with 128 or more chains take (8 x 2048 channels)."""
+    _run(8, T, 2048, *dtypes, seed=400 + T)
+
+
+@pytest.mark.parametrize("dtypes", [("f32", "f32"), ("bf16", "bf16")])
 @pytest.mark.parametrize("D", [1, 2, 3, 64, 66, 130, 320, 1000])
 def test_channel_counts_including_ragged_tiles(D, dtypes):
     _run(2, 131, D, *dtypes, layout="dense" if D < 8 else "half", seed=D)

@@ -63,6 +63,15 @@ def test_time_lengths_around_tile_edges(T, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["f32", "bf16"])
+@pytest.mark.parametrize("T", [1, 5, 63, 64, 65, 100, 129, 200])
+def test_time_lengths_around_tile_edges_with_many_chains(T, dtype):
+    """128 or more independent chains (batch rows x channel tiles) switch the backward to 64-row
+    tiles, which keep alpha from the local pass for the replay; rows past T must stay the
+    identity there too.  8 x 2048 channels: 128 chains in bf16, 256 in fp32."""
+    _run_case(8, T, 2048, dtype, seed=300 + T)
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
 @pytest.mark.parametrize("D", [1, 2, 3, 64, 66, 128, 130, 192, 320, 1000])
 def test_channel_counts_including_ragged_tiles(D, dtype):
     """The C ABI takes any D; odd D runs one channel per lane, and D that does not fill the
