@@ -95,8 +95,8 @@ __device__ __forceinline__ bool try_read(const unsigned long long* p, uint32_t t
 // Every lookback-th chain position is a checkpoint: it publishes the inclusive state at
 // its end; every other position publishes only its own aggregate.  A tile reads the
 // aggregates of its predecessors back to the nearest checkpoint, plus that checkpoint's
-// inclusive state, all in parallel (one predecessor per wave), and folds them oldest
-// first.  The order of the floating-point operations is fixed by the position and the
+// inclusive state, all in parallel (wave k fetches predecessors k, k + NW, ...), and folds them
+// oldest first.  The order of the floating-point operations is fixed by the position and the
 // launch's shape alone, never by timing, so results are bitwise reproducible, and the serial
 // dependency runs over checkpoints only (nseg / lookback hops of one memory round trip each).
 // The distance is chosen per launch: 4 when there are enough independent chains (B x channel
@@ -106,8 +106,13 @@ __device__ __forceinline__ bool try_read(const unsigned long long* p, uint32_t t
 // With 128 or more chains the distance is 2: a tile then reads at most two predecessors'
 // words, and even at one memory round trip per two positions the chain stays ahead of the
 // rate at which the launch gets through a position of all its chains (0.5 % faster).
-constexpr int kMaxLookback = 8;
+// With 8 chains or fewer the hops are all there is to wait for, and the distance grows to 16
+// (5 to 8 chains: 6 % / 3 % faster forward / backward than 8; 12 or more chains are 2 % slower
+// with it) and to 32 (up to 4 chains: one chain, B = 1 and D = 128, runs twice as fast as with 8,
+// 4 chains 28 % / 20 % faster).
+constexpr int kMaxLookback = 32;
 constexpr int kFewChains = 24;
+constexpr int kFewerChains = 8, kFewestChains = 4;   // distance 16 and 32
 #ifndef HAWK_LOOKBACK_MANY
 #define HAWK_LOOKBACK_MANY 2
 #endif
@@ -140,8 +145,8 @@ __device__ __forceinline__ void take_ticket(unsigned long long* ctrl, uint32_t t
 // Carry into chain position `pos` for the V channels of this lane.
 //   tot_p/tot_h  aggregate of this whole tile (every wave holds it)
 //   s_prev       LDS [kMaxLookback][CT] staging of the predecessors' words
-// Wave 0 publishes the tile's own word; wave k (k < number of predecessors) fetches
-// predecessor pos-1-k; after one barrier every wave folds the staged words.
+// Wave 0 publishes the tile's own word; wave k fetches predecessors pos-1-k, pos-1-k-NW, ...;
+// after one barrier every wave folds the staged words.
 template <int V, int NW>
 __device__ __forceinline__ void exchange_carry(const ScanWsPtrs& ws, int pos, int nseg, size_t idx_pos0,
                                                size_t stride, uint32_t tag, int w, int lane,
@@ -159,8 +164,7 @@ __device__ __forceinline__ void exchange_carry(const ScanWsPtrs& ws, int pos, in
         asm volatile("" ::: "memory");
     }
     const int npred = (pos > 0) ? pos - checkpoint_before(pos, lookback) : 0;
-    static_assert(NW >= kMaxLookback, "one wave per predecessor");
-    if (const int k = w; k < npred) {
+    for (int k = w; k < npred; k += NW) {
         const int j = pos - 1 - k;
         const size_t idx = idx_pos0 + (size_t)j * stride;
         const bool cp = (k == npred - 1);
@@ -852,7 +856,9 @@ int lookback_for(int B, int nct) {
     return HAWK_LOOKBACK;
 #else
     const long long chains = (long long)B * nct;
-    return chains <= kFewChains ? kMaxLookback : (chains >= kManyChains ? HAWK_LOOKBACK_MANY : 4);
+    if (chains <= kFewestChains) return 32;
+    if (chains <= kFewerChains) return 16;
+    return chains <= kFewChains ? 8 : (chains >= kManyChains ? HAWK_LOOKBACK_MANY : 4);
 #endif
 }
 FastDiv fast_div_for(uint32_t d) {

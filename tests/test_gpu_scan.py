@@ -71,6 +71,15 @@ def test_time_lengths_around_tile_edges_with_many_chains(T, dtype):
     _run_case(8, T, 2048, dtype, seed=300 + T)
 
 
+@pytest.mark.parametrize("B,T,D", [(1, 9000, 128), (1, 6100, 512), (2, 5000, 512), (3, 4500, 256)])
+def test_long_sequences_on_very_few_chains(B, T, D):
+    """Up to 8 independent chains (batch rows x channel tiles) space the checkpoints of the carry
+    chain 16 positions apart, up to 4 chains 32 apart (a wave then fetches several predecessors):
+    1, 4, 8 and 6 chains here in bf16, over 36 to 71 forward positions."""
+    _run_case(B, T, D, "bf16", seed=500 + D, lo=0.99, hi=0.9999)
+    _run_case(B, T, D, "f32", seed=501 + D)
+
+
 @pytest.mark.parametrize("dtype", ["f32", "bf16"])
 @pytest.mark.parametrize("D", [1, 2, 3, 64, 66, 128, 130, 192, 320, 1000])
 def test_channel_counts_including_ragged_tiles(D, dtype):
